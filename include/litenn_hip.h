@@ -1,0 +1,157 @@
+/* C ABI of liblitenn_hip.so: the MI355X (gfx950) device layer behind LiteNN's
+ * operator API for nn.conv2D / nn.matmul and their backward passes.
+ *
+ * It takes the place of the 26 OpenCL entry points LiteNN binds through
+ * ctypes (litenn/core/minicl/api/OpenCL/OpenCL.py:214-668) plus the kernels
+ * LiteNN generates as OpenCL C text at run time.  Conventions:
+ *   - every function returns an int status: 0 on success, negative on error;
+ *     lnn_last_error() gives the message of the calling thread's last failure
+ *     (the role of CLException/ERROR codes, OpenCL.py:175-198);
+ *   - LNN_ERR_OOM is distinct so a caller-side buffer pool can evict and retry
+ *     (CLDevice.py:134-164 does this on MEM_OBJECT_ALLOCATION_FAILURE);
+ *   - pointers are raw device addresses owned by the caller; the library keeps
+ *     no per-tensor state.  It owns, per device, one stream (all launches are
+ *     asynchronous and in order, like the in-order command queue of
+ *     CLDevice.py:186-190), a grow-only scratch buffer for split-K partial
+ *     sums, and small cached gather tables keyed by convolution geometry;
+ *   - all tensors are dense fp32; every tensor must be smaller than 2 GiB;
+ *   - single-threaded callers per device; no callbacks.
+ *   - `beta` is 0 (overwrite) or 1 (accumulate: out += result), the two forms
+ *     LiteNN selects with is_add_to_output (matmul.py:162, unfold2D.py:110).
+ */
+#ifndef LITENN_HIP_H
+#define LITENN_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LNN_OK 0
+#define LNN_ERR_INVALID (-1)     /* bad argument (shape, alignment, null pointer) */
+#define LNN_ERR_OOM (-2)         /* device allocation failed */
+#define LNN_ERR_NO_DEVICE (-3)   /* no usable HIP device / bad device index */
+#define LNN_ERR_HIP (-4)         /* any other HIP runtime failure */
+#define LNN_ERR_UNSUPPORTED (-5) /* valid request outside the library's limits */
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* lnn_last_error(void);
+
+/* ---- devices: replaces clGetPlatformIDs/clGetDeviceIDs/clGetDeviceInfo
+ *      (OpenCL.py:214-310) as used by devices.get_all (devices.py:88-105). */
+int lnn_device_count(int* count);
+int lnn_device_info(int dev, char* name, int name_cap, uint64_t* total_mem_bytes,
+                    int* compute_units, int* clock_khz);
+/* Frees the stream, scratch and cached tables of a device: the counterpart of
+ * dropping the context/queue in CLDevice._cleanup (CLDevice.py:107-118). */
+int lnn_release_device(int dev);
+
+/* ---- memory: replaces clCreateBuffer / clReleaseMemObject and the
+ *      clEnqueue{Write,Read,Copy,Fill}Buffer calls (OpenCL.py:376-456) behind
+ *      CLDevice._mem_alloc (CLDevice.py:120-165) and CLBuffer.set/fill/np
+ *      (CLBuffer.py:50-115). */
+int lnn_malloc(int dev, uint64_t bytes, void** out);
+int lnn_free(int dev, void* ptr);
+int lnn_mem_info(int dev, uint64_t* free_bytes, uint64_t* total_bytes);
+/* host -> device; returns after the host buffer may be reused (CLBuffer.py:78-80) */
+int lnn_memcpy_h2d(int dev, void* dst, const void* src, uint64_t bytes);
+/* device -> host; returns after the data has arrived (CLBuffer.py:112-113) */
+int lnn_memcpy_d2h(int dev, void* dst, const void* src, uint64_t bytes);
+/* device -> device on the device's stream, asynchronous (CLBuffer.py:66-67) */
+int lnn_memcpy_d2d(int dev, void* dst, const void* src, uint64_t bytes);
+/* fills `count` 32-bit words with `pattern` (CLBuffer.fill, CLBuffer.py:83-96) */
+int lnn_fill_u32(int dev, void* dst, uint32_t pattern, uint64_t count);
+/* waits for all work queued on the device: clFinish (CLDevice.py:51-55) */
+int lnn_synchronize(int dev);
+
+/* ---- timing on the device's stream (no counterpart in the reference, whose
+ *      queue is created without profiling, OpenCL.py:349-351). */
+int lnn_event_create(int dev, void** event);
+int lnn_event_record(int dev, void* event);
+int lnn_event_elapsed_ms(int dev, void* start, void* stop, float* ms); /* waits for `stop` */
+int lnn_event_destroy(int dev, void* event);
+
+/* ---- GEMM: replaces the generated "GeMM" kernel (matmul.py:127-164) and the
+ *      transposes its gradients materialise (matmul.py:64-72).
+ *   C[b] (+)= op(A[b]) * op(B[b]),  op(A) is M x K, op(B) is K x N, C is M x N,
+ *   all row-major with leading dimensions lda/ldb/ldc (elements) and batch
+ *   strides (elements).  trans_a: A is stored K x M.  trans_b: B is stored
+ *   N x K.  nn.matmul forward is (0,0); dA = dC * B^T is (0,1); dB = A^T * dC
+ *   is (1,0). */
+int lnn_gemm_f32(int dev, int trans_a, int trans_b, int batch, int M, int N, int K,
+                 const float* A, int lda, int64_t stride_a,
+                 const float* B, int ldb, int64_t stride_b,
+                 float* C, int ldc, int64_t stride_c, int beta);
+
+/* ---- convolution: replaces unfold2D + GeMM + transpose of conv2D.py:39-54.
+ * Geometry as computed by InfoConv2D (InfoConv2D.py:41-77); only the left/top
+ * pads enter the kernels (unfold2D.py:85-137).  X is [N,C,IH,IW], W is
+ * [O,C,KH,KW], Y is [N,O,OH,OW], all NCHW row-major. */
+typedef struct lnn_conv2d_desc {
+  int32_t N, C, IH, IW;
+  int32_t O, KH, KW;
+  int32_t OH, OW;
+  int32_t PADL, PADT;
+  int32_t stride, dilation;
+} lnn_conv2d_desc;
+
+/* Y (+)= conv(X, W)                      conv2D.py:39-42 */
+int lnn_conv2d_fwd_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* W,
+                       float* Y, int beta);
+/* dX (+)= dgrad(dY, W)                   conv2D.py:46-50 (the reference always accumulates) */
+int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* W,
+                         float* dX, int beta);
+/* dW (+)= wgrad(X, dY)                   conv2D.py:52-54 (the reference always accumulates) */
+int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
+                         float* dW, int beta);
+
+/* ---- nc.op.unfold2D (unfold2D.py:6-48): materialised im2col / im2row /
+ * transposed im2row.  Shares its index arithmetic with the gather loaders of
+ * the convolution kernels and exists so that arithmetic can be checked bit for
+ * bit.  order 0 = 'CJI_NHW', 1 = 'NHW_CJI'.  Arguments as in the reference
+ * call: (H, W) source size, (OH, OW) extent of the H/W output symbols. */
+int lnn_unfold2d_f32(int dev, int N, int C, int H, int W, int OH, int OW, int KH, int KW,
+                     int PADL, int PADT, int dilation, int stride, int order, int is_transpose,
+                     const float* in, float* out, int beta);
+
+/* ---- nc.op.transpose (transpose.py:60-103): out[perm(idx)] (+)= in[idx],
+ * rank <= 8, out shape = shape[axes]. */
+int lnn_transpose_f32(int dev, int rank, const int32_t* shape, const int32_t* axes,
+                      const float* in, float* out, int beta);
+
+/* ---- pointwise / reduction helpers the training step of a conv net needs
+ * around the hot path (element_wise_op.py:83-110, dual_wise_op.py:132-191,
+ * reduce.py:166-301, SGD.py:42-74). */
+enum {
+  LNN_EW_ADD_CONST = 0,  /* out = in + p0                      element_wise_op.py:122-130 */
+  LNN_EW_MUL_CONST = 1,  /* out = in * p0 */
+  LNN_EW_LEAKY_RELU = 2, /* out = in >= 0 ? in : p0*in         element_wise_op.py:208-222 */
+  LNN_EW_SQUARE = 3,     /* out = in*in                        element_wise_op.py:331-344 */
+  LNN_EW_RELU = 4
+};
+/* out (+)= f(in) */
+int lnn_ew_fwd_f32(int dev, int op, uint64_t n, const float* in, float* out, float p0, int beta);
+/* din += f'(in, out_fwd) * dout     (always accumulates, element_wise_op.py:108) */
+int lnn_ew_bwd_f32(int dev, int op, uint64_t n, const float* in, const float* dout, float* din,
+                   float p0);
+/* out (+)= a (op) b with numpy broadcasting; shapes already left-padded with
+ * ones to `rank` <= 8 (dual_wise_op.py:138-152).  op: 0 add, 1 sub, 2 mul. */
+int lnn_binary_bcast_f32(int dev, int op, int rank, const int32_t* out_shape,
+                         const int32_t* a_shape, const int32_t* b_shape, const float* a,
+                         const float* b, float* out, int beta);
+/* out[kept axes] (+)= scale * sum over reduced axes of in; reduce_mask bit i
+ * set = axis i is summed.  rank <= 8. */
+int lnn_reduce_sum_f32(int dev, int rank, const int32_t* shape, uint32_t reduce_mask,
+                       float scale, const float* in, float* out, int beta);
+/* din[idx] += scale * dout[idx with reduced axes set to 0]   (reduce.py:243-255) */
+int lnn_reduce_sum_bwd_f32(int dev, int rank, const int32_t* shape, uint32_t reduce_mask,
+                           float scale, const float* dout, float* din);
+/* SGD.py:42-74: acc = momentum*acc - lr*g;  v += nesterov ? momentum*acc - lr*g : acc */
+int lnn_sgd_update_f32(int dev, uint64_t n, float* v, const float* g, float* acc, float momentum,
+                       float lr, int nesterov);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LITENN_HIP_H */

@@ -1,0 +1,48 @@
+// Shared host-side declarations of the HIP library (not part of the C ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <array>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/litenn_hip.h"
+#include "tile_engine.hpp"
+
+namespace lnn {
+
+struct DeviceCtx {
+  int index = -1;
+  bool ready = false;
+  hipStream_t stream = nullptr;
+  int cus = 0;
+  // grow-only scratch owned by the library (split-K partial sums)
+  void* ws = nullptr;
+  size_t ws_bytes = 0;
+  // gather tables, one per (geometry, kind)
+  std::map<std::array<int, 12>, KEntry*> tables;
+};
+
+int set_error(int code, const std::string& msg);
+int hip_fail(hipError_t e, const char* what);
+DeviceCtx* get_ctx(int dev, int* status);          // makes dev current, creates the stream
+int ensure_workspace(DeviceCtx* ctx, size_t bytes);
+
+#define LNN_HIP(call)                                   \
+  do {                                                  \
+    hipError_t e_ = (call);                             \
+    if (e_ != hipSuccess) return hip_fail(e_, #call);   \
+  } while (0)
+
+constexpr uint64_t kMaxTensorBytes = 0x7fffffffull;   // raw buffer descriptors address < 2 GiB
+
+// launchers implemented in the kernel translation units
+int launch_gemm(DeviceCtx* ctx, int ta, int tb, int batch, int M, int N, int K, const float* A, int lda,
+                long long sA, const float* B, int ldb, long long sB, float* C, int ldc, long long sC, int beta);
+int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta);
+int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta);
+int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta);
+
+}  // namespace lnn

@@ -1,0 +1,296 @@
+// Implicit-GEMM convolution passes on the MFMA tile engine.  Nothing is
+// unfolded to memory: the loaders compute im2col addresses on the fly and the
+// epilogue writes NCHW directly.
+//
+//   forward  Y [O  x P ] = W[O x CKK]        . im2col(X)[CKK x P]     P = N*OH*OW
+//   dgrad    dX[C  x Q ] = Wt[C x O*KK]      . im2rowT(dY)[O*KK x Q]  Q = N*IH*IW
+//   wgrad    dW[O  x CKK] = dY[O x P]        . im2row(X)[P x CKK]     (split over P)
+#include "common.hpp"
+
+namespace lnn {
+
+struct ConvArgs {
+  ConvGeom g;
+  const float* X;    // fwd: X, dgrad: dY, wgrad: X
+  const float* W;    // fwd: W, dgrad: W,  wgrad: dY
+  float* Out;        // fwd: Y, dgrad: dX, wgrad: dW or the partial-sum buffer
+  const KEntry* tab;
+  uint32_t bytesX, bytesW, bytesOut;
+  int M, Ncols, K;   // GEMM extents
+  int beta;
+  int n_units, total_units;
+  int ksplit;        // wgrad: number of K slices (gridDim.y)
+};
+
+// mode 0: k = (c, kh, kw) for forward / wgrad; mode 1: k = (o, kh, kw) for dgrad.
+__global__ void build_ktable(KEntry* tab, int K, int Kpad, int mode, ConvGeom g) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= Kpad) return;
+  KEntry e;
+  if (k < K) {
+    const int ch = k / g.KK, tap = k - ch * g.KK, kh = tap / g.KW, kw = tap - kh * g.KW;
+    e.y = kh * g.D;
+    e.z = kw * g.D;
+    if (mode == 0) {
+      e.x = ch * g.IHW + kh * g.D * g.IW + kw * g.D;
+      e.w = 0;
+    } else {
+      e.x = ch * g.OHW;
+      e.w = ch * g.C * g.KK + tap;
+    }
+  } else {
+    e.x = 0;
+    e.y = BIG;
+    e.z = 0;
+    e.w = 0x20000000;
+  }
+  tab[k] = e;
+}
+
+__global__ void reduce_partials(float* out, const float* part, int n, int slices, int beta) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float s = beta ? out[i] : 0.0f;
+  for (int k = 0; k < slices; ++k) s += part[(size_t)k * n + i];
+  out[i] = s;
+}
+
+enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2 };
+
+template <int PASS, int WM, int NTMAX, bool FLAG>
+struct ConvCfg {
+  static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * NTMAX;
+  // A side is K-contiguous in LDS for all three passes.
+  static constexpr int SA = LdsSize<true, BM>::value;
+  // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
+  static constexpr int SB = LdsSize<PASS == PASS_WGRAD, BNMAX>::value;
+};
+
+template <int PASS, class Cfg, int WM, int NT, bool FLAG>
+__device__ __forceinline__ void conv_tile(const ConvArgs& p, rsrc_t rx, rsrc_t rw, rsrc_t ro, float* lds, int mt,
+                                          int un, int kbeg, int kend) {
+  constexpr int WN = 4 / WM, BM = 32 * WM, BN = 32 * WN * NT;
+  const int m0 = mt * BM, n0 = un * 32 * WN;
+  OutMap om;
+  float* ldsB = lds + 2 * Cfg::SA;
+  if constexpr (PASS == PASS_FWD) {
+    PlainKC<BM, FLAG> la;            // FLAG: 128-bit loads of W rows (CKK % 4 == 0)
+    ConvFwdB<BN> lb;
+    la.init(rw, p.K, m0, p.M, p.K);
+    lb.init(rx, p.g, p.tab, n0, p.Ncols);
+    om.nchw = 1; om.ld = p.g.OHW; om.mtot = p.g.O; om.dHW = p.g.dOHW;
+    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
+  } else if constexpr (PASS == PASS_DGRAD) {
+    ConvDgradA<BM> la;
+    ConvDgradB<BN, FLAG> lb;         // FLAG: stride == 1
+    la.init(rw, p.g, p.tab, m0);
+    lb.init(rx, p.g, p.tab, n0, p.Ncols);
+    om.nchw = 1; om.ld = p.g.IHW; om.mtot = p.g.C; om.dHW = p.g.dIHW;
+    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
+  } else {
+    ConvWgradA<BM, FLAG> la;         // FLAG: 128-bit loads of dY (OHW % 4 == 0)
+    ConvWgradB<BN> lb;
+    la.init(rw, p.g, m0, kend);
+    lb.init(rx, p.g, p.tab, n0, p.Ncols, kend);
+    om.nchw = 0; om.ld = p.Ncols; om.mtot = 0; om.dHW = FastDiv{0, 0, 1};
+    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
+  }
+}
+
+template <int PASS, int WM, int NTMAX, bool FLAG>
+__global__ __launch_bounds__(256, 2) void conv_kernel(ConvArgs p) {
+  using Cfg = ConvCfg<PASS, WM, NTMAX, FLAG>;
+  __shared__ __attribute__((aligned(16))) float lds[2 * (Cfg::SA + Cfg::SB)];
+  const rsrc_t rx = make_rsrc(p.X, p.bytesX);
+  const rsrc_t rw = make_rsrc(p.W, p.bytesW);
+  int kbeg = 0, kend = p.K;
+  float* out = p.Out;
+  if (PASS == PASS_WGRAD && p.ksplit > 1) {
+    const int nkt = (p.K + BK - 1) / BK;
+    const int t0 = (int)((long long)nkt * blockIdx.y / p.ksplit);
+    const int t1 = (int)((long long)nkt * (blockIdx.y + 1) / p.ksplit);
+    kbeg = t0 * BK;
+    kend = t1 * BK < p.K ? t1 * BK : p.K;
+    out += (size_t)blockIdx.y * p.M * p.Ncols;
+  }
+  const rsrc_t ro = make_rsrc(out, p.bytesOut);
+  long long u0 = (long long)p.total_units * blockIdx.x / gridDim.x;
+  const long long u1 = (long long)p.total_units * (blockIdx.x + 1) / gridDim.x;
+  while (u0 < u1) {
+    const int mt = (int)(u0 / p.n_units), un = (int)(u0 - (long long)mt * p.n_units);
+    long long cnt = u1 - u0;
+    if (cnt > p.n_units - un) cnt = p.n_units - un;
+    const int nt = pick_units<NTMAX>((int)cnt);
+    switch (nt) {
+      case 1: conv_tile<PASS, Cfg, WM, 1, FLAG>(p, rx, rw, ro, lds, mt, un, kbeg, kend); break;
+      case 2: conv_tile<PASS, Cfg, WM, (NTMAX >= 2 ? 2 : 1), FLAG>(p, rx, rw, ro, lds, mt, un, kbeg, kend); break;
+      case 3: conv_tile<PASS, Cfg, WM, (NTMAX >= 3 ? 3 : 1), FLAG>(p, rx, rw, ro, lds, mt, un, kbeg, kend); break;
+      default: conv_tile<PASS, Cfg, WM, (NTMAX >= 4 ? 4 : 1), FLAG>(p, rx, rw, ro, lds, mt, un, kbeg, kend); break;
+    }
+    u0 += nt;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+static int fill_geom(const lnn_conv2d_desc* d, ConvGeom& g) {
+  if (!d) return set_error(LNN_ERR_INVALID, "conv2d: null descriptor");
+  const int v[] = {d->N, d->C, d->IH, d->IW, d->O, d->KH, d->KW, d->OH, d->OW, d->stride, d->dilation};
+  for (int x : v)
+    if (x <= 0) return set_error(LNN_ERR_INVALID, "conv2d: non-positive dimension in descriptor");
+  if (d->PADL < 0 || d->PADT < 0) return set_error(LNN_ERR_INVALID, "conv2d: negative padding");
+  g.N = d->N; g.C = d->C; g.IH = d->IH; g.IW = d->IW; g.O = d->O; g.KH = d->KH; g.KW = d->KW;
+  g.OH = d->OH; g.OW = d->OW; g.PADL = d->PADL; g.PADT = d->PADT; g.S = d->stride; g.D = d->dilation;
+  const uint64_t ihw = (uint64_t)d->IH * d->IW, ohw = (uint64_t)d->OH * d->OW, kk = (uint64_t)d->KH * d->KW;
+  const uint64_t xb = (uint64_t)d->N * d->C * ihw * 4, yb = (uint64_t)d->N * d->O * ohw * 4;
+  const uint64_t wb = (uint64_t)d->O * d->C * kk * 4;
+  if (xb > kMaxTensorBytes || yb > kMaxTensorBytes || wb > kMaxTensorBytes)
+    return set_error(LNN_ERR_UNSUPPORTED, "conv2d: a tensor of 2 GiB or more");
+  // coordinates must stay far below the sentinel used for masked elements
+  if ((uint64_t)d->OH * d->stride + (uint64_t)d->KH * d->dilation + d->PADT + d->IH >= (uint64_t)BIG / 2 ||
+      (uint64_t)d->OW * d->stride + (uint64_t)d->KW * d->dilation + d->PADL + d->IW >= (uint64_t)BIG / 2)
+    return set_error(LNN_ERR_UNSUPPORTED, "conv2d: coordinate range too large");
+  g.IHW = (int)ihw; g.OHW = (int)ohw; g.KK = (int)kk;
+  g.dOW = make_fastdiv(g.OW); g.dOHW = make_fastdiv(g.OHW);
+  g.dIW = make_fastdiv(g.IW); g.dIHW = make_fastdiv(g.IHW);
+  g.dS = make_fastdiv(g.S);
+  return LNN_OK;
+}
+
+static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const KEntry** out) {
+  const int K = (mode == 0 ? g.C : g.O) * g.KK;
+  const int Kpad = ((K + BK - 1) / BK) * BK + BK;
+  const std::array<int, 12> key = {mode, g.C, g.O, g.KH, g.KW, g.D, g.IH, g.IW, g.OH, g.OW, 0, 0};
+  auto it = ctx->tables.find(key);
+  if (it != ctx->tables.end()) {
+    *out = it->second;
+    return LNN_OK;
+  }
+  if (ctx->tables.size() >= 256) {   // bound the cache: drop everything once work queued so far is done
+    LNN_HIP(hipStreamSynchronize(ctx->stream));
+    for (auto& kv : ctx->tables) (void)hipFree(kv.second);
+    ctx->tables.clear();
+  }
+  KEntry* tab = nullptr;
+  hipError_t e = hipMalloc((void**)&tab, (size_t)Kpad * sizeof(KEntry));
+  if (e == hipErrorOutOfMemory) {
+    (void)hipGetLastError();
+    return set_error(LNN_ERR_OOM, "conv2d: out of device memory for the gather table");
+  }
+  LNN_HIP(e);
+  hipLaunchKernelGGL(build_ktable, dim3((Kpad + 255) / 256), dim3(256), 0, ctx->stream, tab, K, Kpad, mode, g);
+  LNN_HIP(hipGetLastError());
+  ctx->tables[key] = tab;
+  *out = tab;
+  return LNN_OK;
+}
+
+template <int PASS, int WM, int NTMAX>
+static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
+  constexpr int WN = 4 / WM, BM = 32 * WM;
+  const int m_tiles = (a.M + BM - 1) / BM;
+  a.n_units = (a.Ncols + 32 * WN - 1) / (32 * WN);
+  const long long total = (long long)m_tiles * a.n_units;
+  if (total > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
+  a.total_units = (int)total;
+  const long long slots = 2ll * ctx->cus;
+  int grid, ksplit = 1;
+  float* final_out = a.Out;
+  const int final_beta = a.beta;
+  if (PASS == PASS_WGRAD) {
+    // one full-width sub-tile per workgroup, then as many K slices as fill the chip
+    grid = (int)((total + NTMAX - 1) / NTMAX);
+    const int nkt = (a.K + BK - 1) / BK;
+    long long s = slots / grid;
+    if (s > nkt / 4) s = nkt / 4;
+    if (s > 1024) s = 1024;
+    if (s < 1) s = 1;
+    ksplit = (int)s;
+    if (ksplit > 1) {
+      const size_t need = (size_t)ksplit * a.M * a.Ncols * sizeof(float);
+      int st = ensure_workspace(ctx, need);
+      if (st != LNN_OK) return st;
+      a.Out = static_cast<float*>(ctx->ws);
+      a.beta = 0;
+    }
+  } else {
+    grid = (int)(total < slots ? total : slots);
+  }
+  a.ksplit = ksplit;
+  dim3 g(grid, ksplit, 1), b(256, 1, 1);
+  if (flag)
+    hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, true>), g, b, 0, ctx->stream, a);
+  else
+    hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, false>), g, b, 0, ctx->stream, a);
+  LNN_HIP(hipGetLastError());
+  if (ksplit > 1) {
+    const int n = a.M * a.Ncols;
+    hipLaunchKernelGGL(reduce_partials, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, final_out,
+                       static_cast<const float*>(ctx->ws), n, ksplit, final_beta);
+    LNN_HIP(hipGetLastError());
+  }
+  return LNN_OK;
+}
+
+template <int PASS>
+static int launch_by_m(DeviceCtx* ctx, ConvArgs& a, bool flag) {
+  if (a.M > 64) return launch_pass<PASS, 4, 4>(ctx, a, flag);
+  if (a.M > 32) return launch_pass<PASS, 2, 4>(ctx, a, flag);
+  return launch_pass<PASS, 1, 2>(ctx, a, flag);
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta) {
+  ConvArgs a;
+  int st = fill_geom(d, a.g);
+  if (st != LNN_OK) return st;
+  if (!X || !W || !Y) return set_error(LNN_ERR_INVALID, "conv2d_fwd: null pointer");
+  st = get_table(ctx, a.g, 0, &a.tab);
+  if (st != LNN_OK) return st;
+  const ConvGeom& g = a.g;
+  a.X = X; a.W = W; a.Out = Y;
+  a.bytesX = (uint32_t)((uint64_t)g.N * g.C * g.IHW * 4);
+  a.bytesW = (uint32_t)((uint64_t)g.O * g.C * g.KK * 4);
+  a.bytesOut = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
+  a.M = g.O; a.Ncols = g.N * g.OHW; a.K = g.C * g.KK;
+  a.beta = beta ? 1 : 0;
+  return launch_by_m<PASS_FWD>(ctx, a, a.K % 4 == 0 && aligned16(W));
+}
+
+int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta) {
+  ConvArgs a;
+  int st = fill_geom(d, a.g);
+  if (st != LNN_OK) return st;
+  if (!dY || !W || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
+  st = get_table(ctx, a.g, 1, &a.tab);
+  if (st != LNN_OK) return st;
+  const ConvGeom& g = a.g;
+  a.X = dY; a.W = W; a.Out = dX;
+  a.bytesX = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
+  a.bytesW = (uint32_t)((uint64_t)g.O * g.C * g.KK * 4);
+  a.bytesOut = (uint32_t)((uint64_t)g.N * g.C * g.IHW * 4);
+  a.M = g.C; a.Ncols = g.N * g.IHW; a.K = g.O * g.KK;
+  a.beta = beta ? 1 : 0;
+  return launch_by_m<PASS_DGRAD>(ctx, a, g.S == 1);
+}
+
+int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
+  ConvArgs a;
+  int st = fill_geom(d, a.g);
+  if (st != LNN_OK) return st;
+  if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");
+  st = get_table(ctx, a.g, 0, &a.tab);
+  if (st != LNN_OK) return st;
+  const ConvGeom& g = a.g;
+  a.X = X; a.W = dY; a.Out = dW;
+  a.bytesX = (uint32_t)((uint64_t)g.N * g.C * g.IHW * 4);
+  a.bytesW = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
+  a.bytesOut = (uint32_t)((uint64_t)g.O * g.C * g.KK * 4);
+  a.M = g.O; a.Ncols = g.C * g.KK; a.K = g.N * g.OHW;
+  a.beta = beta ? 1 : 0;
+  return launch_by_m<PASS_WGRAD>(ctx, a, g.OHW % 4 == 0 && aligned16(dY));
+}
+
+}  // namespace lnn

@@ -1,0 +1,392 @@
+// Bandwidth-bound helpers around the contraction kernels: fill, pointwise
+// forward/backward, broadcasting binary ops, axis reductions, transpose,
+// materialised unfold and the SGD update.  One grid-stride thread per element;
+// element counts are below 2^31 (every tensor is smaller than 2 GiB), so index
+// decomposition is done in 32-bit arithmetic.
+#include "common.hpp"
+
+namespace lnn {
+
+constexpr int kMaxRank = 8;
+struct Dims {
+  int rank;
+  int shape[kMaxRank];
+  long long sa[kMaxRank];   // per-axis element strides of operand a (0 = broadcast)
+  long long sb[kMaxRank];
+};
+
+static inline dim3 grid_for(uint64_t n, int cus) {
+  uint64_t blocks = (n + 255) / 256;
+  const uint64_t cap = (uint64_t)cus * 16;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return dim3((unsigned)blocks);
+}
+
+__global__ void fill_u32_kernel(uint32_t* dst, uint32_t v, uint64_t n) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x)
+    dst[i] = v;
+}
+
+__device__ __forceinline__ float ew_f(int op, float x, float p0) {
+  switch (op) {
+    case LNN_EW_ADD_CONST: return x + p0;
+    case LNN_EW_MUL_CONST: return x * p0;
+    case LNN_EW_LEAKY_RELU: return x >= 0.0f ? x : p0 * x;
+    case LNN_EW_SQUARE: return x * x;
+    default: return x >= 0.0f ? x : 0.0f;
+  }
+}
+__device__ __forceinline__ float ew_df(int op, float x, float p0) {
+  switch (op) {
+    case LNN_EW_ADD_CONST: return 1.0f;
+    case LNN_EW_MUL_CONST: return p0;
+    case LNN_EW_LEAKY_RELU: return x >= 0.0f ? 1.0f : p0;
+    case LNN_EW_SQUARE: return 2.0f * x;
+    default: return x >= 0.0f ? 1.0f : 0.0f;
+  }
+}
+
+__global__ void ew_fwd_kernel(int op, uint64_t n, const float* in, float* out, float p0, int beta) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const float r = ew_f(op, in[i], p0);
+    out[i] = beta ? out[i] + r : r;
+  }
+}
+
+__global__ void ew_bwd_kernel(int op, uint64_t n, const float* in, const float* dout, float* din, float p0) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x)
+    din[i] += dout[i] * ew_df(op, in[i], p0);
+}
+
+__global__ void binary_bcast_kernel(int op, Dims d, uint64_t n, const float* a, const float* b, float* out, int beta) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    uint32_t g = (uint32_t)i;
+    long long oa = 0, ob = 0;
+    for (int ax = d.rank - 1; ax >= 0; --ax) {
+      const uint32_t x = g % (uint32_t)d.shape[ax];
+      g /= (uint32_t)d.shape[ax];
+      oa += (long long)x * d.sa[ax];
+      ob += (long long)x * d.sb[ax];
+    }
+    const float x = a[oa], y = b[ob];
+    const float r = op == 0 ? x + y : (op == 1 ? x - y : x * y);
+    out[i] = beta ? out[i] + r : r;
+  }
+}
+
+// Reduction plan: kept axes index the output (row-major in axis order), reduced
+// axes are walked by the threads of one workgroup (and, for long reductions,
+// by several workgroups that leave partial sums for a second pass).
+struct RedPlan {
+  int nk, nr;
+  int kshape[kMaxRank], rshape[kMaxRank];
+  long long kstride[kMaxRank], rstride[kMaxRank];
+  uint64_t outs, red;
+};
+
+__device__ __forceinline__ long long offset_of(uint32_t idx, int n, const int* shape, const long long* stride) {
+  long long off = 0;
+  for (int ax = n - 1; ax >= 0; --ax) {
+    const uint32_t x = idx % (uint32_t)shape[ax];
+    idx /= (uint32_t)shape[ax];
+    off += (long long)x * stride[ax];
+  }
+  return off;
+}
+
+// grid = (outs, parts).  dst[o*parts + part] = partial sum (parts > 1) or the
+// finished value (parts == 1: scaled, optionally accumulated).
+__global__ void reduce_sum_kernel(RedPlan p, const float* in, float* dst, int parts, float scale, int beta) {
+  __shared__ float sh[256];
+  const uint64_t o = blockIdx.x;
+  const int part = blockIdx.y;
+  const long long base = offset_of((uint32_t)o, p.nk, p.kshape, p.kstride);
+  const uint64_t r0 = p.red * part / parts, r1 = p.red * (part + 1) / parts;
+  float s = 0.0f;
+  for (uint64_t r = r0 + threadIdx.x; r < r1; r += 256) s += in[base + offset_of((uint32_t)r, p.nr, p.rshape, p.rstride)];
+  sh[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) sh[threadIdx.x] += sh[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    if (parts > 1) {
+      dst[o * parts + part] = sh[0];
+    } else {
+      const float r = sh[0] * scale;
+      dst[o] = beta ? dst[o] + r : r;
+    }
+  }
+}
+
+__global__ void reduce_finish_kernel(const float* part, float* out, uint64_t outs, int parts, float scale, int beta) {
+  const uint64_t o = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x;
+  if (o >= outs) return;
+  float s = 0.0f;
+  for (int k = 0; k < parts; ++k) s += part[o * parts + k];
+  s *= scale;
+  out[o] = beta ? out[o] + s : s;
+}
+
+// din[idx] += scale * dout[kept part of idx]
+__global__ void reduce_bwd_kernel(Dims d, uint64_t n, float scale, const float* dout, float* din) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    uint32_t g = (uint32_t)i;
+    long long oa = 0;
+    for (int ax = d.rank - 1; ax >= 0; --ax) {
+      const uint32_t x = g % (uint32_t)d.shape[ax];
+      g /= (uint32_t)d.shape[ax];
+      oa += (long long)x * d.sa[ax];
+    }
+    din[i] += scale * dout[oa];
+  }
+}
+
+// out[perm(idx)] (+)= in[idx]; d.sa holds, per input axis, the stride of that axis in the output.
+__global__ void transpose_kernel(Dims d, uint64_t n, const float* in, float* out, int beta) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    uint32_t g = (uint32_t)i;
+    long long oo = 0;
+    for (int ax = d.rank - 1; ax >= 0; --ax) {
+      const uint32_t x = g % (uint32_t)d.shape[ax];
+      g /= (uint32_t)d.shape[ax];
+      oo += (long long)x * d.sa[ax];
+    }
+    out[oo] = beta ? out[oo] + in[i] : in[i];
+  }
+}
+
+struct UnfoldArgs {
+  int N, C, H, W, OH, OW, KH, KW, PADL, PADT, D, S, order, transposed;
+};
+
+// One thread per element of the unfolded matrix, written in row-major order
+// of the symbol string (last symbol fastest).
+__global__ void unfold2d_kernel(UnfoldArgs a, uint64_t n, const float* in, float* out, int beta) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    uint32_t g = (uint32_t)i;
+    int on, oc, oh, ow, oj, oi;
+    if (a.order == 0) {   // C J I N H W
+      ow = (int)(g % a.OW); g /= a.OW;
+      oh = (int)(g % a.OH); g /= a.OH;
+      on = (int)(g % a.N);  g /= a.N;
+      oi = (int)(g % a.KW); g /= a.KW;
+      oj = (int)(g % a.KH); g /= a.KH;
+      oc = (int)g;
+    } else {              // N H W C J I
+      oi = (int)(g % a.KW); g /= a.KW;
+      oj = (int)(g % a.KH); g /= a.KH;
+      oc = (int)(g % a.C);  g /= a.C;
+      ow = (int)(g % a.OW); g /= a.OW;
+      oh = (int)(g % a.OH); g /= a.OH;
+      on = (int)g;
+    }
+    int ih, iw;
+    bool ok;
+    if (!a.transposed) {
+      ih = -a.PADT + oj * a.D + oh * a.S;
+      iw = -a.PADL + oi * a.D + ow * a.S;
+      ok = ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+    } else {
+      const int nh = a.PADT + oh - oj * a.D, nw = a.PADL + ow - oi * a.D;
+      ih = nh >= 0 ? nh / a.S : 0;
+      iw = nw >= 0 ? nw / a.S : 0;
+      ok = nh >= 0 && nw >= 0 && ih * a.S == nh && iw * a.S == nw && ih < a.H && iw < a.W;
+    }
+    const float v = ok ? in[(((size_t)on * a.C + oc) * a.H + ih) * a.W + iw] : 0.0f;
+    out[i] = beta ? out[i] + v : v;
+  }
+}
+
+__global__ void sgd_kernel(uint64_t n, float* v, const float* g, float* acc, float momentum, float lr, int nesterov) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const float a = momentum * acc[i] - lr * g[i];
+    acc[i] = a;
+    v[i] += nesterov ? momentum * a - lr * g[i] : a;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host launchers (called from the C ABI)
+// ---------------------------------------------------------------------------
+int launch_fill_u32(DeviceCtx* ctx, void* dst, uint32_t pattern, uint64_t count) {
+  if (count == 0) return LNN_OK;
+  hipLaunchKernelGGL(fill_u32_kernel, grid_for(count, ctx->cus), dim3(256), 0, ctx->stream,
+                     static_cast<uint32_t*>(dst), pattern, count);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+int launch_ew_fwd(DeviceCtx* ctx, int op, uint64_t n, const float* in, float* out, float p0, int beta) {
+  if (op < 0 || op > LNN_EW_RELU) return set_error(LNN_ERR_INVALID, "ew_fwd: unknown op");
+  if (n == 0) return LNN_OK;
+  hipLaunchKernelGGL(ew_fwd_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, op, n, in, out, p0, beta ? 1 : 0);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+int launch_ew_bwd(DeviceCtx* ctx, int op, uint64_t n, const float* in, const float* dout, float* din, float p0) {
+  if (op < 0 || op > LNN_EW_RELU) return set_error(LNN_ERR_INVALID, "ew_bwd: unknown op");
+  if (n == 0) return LNN_OK;
+  hipLaunchKernelGGL(ew_bwd_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, op, n, in, dout, din, p0);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+static int check_rank(int rank, const int32_t* shape, const char* who) {
+  if (rank < 1 || rank > kMaxRank || !shape) return set_error(LNN_ERR_INVALID, std::string(who) + ": rank must be 1..8");
+  for (int i = 0; i < rank; ++i)
+    if (shape[i] <= 0) return set_error(LNN_ERR_INVALID, std::string(who) + ": non-positive extent");
+  return LNN_OK;
+}
+
+int launch_binary_bcast(DeviceCtx* ctx, int op, int rank, const int32_t* os, const int32_t* as, const int32_t* bs,
+                        const float* a, const float* b, float* out, int beta) {
+  if (op < 0 || op > 2) return set_error(LNN_ERR_INVALID, "binary_bcast: unknown op");
+  int st = check_rank(rank, os, "binary_bcast");
+  if (st != LNN_OK) return st;
+  Dims d;
+  d.rank = rank;
+  uint64_t n = 1;
+  long long ca = 1, cb = 1;
+  for (int ax = rank - 1; ax >= 0; --ax) {
+    if ((as[ax] != os[ax] && as[ax] != 1) || (bs[ax] != os[ax] && bs[ax] != 1))
+      return set_error(LNN_ERR_INVALID, "binary_bcast: shapes do not broadcast");
+    d.shape[ax] = os[ax];
+    d.sa[ax] = as[ax] == 1 ? 0 : ca;
+    d.sb[ax] = bs[ax] == 1 ? 0 : cb;
+    ca *= as[ax];
+    cb *= bs[ax];
+    n *= (uint64_t)os[ax];
+  }
+  hipLaunchKernelGGL(binary_bcast_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, op, d, n, a, b, out,
+                     beta ? 1 : 0);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+int launch_reduce_sum(DeviceCtx* ctx, int rank, const int32_t* shape, uint32_t mask, float scale, const float* in,
+                      float* out, int beta) {
+  int st = check_rank(rank, shape, "reduce_sum");
+  if (st != LNN_OK) return st;
+  RedPlan p;
+  p.nk = p.nr = 0;
+  p.outs = p.red = 1;
+  long long stride = 1;
+  long long strides[kMaxRank];
+  for (int ax = rank - 1; ax >= 0; --ax) {
+    strides[ax] = stride;
+    stride *= shape[ax];
+  }
+  for (int ax = 0; ax < rank; ++ax) {
+    if (mask & (1u << ax)) {
+      p.rshape[p.nr] = shape[ax];
+      p.rstride[p.nr++] = strides[ax];
+      p.red *= (uint64_t)shape[ax];
+    } else {
+      p.kshape[p.nk] = shape[ax];
+      p.kstride[p.nk++] = strides[ax];
+      p.outs *= (uint64_t)shape[ax];
+    }
+  }
+  if (p.outs > 0x7fffffffull) return set_error(LNN_ERR_UNSUPPORTED, "reduce_sum: too many outputs");
+  // long reductions with few outputs are split so the whole chip takes part
+  int parts = 1;
+  if (p.red >= 8192) {
+    uint64_t want = (uint64_t)ctx->cus * 4 / p.outs;
+    uint64_t most = p.red / 2048;
+    if (want > most) want = most;
+    if (want > 1024) want = 1024;
+    if (want > 1) parts = (int)want;
+  }
+  float* dst = out;
+  if (parts > 1) {
+    st = ensure_workspace(ctx, (size_t)p.outs * parts * sizeof(float));
+    if (st != LNN_OK) return st;
+    dst = static_cast<float*>(ctx->ws);
+  }
+  hipLaunchKernelGGL(reduce_sum_kernel, dim3((unsigned)p.outs, parts), dim3(256), 0, ctx->stream, p, in, dst, parts,
+                     scale, beta ? 1 : 0);
+  LNN_HIP(hipGetLastError());
+  if (parts > 1) {
+    hipLaunchKernelGGL(reduce_finish_kernel, dim3((unsigned)((p.outs + 255) / 256)), dim3(256), 0, ctx->stream,
+                       static_cast<const float*>(dst), out, p.outs, parts, scale, beta ? 1 : 0);
+    LNN_HIP(hipGetLastError());
+  }
+  return LNN_OK;
+}
+
+int launch_reduce_sum_bwd(DeviceCtx* ctx, int rank, const int32_t* shape, uint32_t mask, float scale,
+                          const float* dout, float* din) {
+  int st = check_rank(rank, shape, "reduce_sum_bwd");
+  if (st != LNN_OK) return st;
+  Dims d;
+  d.rank = rank;
+  uint64_t n = 1;
+  long long c = 1;
+  for (int ax = rank - 1; ax >= 0; --ax) {
+    d.shape[ax] = shape[ax];
+    const bool red = mask & (1u << ax);
+    d.sa[ax] = red ? 0 : c;
+    d.sb[ax] = 0;
+    if (!red) c *= shape[ax];
+    n *= (uint64_t)shape[ax];
+  }
+  hipLaunchKernelGGL(reduce_bwd_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, d, n, scale, dout, din);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+int launch_transpose(DeviceCtx* ctx, int rank, const int32_t* shape, const int32_t* axes, const float* in, float* out,
+                     int beta) {
+  int st = check_rank(rank, shape, "transpose");
+  if (st != LNN_OK) return st;
+  bool seen[kMaxRank] = {false};
+  for (int i = 0; i < rank; ++i) {
+    if (axes[i] < 0 || axes[i] >= rank || seen[axes[i]]) return set_error(LNN_ERR_INVALID, "transpose: axes are not a permutation");
+    seen[axes[i]] = true;
+  }
+  Dims d;
+  d.rank = rank;
+  uint64_t n = 1;
+  long long ostride[kMaxRank];
+  long long c = 1;
+  for (int i = rank - 1; i >= 0; --i) {   // output axis i has extent shape[axes[i]]
+    ostride[i] = c;
+    c *= shape[axes[i]];
+  }
+  for (int i = 0; i < rank; ++i) {
+    d.shape[i] = shape[i];
+    d.sb[i] = 0;
+    n *= (uint64_t)shape[i];
+  }
+  for (int i = 0; i < rank; ++i) d.sa[axes[i]] = ostride[i];
+  hipLaunchKernelGGL(transpose_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, d, n, in, out, beta ? 1 : 0);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+int launch_unfold2d(DeviceCtx* ctx, int N, int C, int H, int W, int OH, int OW, int KH, int KW, int PADL, int PADT,
+                    int D, int S, int order, int transposed, const float* in, float* out, int beta) {
+  const int v[] = {N, C, H, W, OH, OW, KH, KW, D, S};
+  for (int x : v)
+    if (x <= 0) return set_error(LNN_ERR_INVALID, "unfold2d: non-positive dimension");
+  if (order != 0 && order != 1) return set_error(LNN_ERR_INVALID, "unfold2d: order must be 0 or 1");
+  UnfoldArgs a = {N, C, H, W, OH, OW, KH, KW, PADL, PADT, D, S, order, transposed ? 1 : 0};
+  const uint64_t n = (uint64_t)N * C * OH * OW * KH * KW;
+  hipLaunchKernelGGL(unfold2d_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, a, n, in, out, beta ? 1 : 0);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+int launch_sgd(DeviceCtx* ctx, uint64_t n, float* v, const float* g, float* acc, float momentum, float lr, int nesterov) {
+  if (n == 0) return LNN_OK;
+  hipLaunchKernelGGL(sgd_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, n, v, g, acc, momentum, lr,
+                     nesterov ? 1 : 0);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+}  // namespace lnn

@@ -1,0 +1,255 @@
+"""GPU parity tests of the C ABI (liblitenn_hip.so) against the CPU oracle.
+
+Bars: bit-exact on integer-valued data (the reference's own test trick,
+conv2D.py:90-115, matmul.py:192-225: all partial sums are exactly
+representable, so the result does not depend on summation order) and
+normalised max error <= 1e-4 against the fp64 oracle on the seeded float
+data of the benchmark configurations.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import (info_conv2d, conv2d_all, conv2d_fwd, conv2d_dx, conv2d_dw, unfold_index_map,
+                    unfold_T_index_map, matmul_fwd)
+from tests.gpu_util import DevArr, rel_err, say
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def _desc(api, xs, ws, s, d, padding):
+    N, C, IH, IW = xs
+    O, _, KH, KW = ws
+    ci = info_conv2d(IH, IW, KH, KW, s, d, padding)
+    return api.conv_desc(N, C, IH, IW, O, KH, KW, ci.OH, ci.OW, ci.PADL, ci.PADT, s, d), ci
+
+
+def _run_conv(api, x, w, dy, s, d, padding, prefill=None):
+    """fwd (beta 0), dgrad and wgrad through the C ABI.  prefill=None: grads
+    written with beta 0; else grads pre-filled with that value and beta 1."""
+    desc, ci = _desc(api, x.shape, w.shape, s, d, padding)
+    X, W, dY = DevArr(api, x), DevArr(api, w), DevArr(api, dy)
+    Y = DevArr(api, shape=dy.shape, fill=np.nan)
+    beta = 0 if prefill is None else 1
+    dX = DevArr(api, shape=x.shape, fill=np.nan if prefill is None else prefill)
+    dW = DevArr(api, shape=w.shape, fill=np.nan if prefill is None else prefill)
+    api.conv2d_fwd(0, desc, X.ptr, W.ptr, Y.ptr, 0)
+    api.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, beta)
+    api.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW.ptr, beta)
+    return Y.get(), dX.get(), dW.get()
+
+
+# ------------------------------------------------------------------ GEMM
+@pytest.mark.parametrize('ta,tb', [(0, 0), (0, 1), (1, 0)])
+def test_gemm_integer_exact(hip, ta, tb):
+    rs = np.random.RandomState(10 + 2 * ta + tb)
+    shapes = [(1, 1, 1, 1), (1, 5, 7, 3), (1, 33, 65, 17), (1, 128, 128, 16), (1, 130, 257, 100),
+              (3, 8, 32, 16), (2, 70, 40, 24), (1, 64, 512, 48), (1, 256, 384, 160), (1, 2, 3000, 5),
+              (4, 1, 9, 1), (1, 97, 31, 1000)]
+    for batch, M, N, K in shapes:
+        say(f'gemm ta={ta} tb={tb} batch={batch} M={M} N={N} K={K}')
+        a = rs.randint(16, size=(batch, K, M) if ta else (batch, M, K)).astype(np.float32)
+        b = rs.randint(16, size=(batch, N, K) if tb else (batch, K, N)).astype(np.float32)
+        c0 = rs.randint(8, size=(batch, M, N)).astype(np.float32)
+        ref = np.matmul(a.transpose(0, 2, 1) if ta else a, b.transpose(0, 2, 1) if tb else b)
+        A, B = DevArr(hip, a), DevArr(hip, b)
+        for beta in (0, 1):
+            C = DevArr(hip, c0)
+            hip.gemm(0, ta, tb, batch, M, N, K, A.ptr, a.shape[2], a.shape[1] * a.shape[2],
+                     B.ptr, b.shape[2], b.shape[1] * b.shape[2], C.ptr, N, M * N, beta)
+            got = C.get()
+            assert np.array_equal(got, ref + (c0 if beta else 0)), (batch, M, N, K, beta)
+
+
+def test_gemm_leading_dimensions_and_unaligned(hip):
+    rs = np.random.RandomState(3)
+    M, N, K, lda, ldb, ldc = 45, 70, 37, 41, 75, 77
+    a = rs.randint(16, size=(M, lda)).astype(np.float32)
+    b = rs.randint(16, size=(K, ldb)).astype(np.float32)
+    c0 = rs.randint(16, size=(M, ldc)).astype(np.float32)
+    A, B, C = DevArr(hip, a), DevArr(hip, b), DevArr(hip, c0)
+    say('gemm with padded leading dimensions')
+    hip.gemm(0, 0, 0, 1, M, N, K, A.ptr, lda, 0, B.ptr, ldb, 0, C.ptr, ldc, 0, 0)
+    got = C.get()
+    assert np.array_equal(got[:, :N], a[:, :K] @ b[:, :N])
+    assert np.array_equal(got[:, N:], c0[:, N:])          # padding columns untouched
+    # operands that start 4 bytes into an allocation take the scalar-load path
+    a2 = rs.randint(16, size=(64 * 64 + 1)).astype(np.float32)
+    A2 = DevArr(hip, a2)
+    b2 = rs.randint(16, size=(64, 64)).astype(np.float32)
+    B2, C2 = DevArr(hip, b2), DevArr(hip, shape=(64, 64), fill=0.0)
+    say('gemm with a 4-byte-offset operand')
+    hip.gemm(0, 0, 0, 1, 64, 64, 64, A2.ptr + 4, 64, 0, B2.ptr, 64, 0, C2.ptr, 64, 0, 0)
+    assert np.array_equal(C2.get(), a2[1:].reshape(64, 64) @ b2)
+
+
+def test_gemm_float_tolerance(hip):
+    rs = np.random.RandomState(0)
+    M = N = K = 768
+    a, b, dc = (rs.normal(0, 1, (M, K)).astype(np.float32) for _ in range(3))
+    A, B, D = DevArr(hip, a), DevArr(hip, b), DevArr(hip, dc)
+    C, dA, dB = (DevArr(hip, shape=(M, N), fill=0.0) for _ in range(3))
+    say('gemm 768^3 fwd / dA / dB')
+    hip.gemm(0, 0, 0, 1, M, N, K, A.ptr, K, 0, B.ptr, N, 0, C.ptr, N, 0, 0)
+    hip.gemm(0, 0, 1, 1, M, K, N, D.ptr, N, 0, B.ptr, N, 0, dA.ptr, K, 0, 1)
+    hip.gemm(0, 1, 0, 1, K, N, M, A.ptr, K, 0, D.ptr, N, 0, dB.ptr, N, 0, 1)
+    a64, b64, d64 = a.astype(np.float64), b.astype(np.float64), dc.astype(np.float64)
+    assert rel_err(C.get(), a64 @ b64) <= TOL
+    assert rel_err(dA.get(), d64 @ b64.T) <= TOL
+    assert rel_err(dB.get(), a64.T @ d64) <= TOL
+
+
+def test_gemm_argument_errors(hip):
+    A = DevArr(hip, shape=(16, 16), fill=0.0)
+    with pytest.raises(hip.HipException) as e:
+        hip.gemm(0, 0, 0, 1, 16, 16, 0, A.ptr, 16, 0, A.ptr, 16, 0, A.ptr, 16, 0, 0)
+    assert e.value.code == hip.ERR_INVALID
+    with pytest.raises(hip.HipException):
+        hip.gemm(0, 0, 0, 1, 16, 16, 16, A.ptr, 8, 0, A.ptr, 16, 0, A.ptr, 16, 0, 0)
+    with pytest.raises(hip.HipException) as e:
+        hip.gemm(0, 1, 1, 1, 16, 16, 16, A.ptr, 16, 0, A.ptr, 16, 0, A.ptr, 16, 0, 0)
+    assert e.value.code == hip.ERR_UNSUPPORTED
+    with pytest.raises(hip.HipException) as e:
+        hip.malloc(99, 16)
+    assert e.value.code == hip.ERR_NO_DEVICE
+
+
+# ------------------------------------------------------------------ conv
+def _grid(pads):
+    # the reference's own grid (conv2D.py:77-85)
+    for padding, d, s, ks, n, ic, oc, hw in itertools.product(pads, [1, 2], [1, 2, 3], [7, 5, 3, 1], [1, 4],
+                                                                [1, 2, 4], [1, 2, 4], [4, 8, 16]):
+        if padding == 'valid' and hw < ks:
+            continue
+        yield padding, d, s, ks, n, ic, oc, hw
+
+
+@pytest.mark.parametrize('pads', [['same'], ['valid'], [0], [1], [2]])
+def test_conv_reference_grid_integer_exact(hip, pads):
+    """Every case of the reference's conv2d_test: Y exact; gradients written
+    into buffers pre-filled with 1.0 must equal 1 + oracle (pins '+=')."""
+    rs = np.random.RandomState(len(str(pads)) * 7 + (pads[0] if isinstance(pads[0], int) else 0))
+    cnt = 0
+    for padding, d, s, ks, n, ic, oc, hw in _grid(pads):
+        if cnt % 100 == 0:
+            say(f'conv grid padding={padding} case {cnt}: d={d} s={s} ks={ks} n={n} ic={ic} oc={oc} hw={hw}')
+        x = rs.randint(16, size=(n, ic, hw, hw)).astype(np.float32)
+        w = rs.randint(16, size=(oc, ic, ks, ks)).astype(np.float32)
+        ci = info_conv2d(hw, hw, ks, ks, s, d, padding)
+        dy = rs.randint(16, size=(n, oc, ci.OH, ci.OW)).astype(np.float32)
+        y, dx, dw = _run_conv(hip, x, w, dy, s, d, padding, prefill=1.0)
+        ry, rdx, rdw = conv2d_all(x, w, dy, s, d, padding)
+        tag = (padding, d, s, ks, n, ic, oc, hw)
+        assert np.array_equal(y, ry), ('fwd', tag)
+        assert np.array_equal(dx - 1.0, rdx), ('dX', tag)
+        assert np.array_equal(dw - 1.0, rdw), ('dW', tag)
+        cnt += 1
+    assert cnt > 500
+
+
+def test_conv_odd_corners_integer_exact(hip):
+    """Even kernels with asymmetric 'same' padding, non-square images and
+    kernels, explicit 4-tuple pads, output clamped to 1x1, many channels
+    (several M tiles, ragged K), large strides."""
+    rs = np.random.RandomState(5)
+    cases = [
+        ((2, 3, 9, 7), (5, 3, 2, 4), 1, 1, 'same'), ((1, 2, 4, 4), (3, 2, 7, 7), 1, 1, 0),
+        ((2, 5, 12, 10), (6, 5, 3, 2), 2, 1, (1, 2, 0, 3)), ((1, 130, 6, 6), (70, 130, 3, 3), 1, 1, 'same'),
+        ((3, 33, 10, 10), (129, 33, 1, 1), 1, 1, 'same'), ((2, 4, 20, 20), (4, 4, 3, 3), 4, 3, 2),
+        ((1, 1, 40, 40), (1, 1, 5, 5), 3, 2, 'same'), ((2, 16, 17, 13), (40, 16, 4, 4), 2, 1, 'same'),
+        ((1, 7, 30, 30), (9, 7, 3, 3), 1, 1, 'valid'), ((5, 3, 8, 8), (2, 3, 8, 8), 1, 1, 'valid'),
+    ]
+    for xs, ws, s, d, padding in cases:
+        say(f'conv corner x={xs} w={ws} s={s} d={d} pad={padding}')
+        x = rs.randint(8, size=xs).astype(np.float32)
+        w = rs.randint(8, size=ws).astype(np.float32)
+        ci = info_conv2d(xs[2], xs[3], ws[2], ws[3], s, d, padding)
+        dy = rs.randint(8, size=(xs[0], ws[0], ci.OH, ci.OW)).astype(np.float32)
+        ry, rdx, rdw = conv2d_all(x, w, dy, s, d, padding)
+        for prefill in (None, 2.0):
+            y, dx, dw = _run_conv(hip, x, w, dy, s, d, padding, prefill=prefill)
+            off = 0.0 if prefill is None else prefill
+            assert np.array_equal(y, ry), ('fwd', xs, ws)
+            assert np.array_equal(dx - off, rdx), ('dX', xs, ws)
+            assert np.array_equal(dw - off, rdw), ('dW', xs, ws)
+
+
+# benchmark geometries at a reduced batch (the oracle materialises im2col in fp64)
+_BENCH = {
+    'cfg1': ((8, 3, 64, 64), (32, 3, 3, 3), 1, 1, 'same', 0),
+    'cfg3': ((2, 128, 56, 56), (128, 128, 3, 3), 1, 1, 'same', 0),
+    'cfg4a': ((2, 3, 224, 224), (64, 3, 7, 7), 2, 1, 3, 0),
+    'cfg4b': ((4, 256, 28, 28), (512, 256, 1, 1), 1, 1, 'same', 1),
+    'cfg4c': ((2, 64, 64, 64), (64, 64, 3, 3), 1, 2, 2, 2),
+    'cfg5_L1': ((2, 3, 128, 128), (64, 3, 5, 5), 2, 1, 2, 0),
+    'cfg5_L2': ((2, 64, 64, 64), (128, 64, 5, 5), 2, 1, 2, 0),
+    'cfg5_L3': ((4, 128, 32, 32), (256, 128, 5, 5), 2, 1, 2, 0),
+    'cfg5_L4': ((8, 256, 16, 16), (512, 256, 5, 5), 2, 1, 2, 0),
+}
+
+
+@pytest.mark.parametrize('name', list(_BENCH))
+def test_conv_benchmark_geometries_float(hip, name):
+    xs, ws, s, d, padding, seed = _BENCH[name]
+    rs = np.random.RandomState(seed)
+    x = rs.uniform(-1, 1, xs).astype(np.float32)
+    w = rs.normal(0, np.sqrt(2.0 / (ws[1] * ws[2] * ws[3])), ws).astype(np.float32)
+    ci = info_conv2d(xs[2], xs[3], ws[2], ws[3], s, d, padding)
+    dy = rs.normal(0, 1, (xs[0], ws[0], ci.OH, ci.OW)).astype(np.float32)
+    say(f'conv {name} x={xs} w={ws} s={s} d={d} pad={padding}')
+    y, dx, dw = _run_conv(hip, x, w, dy, s, d, padding)
+    ry, rdx, rdw = conv2d_all(x, w, dy, s, d, padding)
+    errs = (rel_err(y, ry), rel_err(dx, rdx), rel_err(dw, rdw))
+    say(f'  normalised errors fwd/dX/dW = {errs}')
+    assert max(errs) <= TOL
+
+
+def test_conv_descriptor_errors(hip):
+    A = DevArr(hip, shape=(64,), fill=0.0)
+    bad = hip.conv_desc(1, 1, 4, 4, 1, 3, 3, 4, 4, 1, 1, 0, 1)          # stride 0
+    with pytest.raises(hip.HipException) as e:
+        hip.conv2d_fwd(0, bad, A.ptr, A.ptr, A.ptr, 0)
+    assert e.value.code == hip.ERR_INVALID
+    big = hip.conv_desc(4096, 4096, 64, 64, 1, 3, 3, 64, 64, 1, 1, 1, 1)  # 256 GiB input
+    with pytest.raises(hip.HipException) as e:
+        hip.conv2d_fwd(0, big, A.ptr, A.ptr, A.ptr, 0)
+    assert e.value.code == hip.ERR_UNSUPPORTED
+
+
+# ------------------------------------------------------------------ unfold / transpose
+def test_unfold_index_maps_bit_exact(hip):
+    """Input element i holds the value i+1 (exact in fp32 up to 2^24), so the
+    unfolded matrix reveals which flat input index every output element read."""
+    for padding, d, s, ks in itertools.product(['same', 'valid', 2], [1, 2], [1, 2, 3], [5, 3, 2, 1]):
+        n, c, o, h, w_ = 2, 3, 2, 9, 8
+        if padding == 'valid' and min(h, w_) < (ks - 1) * d + 1:
+            continue
+        ci = info_conv2d(h, w_, ks, ks, s, d, padding)
+        x = np.arange(1, n * c * h * w_ + 1, dtype=np.float32)
+        X = DevArr(hip, x)
+        for order, name in ((0, 'CJI_NHW'), (1, 'NHW_CJI')):
+            shape, m = unfold_index_map(n, c, h, w_, ci.OH, ci.OW, ks, ks, ci.PADL, ci.PADT, d, s, name)
+            out = DevArr(hip, shape=shape, fill=np.nan)
+            hip.unfold2d(0, n, c, h, w_, ci.OH, ci.OW, ks, ks, ci.PADL, ci.PADT, d, s, order, False, X.ptr, out.ptr)
+            assert np.array_equal(out.get().reshape(-1).astype(np.int64) - 1, m)
+        dy = np.arange(1, n * o * ci.OH * ci.OW + 1, dtype=np.float32)
+        DY = DevArr(hip, dy)
+        shape, m = unfold_T_index_map(n, o, ci.OH, ci.OW, h, w_, ks, ks, ci.PADL, ci.PADT, d, s)
+        out = DevArr(hip, shape=shape, fill=np.nan)
+        hip.unfold2d(0, n, o, ci.OH, ci.OW, h, w_, ks, ks, ci.PADL, ci.PADT, d, s, 1, True, DY.ptr, out.ptr)
+        assert np.array_equal(out.get().reshape(-1).astype(np.int64) - 1, m)
+
+
+def test_transpose_exact(hip):
+    rs = np.random.RandomState(1)
+    for rank in (2, 3, 4, 5):
+        for _ in range(4):
+            shape = tuple(int(v) for v in rs.randint(1, 9, size=rank))
+            axes = tuple(int(v) for v in rs.permutation(rank))
+            v = rs.randint(256, size=shape).astype(np.float32)
+            V = DevArr(hip, v)
+            out = DevArr(hip, shape=tuple(shape[a] for a in axes), fill=1.0)
+            hip.transpose(0, shape, axes, V.ptr, out.ptr, 1)
+            assert np.array_equal(out.get() - 1.0, v.transpose(axes))
