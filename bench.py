@@ -1,0 +1,338 @@
+#!/usr/bin/env python3
+"""Benchmark of the conv2D / matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
+
+Default workload (the configuration the headline metric is quoted on): the
+VGG-style 3x3 convolution layer, fp32 NCHW, N=32, C=128, H=W=56, O=128,
+stride 1, padding 'same'.  One step = forward + dX + dW (gradients accumulate
+into their buffers, as the reference's backward does), inputs resident in HBM.
+Prints ONE JSON line: whole-step TFLOP/s, the fp32-MFMA roofline fraction of
+the dominant kernel (timed with HIP events on the library's stream), and the
+CPU restatement of the reference algorithm timed on the host cores.
+
+--all additionally measures every benchmark configuration (conv geometries,
+the 4096^3 matmul with both gradients, the 4-layer encoder training step) and
+writes one JSON object per line to gpurun_out/bench_all.jsonl.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 2.4 GHz x 256 flop/clk/CU
+PEAK_HBM_GBS = 8000.0
+
+CONV_CONFIGS = {
+    # name: (x shape, w shape, stride, dilation, padding, seed)
+    'cfg1_stem3x3': ((8, 3, 64, 64), (32, 3, 3, 3), 1, 1, 'same', 0),
+    'cfg3_vgg3x3': ((32, 128, 56, 56), (128, 128, 3, 3), 1, 1, 'same', 0),
+    'cfg4a_stem7x7s2': ((32, 3, 224, 224), (64, 3, 7, 7), 2, 1, 3, 0),
+    'cfg4b_pointwise': ((64, 256, 28, 28), (512, 256, 1, 1), 1, 1, 'same', 1),
+    'cfg4c_dilated': ((16, 64, 64, 64), (64, 64, 3, 3), 1, 2, 2, 2),
+}
+
+
+def conv_info(xs, ws, s, d, padding):
+    from litenn_amd.core.info import InfoConv2D
+    return InfoConv2D(xs[2], xs[3], ws[2], ws[3], s, d, padding)
+
+
+def conv_tensors(xs, ws, s, d, padding, seed):
+    rs = np.random.RandomState(seed)
+    x = rs.uniform(-1, 1, xs).astype(np.float32)
+    w = rs.normal(0, np.sqrt(2.0 / (ws[1] * ws[2] * ws[3])), ws).astype(np.float32)
+    ci = conv_info(xs, ws, s, d, padding)
+    dy = rs.normal(0, 1, (xs[0], ws[0], ci.OH, ci.OW)).astype(np.float32)
+    return x, w, dy, ci
+
+
+class Dev:
+    """Device array helper over the C ABI."""
+
+    def __init__(self, api, array=None, shape=None):
+        self.api = api
+        if array is not None:
+            shape = array.shape
+        self.shape = tuple(shape)
+        self.count = int(np.prod(self.shape, dtype=np.int64))
+        self.ptr = api.malloc(0, self.count * 4)
+        if array is not None:
+            api.memcpy_h2d(0, self.ptr, np.ascontiguousarray(array, dtype=np.float32))
+        else:
+            api.fill_f32(0, self.ptr, 0.0, self.count)
+
+    def get(self):
+        out = np.empty(self.shape, np.float32)
+        self.api.memcpy_d2h(0, out, self.ptr)
+        return out
+
+    def zero(self):
+        self.api.fill_f32(0, self.ptr, 0.0, self.count)
+
+    def free(self):
+        self.api.free(0, self.ptr)
+
+
+def time_events(api, fn, iters):
+    """Average milliseconds of fn() over `iters` back-to-back launches, from
+    HIP events recorded on the stream the kernels run on."""
+    e0, e1 = api.Event(0), api.Event(0)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    return api.Event.elapsed_ms(e0, e1) / iters
+
+
+def rel_err(got, ref):
+    ref = np.asarray(ref, np.float64)
+    return float(np.abs(np.asarray(got, np.float64) - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
+    xs, ws, s, d, padding, seed = CONV_CONFIGS[name]
+    x, w, dy, ci = conv_tensors(xs, ws, s, d, padding, seed)
+    N, C, IH, IW = xs
+    O, _, KH, KW = ws
+    desc = api.conv_desc(N, C, IH, IW, O, KH, KW, ci.OH, ci.OW, ci.PADL, ci.PADT, s, d)
+    flops = 2.0 * N * O * ci.OH * ci.OW * C * KH * KW          # per pass
+    nx, nw, ny = x.size, w.size, dy.size
+    bytes_pass = {'fwd': 4.0 * (nx + nw + ny), 'dX': 4.0 * (ny + nw + 2 * nx), 'dW': 4.0 * (nx + ny + 2 * nw)}
+    X, W, dY = Dev(api, x), Dev(api, w), Dev(api, dy)
+    Y, dX, dW = Dev(api, shape=dy.shape), Dev(api, shape=xs), Dev(api, shape=ws)
+    passes = {
+        'fwd': lambda: api.conv2d_fwd(0, desc, X.ptr, W.ptr, Y.ptr, 0),
+        'dX': lambda: api.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, 1),
+        'dW': lambda: api.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW.ptr, 1),
+    }
+
+    def step():
+        for fn in passes.values():
+            fn()
+
+    for _ in range(warmup):
+        step()
+    api.synchronize(0)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    api.synchronize(0)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+
+    per_pass = {}
+    for k, fn in passes.items():
+        ms = time_events(api, fn, max(steps, 5))
+        per_pass[k] = {'ms': ms, 'tflops': flops / ms / 1e9, 'frac_mfma': flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS,
+                       'alg_gbs': bytes_pass[k] / ms / 1e6, 'frac_hbm': bytes_pass[k] / ms / 1e6 / PEAK_HBM_GBS}
+    dom = max(per_pass, key=lambda k: per_pass[k]['ms'])
+    # the roofline that binds is the one whose minimum time is larger
+    t_mfma = flops / (PEAK_FP32_MFMA_TFLOPS * 1e9)
+    t_hbm = bytes_pass[dom] / (PEAK_HBM_GBS * 1e6)
+    if t_mfma >= t_hbm:
+        roof = {'bound': 'mfma', 'kernel': dom, 'achieved': per_pass[dom]['tflops'], 'peak': PEAK_FP32_MFMA_TFLOPS,
+                'unit': 'TFLOP/s', 'frac': per_pass[dom]['frac_mfma'], 'traffic': None}
+    else:
+        roof = {'bound': 'hbm', 'kernel': dom, 'achieved': per_pass[dom]['alg_gbs'], 'peak': PEAK_HBM_GBS,
+                'unit': 'GB/s', 'frac': per_pass[dom]['frac_hbm'], 'traffic': None}
+
+    # parity on the very tensors that were timed (fresh outputs, no accumulation history)
+    dX.zero()
+    dW.zero()
+    step()
+    got = (Y.get(), dX.get(), dW.get())
+    result = {
+        'metric': 'conv2D fwd+bwd fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
+        'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True,
+        'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': f'{name}: x{list(xs)} w{list(ws)} stride {s} dilation {d} padding {padding!r}, '
+                               'step = fwd + dX(+=) + dW(+=)'},
+        'images_per_s': N / wall_ms * 1e3,
+        'frac_mfma_peak_step': 3 * flops / wall_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS,
+        'roofline': roof, 'passes': per_pass,
+    }
+    if cpu:
+        from oracle import refpath
+        cores = refpath.num_threads()
+        ref = None
+        times = []
+        for i in range(cpu_steps + 1):
+            t0 = time.perf_counter()
+            ry = refpath.conv2d_fwd(x, w, s, d, padding)
+            rdx = refpath.conv2d_dx(dy, w, xs, s, d, padding)
+            rdw = refpath.conv2d_dw(x, dy, ws, s, d, padding)
+            if i > 0:
+                times.append(time.perf_counter() - t0)
+            ref = (ry, rdx, rdw)
+        cpu_s = float(np.median(times))
+        result['cpu_baseline'] = {
+            'value': 3 * flops / cpu_s / 1e12, 'unit': 'TFLOP/s', 'cores': cores, 'kind': 'port',
+            'ms_per_step': cpu_s * 1e3,
+            'sample': f'the full {name} step (fwd + dX + dW), median of {cpu_steps} after 1 warm-up, '
+                      'C restatement of unfold -> register-tiled GeMM -> transpose incl. zero fills, OpenMP'}
+        result['parity'] = {'checked_against': 'cpu_baseline outputs (fp32 reference data flow)',
+                            'max_rel_err': max(rel_err(g, r) for g, r in zip(got, ref)), 'tolerance': 1e-4}
+    for a in (X, W, dY, Y, dX, dW):
+        a.free()
+    return result
+
+
+def bench_matmul(api, steps, warmup, n=4096, cpu=True):
+    rs = np.random.RandomState(0)
+    a, b, dc = (rs.normal(0, 1, (n, n)).astype(np.float32) for _ in range(3))
+    A, B, dC = Dev(api, a), Dev(api, b), Dev(api, dc)
+    C, dA, dB = Dev(api, shape=(n, n)), Dev(api, shape=(n, n)), Dev(api, shape=(n, n))
+    flops = 2.0 * n * n * n
+    passes = {
+        'fwd': lambda: api.gemm(0, 0, 0, 1, n, n, n, A.ptr, n, 0, B.ptr, n, 0, C.ptr, n, 0, 0),
+        'dA': lambda: api.gemm(0, 0, 1, 1, n, n, n, dC.ptr, n, 0, B.ptr, n, 0, dA.ptr, n, 0, 1),
+        'dB': lambda: api.gemm(0, 1, 0, 1, n, n, n, A.ptr, n, 0, dC.ptr, n, 0, dB.ptr, n, 0, 1),
+    }
+
+    def step():
+        for fn in passes.values():
+            fn()
+
+    for _ in range(warmup):
+        step()
+    api.synchronize(0)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    api.synchronize(0)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    per_pass = {}
+    for k, fn in passes.items():
+        ms = time_events(api, fn, max(steps, 5))
+        per_pass[k] = {'ms': ms, 'tflops': flops / ms / 1e9, 'frac_mfma': flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS}
+    dom = max(per_pass, key=lambda k: per_pass[k]['ms'])
+    dA.zero()
+    dB.zero()
+    step()
+    res = {'metric': 'matmul fwd+dA+dB fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
+           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True,
+           'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+           'config': {'workload': f'cfg2_matmul: [{n}x{n}] @ [{n}x{n}], step = C + dA(+=) + dB(+=)'},
+           'roofline': {'bound': 'mfma', 'kernel': dom, 'achieved': per_pass[dom]['tflops'],
+                        'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s', 'frac': per_pass[dom]['frac_mfma'],
+                        'traffic': None},
+           'passes': per_pass}
+    if cpu:
+        from oracle import refpath
+        m = 1024   # bounded sample: the reference GeMM at 1024^3 (1/64 of the flops)
+        t0 = time.perf_counter()
+        refpath.matmul(a[:m, :m].copy(), b[:m, :m].copy())
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': 2.0 * m ** 3 / dt / 1e12, 'unit': 'TFLOP/s', 'cores': refpath.num_threads(),
+                               'kind': 'port', 'sample': f'forward GeMM only at {m}^3, one run'}
+        # parity of the full-size result on a row sample against fp64
+        rows = np.arange(0, n, 257)
+        c = C.get()
+        res['parity'] = {'checked_against': 'fp64 numpy on every 257th row of C',
+                         'max_rel_err': rel_err(c[rows], a[rows].astype(np.float64) @ b.astype(np.float64)),
+                         'tolerance': 1e-4}
+    for t in (A, B, dC, C, dA, dB):
+        t.free()
+    return res
+
+
+def bench_encoder(steps, warmup):
+    """cfg5: full training step (forward, backward, SGD) of the 4-layer 5x5
+    stride-2 encoder through the litenn-compatible Python API."""
+    import litenn_amd as nn
+    rs = np.random.RandomState(0)
+    x_n = rs.uniform(-1, 1, (16, 3, 128, 128)).astype(np.float32)
+    chans = [3, 64, 128, 256, 512]
+    layers = []
+    for i in range(4):
+        w = rs.normal(0, np.sqrt(2.0 / (chans[i] * 25)), (chans[i + 1], chans[i], 5, 5)).astype(np.float32)
+        layers.append(nn.Conv2D(chans[i], chans[i + 1], 5, stride=2, padding=2,
+                                kernel_initializer=nn.initializer.NumpyArray(w)))
+
+    class Enc(nn.Module):
+        def __init__(self):
+            self.convs = layers
+
+        def forward(self, x):
+            for i, c in enumerate(self.convs):
+                x = c(x)
+                if i < 3:
+                    x = nn.leaky_relu(x, 0.1)
+            return x
+
+    enc = Enc()
+    opt = nn.optimizer.SGD(enc.trainables(), lr=1e-3)
+    x_t = nn.Tensor_from_value(x_n)
+
+    def step():
+        opt.zero_grad()
+        loss = nn.square(enc(x_t)).mean()
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(warmup):
+        step()
+    nn.devices.wait()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = step()
+    nn.devices.wait()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    flops = 61.66e9
+    res = {'metric': 'encoder training step images/s', 'value': 16 / wall_ms * 1e3, 'unit': 'images/s', 'n_gpus': 1,
+           'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True, 'scaling': 'weak',
+           'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+           'config': {'workload': 'cfg5_encoder: 16x3x128x128, 3->64->128->256->512, 5x5 s2 p2, leaky_relu(0.1), '
+                                  'loss mean(square), SGD lr 1e-3; forward + backward + update'},
+           'conv_tflops': flops / wall_ms / 1e9, 'final_loss': float(loss.np()[0])}
+    del loss, x_t, opt, enc, layers
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--all', action='store_true', help='also measure every benchmark configuration')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)')
+    from litenn_amd.core.hip import api
+    if api.device_count() < 1:
+        sys.exit('bench.py needs an MI355X: no HIP device is visible')
+    if args.all:
+        os.makedirs(os.path.join(ROOT, 'gpurun_out'), exist_ok=True)
+        with open(os.path.join(ROOT, 'gpurun_out', 'bench_all.jsonl'), 'w') as f:
+            for name in CONV_CONFIGS:
+                if name == 'cfg3_vgg3x3':
+                    continue
+                r = bench_conv(api, name, args.steps, args.warmup, cpu=not args.no_cpu, cpu_steps=1)
+                f.write(json.dumps(r) + '\n')
+                f.flush()
+                print(f'[bench] {name}: {r["value"]:.1f} TFLOP/s step, passes '
+                      + ', '.join(f'{k} {v["ms"]:.3f} ms' for k, v in r['passes'].items()), file=sys.stderr, flush=True)
+            r = bench_matmul(api, args.steps, args.warmup, cpu=not args.no_cpu)
+            f.write(json.dumps(r) + '\n')
+            print(f'[bench] cfg2 matmul: {r["value"]:.1f} TFLOP/s', file=sys.stderr, flush=True)
+            r = bench_encoder(args.steps, args.warmup)
+            f.write(json.dumps(r) + '\n')
+            print(f'[bench] cfg5 encoder: {r["value"]:.0f} images/s, {r["ms_per_step"]:.3f} ms/step', file=sys.stderr,
+                  flush=True)
+    res = bench_conv(api, 'cfg3_vgg3x3', args.steps, args.warmup, cpu=not args.no_cpu)
+    if args.all:
+        with open(os.path.join(ROOT, 'gpurun_out', 'bench_all.jsonl'), 'a') as f:
+            f.write(json.dumps(res) + '\n')
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == '__main__':
+    main()
