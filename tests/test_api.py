@@ -1,0 +1,399 @@
+"""The litenn-compatible Python layer: the reference's own self-tests restated
+(conv2d_test conv2D.py:76-126, matmul_test matmul.py:167-234, transpose_test
+transpose.py:106-163, backward_test test.py:166-195, Conv2D_test / Dense_test,
+shallow_mode_test test.py:147-164, SGD_test test.py:265-270) plus behaviour the
+user guide documents.  Every test runs twice: on the numpy stand-in (host
+logic, no GPU) and - marked gpu - on the real library."""
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import conv2d_all, info_conv2d
+
+
+def test_conv2d_reference_style(nn_backend):
+    nn = nn_backend
+    rs = np.random.RandomState(0)
+    n_cases = 0
+    for padding, dilation, stride, ks in itertools.product(['same', 'valid', 0, 2], [1, 2], [1, 2, 3], [5, 3, 1]):
+        for n, ic, oc, hw in [(1, 1, 1, 8), (4, 2, 4, 8), (1, 4, 2, 16)]:
+            if padding == 'valid' and hw < ks:
+                continue
+            input_n = rs.randint(2 ** 4, size=(n, ic, hw, hw)).astype(np.float32)
+            kernel_n = rs.randint(2 ** 4, size=(oc, ic, ks, ks)).astype(np.float32)
+            input_t = nn.Tensor_from_value(input_n)
+            kernel_t = nn.Tensor_from_value(kernel_n)
+            conved_t = nn.conv2D(input_t, kernel_t, stride=stride, dilation=dilation, padding=padding)
+            grad_n = rs.randint(2 ** 4, size=tuple(conved_t.shape)).astype(np.float32)
+            y, dI, dK = conv2d_all(input_n, kernel_n, grad_n, stride, dilation, padding)
+            assert y.shape == conved_t.shape
+            assert np.array_equal(conved_t.np(), y)
+            input_t.get_grad().fill(1.0)
+            kernel_t.get_grad().fill(1.0)
+            nn.backward({conved_t: grad_n}, grad_for_non_trainables=True)
+            assert np.array_equal(input_t.get_grad().np() - 1.0, dI)
+            assert np.array_equal(kernel_t.get_grad().np() - 1.0, dK)
+            n_cases += 1
+    assert n_cases > 150
+
+
+def test_matmul_reference_style(nn_backend):
+    nn = nn_backend
+    rs = np.random.RandomState(1)
+    for _ in range(10):
+        BATCH, M = rs.randint(8) + 1, rs.randint(8) + 1
+        N, K = rs.randint(32768) + 1, rs.randint(32768) + 1
+        while K * N > (400000 // BATCH):
+            K, N = max(1, K // 2), max(1, N // 2)
+        if rs.randint(2) == 0:
+            size = [2, 4, 8, 16][rs.randint(4)]
+            M, N, K = (max(1, v // size) * size for v in (M, N, K))
+        A_shape, B_shape = ((M, K), (K, N)) if BATCH == 1 else ((BATCH, M, K), (BATCH, K, N))
+        A_n = rs.randint(2 ** 4, size=A_shape).astype(np.float32)
+        B_n = rs.randint(2 ** 4, size=B_shape).astype(np.float32)
+        O_n = np.matmul(A_n, B_n)
+        A_t, B_t = nn.Tensor_from_value(A_n), nn.Tensor_from_value(B_n)
+        O_t = nn.matmul(A_t, B_t)
+        assert O_n.shape == O_t.shape
+        assert np.array_equal(O_t.np(), O_n)
+        O_n_grad = rs.randint(2 ** 3, size=O_n.shape).astype(np.float32)
+        A_t.get_grad().fill(1.0)
+        B_t.get_grad().fill(1.0)
+        nn.backward({O_t: O_n_grad}, grad_for_non_trainables=True)
+        assert np.array_equal(A_t.get_grad().np() - 1.0, np.matmul(O_n_grad, np.swapaxes(B_n, -1, -2)))
+        assert np.array_equal(B_t.get_grad().np() - 1.0, np.matmul(np.swapaxes(A_n, -1, -2), O_n_grad))
+
+
+def test_matmul_and_conv_shape_errors(nn_backend):
+    nn = nn_backend
+    with pytest.raises(ValueError):
+        nn.matmul(nn.Tensor((2, 3)), nn.Tensor((1, 3, 4)))
+    with pytest.raises(ValueError):
+        nn.matmul(nn.Tensor((3,)), nn.Tensor((3,)))
+    with pytest.raises(ValueError):
+        nn.matmul(nn.Tensor((2, 3)), nn.Tensor((4, 5)))
+    with pytest.raises(ValueError):
+        nn.matmul(nn.Tensor((2, 2, 3)), nn.Tensor((3, 3, 4)))
+    with pytest.raises(ValueError):
+        nn.conv2D(nn.Tensor((1, 3, 4, 4)), nn.Tensor((2, 4, 3, 3)))
+    with pytest.raises(ValueError):
+        nn.conv2D(nn.Tensor((1, 3, 4, 4)), nn.Tensor((2, 3, 3, 3)), padding='full')
+    with pytest.raises(ValueError):
+        nn.conv2D(nn.Tensor((1, 3, 4, 4)), nn.Tensor((2, 3, 3, 3)), padding=(1, 2, 3))
+
+
+def test_output_t_and_is_add_to_output(nn_backend):
+    nn = nn_backend
+    import litenn_amd.core as nc
+    rs = np.random.RandomState(2)
+    a = rs.randint(8, size=(6, 5)).astype(np.float32)
+    b = rs.randint(8, size=(5, 7)).astype(np.float32)
+    a_t, b_t = nn.Tensor_from_value(a), nn.Tensor_from_value(b)
+    out = nn.Tensor((42,), init=nn.initializer.Scalar(3.0))          # any shape of equal size
+    r = nc.op.matmul(a_t, b_t, output_t=out, is_add_to_output=True)
+    assert r is out and not out._is_produced_by_op()
+    assert np.array_equal(out.np().reshape(6, 7), a @ b + 3.0)
+    nc.op.matmul(a_t, b_t, output_t=out)                             # overwrite
+    assert np.array_equal(out.np().reshape(6, 7), a @ b)
+    with pytest.raises(ValueError):
+        nc.op.matmul(a_t, b_t, output_t=nn.Tensor((41,)))
+    t = nn.Tensor((7, 6), init=nn.initializer.Scalar(1.0))
+    nc.op.transpose(nn.Tensor_from_value(a @ b), (1, 0), output_t=t, is_add_to_output=True)
+    assert np.array_equal(t.np(), (a @ b).T + 1.0)
+
+
+def test_transpose_reference_style(nn_backend):
+    nn = nn_backend
+    rs = np.random.RandomState(3)
+    for _ in range(5):
+        for rank in range(2, 5):
+            shape = rs.randint(8, size=(rank,)) + 1
+            axes = rs.permutation(rank)
+            val_n = rs.randint(2 ** 8, size=shape).astype(np.float32)
+            val_t = nn.Tensor_from_value(val_n)
+            tr_t = nn.transpose(val_t, axes)
+            assert np.array_equal(tr_t.np(), np.transpose(val_n, axes))
+            g = rs.randint(2 ** 8, size=tuple(tr_t.shape)).astype(np.float32)
+            val_t.get_grad().fill(1.0)
+            nn.backward({tr_t: g}, grad_for_non_trainables=True)
+            assert np.array_equal(np.transpose(val_t.get_grad().np() - 1.0, axes), g)
+    for size in (2, 3):
+        v = rs.randint(2 ** 8, size=(2, 2 * size * size, 3 * size, 3 * size)).astype(np.float32)
+        v_t = nn.Tensor_from_value(v)
+        assert np.array_equal(nn.space_to_depth(nn.depth_to_space(v_t, size), size).np(), v)
+
+
+def test_reshape_is_a_view(nn_backend):
+    nn = nn_backend
+    v = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    t = nn.Tensor_from_value(v)
+    r = t.reshape((4, -1))
+    assert r._is_reference() and r.shape == (4, 6)
+    assert np.array_equal(r.np(), v.reshape(4, 6))
+    r.set(np.ones((4, 6)))
+    assert np.array_equal(t.np(), np.ones((2, 3, 4)))                 # same storage
+    assert nn.flatten(t).shape == (2, 12)
+    with pytest.raises(ValueError):
+        t.reshape((5, -1))
+    g = r.get_grad()
+    assert t.has_grad() and g.shape == (4, 6)
+
+
+def test_backward_freeze_and_optimizer(nn_backend):
+    nn = nn_backend
+    inp_t = nn.Tensor((2, 2, 8, 8), init=nn.initializer.Scalar(1.0))
+    kernel_t = nn.Tensor((4, 2, 3, 3), init=nn.initializer.Scalar(0.0))
+    kernel_2_t = nn.Tensor((4, 2, 3, 3), init=nn.initializer.Scalar(0.0))
+    opt = nn.optimizer.SGD([inp_t, kernel_t, kernel_2_t])
+    opt.zero_grad()
+    with nn.optimizer.freeze():
+        r = nn.conv2D(inp_t, kernel_2_t)
+    r.backward()
+    assert not kernel_2_t.has_grad()
+    r = nn.conv2D(inp_t, kernel_t)
+    r.backward()
+    assert kernel_t.has_grad()
+    assert not np.all(kernel_t.get_grad().np() == 0)
+    opt.step()
+    assert not np.all(kernel_t.np() == 0)
+    assert opt.get_iteration() == 1
+
+
+def test_non_trainable_gradients_are_dropped(nn_backend):
+    nn = nn_backend
+    x = nn.Tensor_from_value(np.ones((1, 2, 4, 4), np.float32))
+    w = nn.Tensor_from_value(np.ones((3, 2, 3, 3), np.float32))
+    y = nn.leaky_relu(nn.conv2D(x, w))
+    y.backward()                                   # nothing is attached to an optimizer
+    assert not x.has_grad() and not w.has_grad() and not y.has_grad()
+    y.backward(grad_for_non_trainables=True)
+    assert x.has_grad() and w.has_grad() and y.has_grad()
+    x.free_grad(); w.free_grad()
+    opt = nn.optimizer.SGD([w])
+    y2 = nn.leaky_relu(nn.conv2D(x, w))
+    y2.backward()
+    assert w.has_grad() and not x.has_grad() and not y2.has_grad()   # only the trainable keeps its grad
+    w.zero_grad()
+    y3 = nn.conv2D(x, w)
+    y3.backward(stop_grad=[y3])
+    assert not w.has_grad()
+    del opt
+
+
+def test_conv2d_and_dense_modules(nn_backend):
+    nn = nn_backend
+    module = nn.Conv2D(4, 8, 3)
+    x = nn.Tensor((2, 4, 8, 8))
+    y = module(x)
+    y.backward(grad_for_non_trainables=True)
+    assert x.has_grad() and y.shape == (2, 8, 8, 8)
+    assert [t.get_name() for t in module.trainables()] == ['Conv2D.kernel', 'Conv2D.bias']
+    dense = nn.Dense(4, 8)
+    x2 = nn.Tensor((2, 4))
+    y2 = dense(x2)
+    y2.backward(grad_for_non_trainables=True)
+    assert x2.has_grad() and y2.shape == (2, 8)
+    # numeric check with a bias
+    rs = np.random.RandomState(4)
+    k = rs.randint(4, size=(5, 3, 3, 3)).astype(np.float32)
+    b = rs.randint(4, size=(5,)).astype(np.float32)
+    conv = nn.Conv2D(3, 5, 3, stride=2, kernel_initializer=nn.initializer.NumpyArray(k),
+                     bias_initializer=nn.initializer.NumpyArray(b))
+    xv = rs.randint(4, size=(2, 3, 9, 9)).astype(np.float32)
+    out = conv(nn.Tensor_from_value(xv))
+    ci = info_conv2d(9, 9, 3, 3, 2, 1, 'same')
+    gy = rs.randint(4, size=(2, 5, ci.OH, ci.OW)).astype(np.float32)
+    ry, rdx, rdw = conv2d_all(xv, k, gy, 2, 1, 'same')
+    assert np.array_equal(out.np(), ry + b.reshape(1, 5, 1, 1))
+    nn.backward({out: gy}, grad_for_non_trainables=True)
+    assert np.array_equal(conv.kernel.get_grad().np(), rdw)
+    assert np.array_equal(conv.bias.get_grad().np(), gy.sum((0, 2, 3)))
+
+
+def test_shallow_mode_allocates_nothing(nn_backend):
+    nn = nn_backend
+
+    class M(nn.Module):
+        def __init__(self):
+            self.conv = nn.Conv2D(1, 1, 3, stride=2)
+
+        def forward(self, x):
+            return self.conv(x)
+
+    m = M()
+    m.set_training(True)
+    out = m.shallow_forward(nn.Tensor((1, 1, 16, 16)))
+    assert out.shape == (1, 1, 8, 8)
+    assert nn.devices.get_current()[0].get_used_memory() == 0
+    assert m.is_training() and m.conv.is_training()
+
+
+def test_sgd_closed_form(nn_backend):
+    nn = nn_backend
+    for momentum, nesterov, decay in [(0.0, False, 0.0), (0.9, False, 0.0), (0.9, True, 0.1)]:
+        w0 = np.linspace(-1, 1, 16).astype(np.float32)
+        g = np.linspace(1, 2, 16).astype(np.float32)
+        w_t = nn.Tensor_from_value(w0)
+        opt = nn.optimizer.SGD([w_t], momentum=momentum, nesterov=nesterov, lr=0.01, lr_decay=decay)
+        w, acc = w0.astype(np.float64), np.zeros(16)
+        for it in range(3):
+            w_t.get_grad().set(g)
+            opt.step()
+            lr = 0.01 / (1.0 + decay * it)
+            acc = momentum * acc - lr * g
+            w = w + (momentum * acc - lr * g if nesterov else acc)
+        np.testing.assert_allclose(w_t.np(), w, rtol=1e-5, atol=1e-6)
+        w_t._set_trainable(False)
+    with pytest.raises(NotImplementedError):
+        nn.optimizer.SGD([nn.Tensor((4,))], lr_dropout=0.7)
+
+
+def test_pointwise_broadcast_and_reduce(nn_backend):
+    nn = nn_backend
+    rs = np.random.RandomState(5)
+    a = rs.randint(-8, 8, size=(2, 3, 4, 5)).astype(np.float32)
+    b = rs.randint(-8, 8, size=(1, 3, 1, 1)).astype(np.float32)
+    a_t, b_t = nn.Tensor_from_value(a), nn.Tensor_from_value(b)
+    s = a_t + b_t
+    assert np.array_equal(s.np(), a + b)
+    m = a_t * b_t
+    assert np.array_equal(m.np(), a * b)
+    d = a_t - b_t
+    g = rs.randint(-4, 4, size=(2, 3, 4, 5)).astype(np.float32)
+    nn.backward({s: g, m: g, d: g}, grad_for_non_trainables=True)
+    assert np.array_equal(a_t.get_grad().np(), g + g * b + g)
+    assert np.array_equal(b_t.get_grad().np(), (g + g * a - g).sum((0, 2, 3), keepdims=True))
+    a_t.free_grad()
+    lr = nn.leaky_relu(a_t, 0.5)
+    assert np.array_equal(lr.np(), np.where(a >= 0, a, 0.5 * a))
+    sq = nn.square(a_t)
+    mean = sq.mean()
+    assert mean.shape == (1,)
+    np.testing.assert_allclose(mean.np()[0], (a * a).mean(), rtol=1e-6)
+    nn.backward([mean], grad_for_non_trainables=True)
+    np.testing.assert_allclose(a_t.get_grad().np(), 2 * a / a.size, rtol=1e-6)
+    r = nn.reduce_sum(a_t, axes=(1, -1), keepdims=True)
+    assert r.shape == (2, 1, 4, 1) and np.array_equal(r.np(), a.sum((1, 3), keepdims=True))
+    r2 = a_t.sum(axes=0)
+    assert r2.shape == (3, 4, 5) and np.array_equal(r2.np(), a.sum(0))
+    assert np.array_equal((a_t + 2).np(), a + 2) and np.array_equal((3 * a_t).np(), 3 * a)
+    assert np.array_equal((a_t + a_t).np(), 2 * a) and np.array_equal((-a_t).np(), -a)
+
+
+def test_buffer_pool_and_lifetime_guards(nn_backend):
+    nn = nn_backend
+    dev = nn.devices.get_current()[0]
+    t = nn.Tensor((256,))
+    assert dev.get_used_memory() == 0                       # allocation is lazy
+    t.np()
+    assert dev.get_used_memory() == 1024
+    del t
+    assert dev.get_used_memory() == 0 and dev.get_total_pooled_memory() == 1024
+    t2 = nn.Tensor((256,), init=nn.initializer.Scalar(2.0))
+    assert np.array_equal(t2.np(), np.full(256, 2.0, np.float32))     # pooled block is re-initialised
+    assert dev.get_total_allocated_memory() == 1024
+    with pytest.raises(Exception):
+        nn.cleanup()                                         # a Tensor is alive
+    with pytest.raises(Exception):
+        nn.devices.set_current(dev)
+    del t2
+    nn.cleanup()
+    assert dev.get_total_allocated_memory() == 0
+
+
+def test_module_names_save_and_load(nn_backend, tmp_path):
+    nn = nn_backend
+
+    class Net(nn.Module):
+        def __init__(self):
+            self.blocks = [nn.Conv2D(2, 2, 3), nn.Conv2D(2, 2, 1, use_bias=False)]
+            self.head = nn.Dense(8, 3)
+            self.note = 'v1'
+
+        def forward(self, x):
+            for b in self.blocks:
+                x = b(x)
+            return self.head(nn.flatten(x))
+
+    net = Net()
+    names = [t.get_name() for t in net.trainables()]
+    assert names == ['Net.blocks[0].kernel', 'Net.blocks[0].bias', 'Net.blocks[1].kernel', 'Net.head.weight',
+                     'Net.head.bias']
+    assert net(nn.Tensor((1, 2, 2, 2))).shape == (1, 3)
+    opt = nn.optimizer.SGD(net.trainables(), momentum=0.5)
+    before = net.blocks[0].kernel.np().copy()
+    path = tmp_path / 'net.bin'
+    net.save(path)
+    net.blocks[0].kernel.fill(7.0)
+    net.note = 'changed'
+    assert net.load(path) is True
+    assert np.array_equal(net.blocks[0].kernel.np(), before) and net.note == 'v1'
+    assert net.load(tmp_path / 'missing.bin') is False
+    opt.iteration = 5
+    opt.save(tmp_path / 'opt.bin')
+    opt.iteration = 0
+    opt.load(tmp_path / 'opt.bin')
+    assert opt.iteration == 5
+    with pytest.raises(ValueError):
+        nn.optimizer.SGD(net.trainables())                  # already attached
+
+
+def test_training_step_matches_numpy(nn_backend):
+    """Two-layer version of the encoder benchmark: conv(5x5, s2, p2) + bias ->
+    leaky_relu(0.1) -> conv -> mean(square); SGD.  Compared with a float64
+    restatement built from the oracle."""
+    nn = nn_backend
+    rs = np.random.RandomState(0)
+    x = rs.uniform(-1, 1, (4, 3, 16, 16)).astype(np.float32)
+    w1 = rs.normal(0, np.sqrt(2 / 75), (8, 3, 5, 5)).astype(np.float32)
+    w2 = rs.normal(0, np.sqrt(2 / 200), (16, 8, 5, 5)).astype(np.float32)
+    c1 = nn.Conv2D(3, 8, 5, stride=2, padding=2, kernel_initializer=nn.initializer.NumpyArray(w1))
+    c2 = nn.Conv2D(8, 16, 5, stride=2, padding=2, kernel_initializer=nn.initializer.NumpyArray(w2))
+
+    class A(nn.Module):
+        def __init__(self): self.c1 = c1
+    class B(nn.Module):
+        def __init__(self): self.c2 = c2
+    ma, mb = A(), B()
+    opt = nn.optimizer.SGD(ma.trainables() + mb.trainables(), lr=1e-2)
+    x_t = nn.Tensor_from_value(x)
+    losses = []
+    W1, W2 = w1.astype(np.float64), w2.astype(np.float64)
+    B1, B2 = np.zeros(8), np.zeros(16)
+    from oracle import conv2d_fwd, conv2d_dx, conv2d_dw
+    for _ in range(2):
+        opt.zero_grad()
+        loss = nn.square(c2(nn.leaky_relu(c1(x_t), 0.1))).mean()
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.np()[0]))
+        # float64 restatement
+        z1 = conv2d_fwd(x, W1, 2, 1, 2) + B1.reshape(1, -1, 1, 1)
+        a1 = np.where(z1 >= 0, z1, 0.1 * z1)
+        z2 = conv2d_fwd(a1, W2, 2, 1, 2) + B2.reshape(1, -1, 1, 1)
+        ref_loss = (z2 * z2).mean()
+        dz2 = 2 * z2 / z2.size
+        dW2, dB2 = conv2d_dw(a1, dz2, W2.shape, 2, 1, 2), dz2.sum((0, 2, 3))
+        da1 = conv2d_dx(dz2, W2, a1.shape, 2, 1, 2)
+        dz1 = da1 * np.where(z1 >= 0, 1.0, 0.1)
+        dW1, dB1 = conv2d_dw(x, dz1, W1.shape, 2, 1, 2), dz1.sum((0, 2, 3))
+        W1, W2, B1, B2 = W1 - 1e-2 * dW1, W2 - 1e-2 * dW2, B1 - 1e-2 * dB1, B2 - 1e-2 * dB2
+        assert abs(losses[-1] - ref_loss) <= 1e-4 * abs(ref_loss)
+    assert np.abs(c1.kernel.np() - W1).max() <= 1e-4 * np.abs(W1).max()
+    assert np.abs(c2.kernel.np() - W2).max() <= 1e-4 * np.abs(W2).max()
+    assert np.abs(c2.bias.np() - B2).max() <= 1e-4 * max(np.abs(B2).max(), 1e-3)
+    assert not x_t.has_grad()                          # the input is not trainable: its dX is skipped
+
+
+def test_unfold2d_operator(nn_backend):
+    nn = nn_backend
+    import litenn_amd.core as nc
+    from oracle import unfold_index_map, apply_index_map
+    x = np.arange(1, 2 * 3 * 6 * 6 + 1, dtype=np.float32).reshape(2, 3, 6, 6)
+    ci = info_conv2d(6, 6, 3, 3, 2, 1, 'same')
+    t = nc.op.unfold2D(nn.Tensor_from_value(x), 2, 3, 6, 6, ci.OH, ci.OW, 3, 3, ci.PADL, ci.PADT, 1, 2, 'CJI_NHW', False)
+    shape, m = unfold_index_map(2, 3, 6, 6, ci.OH, ci.OW, 3, 3, ci.PADL, ci.PADT, 1, 2, 'CJI_NHW')
+    assert t.shape == shape and np.array_equal(t.np(), apply_index_map(x, shape, m))
+    with pytest.raises(ValueError):
+        nc.op.unfold2D(nn.Tensor_from_value(x), 2, 3, 6, 6, 3, 3, 3, 3, 1, 1, 1, 2, 'N_C_H_W_JI', False)
