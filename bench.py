@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the conv2D / matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all] [--config NAME]
 
 Default workload (the configuration the headline metric is quoted on): the
 VGG-style 3x3 convolution layer, fp32 NCHW, N=32, C=128, H=W=56, O=128,
@@ -303,6 +303,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--all', action='store_true', help='also measure every benchmark configuration')
+    ap.add_argument('--config', default='cfg3_vgg3x3', choices=list(CONV_CONFIGS) + ['cfg2_matmul', 'cfg5_encoder'],
+                    help='workload of the JSON line (default: the headline configuration)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)')
@@ -327,7 +329,12 @@ def main():
             f.write(json.dumps(r) + '\n')
             print(f'[bench] cfg5 encoder: {r["value"]:.0f} images/s, {r["ms_per_step"]:.3f} ms/step', file=sys.stderr,
                   flush=True)
-    res = bench_conv(api, 'cfg3_vgg3x3', args.steps, args.warmup, cpu=not args.no_cpu)
+    if args.config == 'cfg2_matmul':
+        res = bench_matmul(api, args.steps, args.warmup, cpu=not args.no_cpu)
+    elif args.config == 'cfg5_encoder':
+        res = bench_encoder(args.steps, args.warmup)
+    else:
+        res = bench_conv(api, args.config, args.steps, args.warmup, cpu=not args.no_cpu)
     if args.all:
         with open(os.path.join(ROOT, 'gpurun_out', 'bench_all.jsonl'), 'a') as f:
             f.write(json.dumps(res) + '\n')

@@ -55,7 +55,24 @@ __global__ void reduce_partials(float* out, const float* part, int n, int slices
   out[i] = s;
 }
 
-enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2 };
+// *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
+enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4 };
+
+// Wp[a][tap][b] = W[..] so that the tap-major K index tap*CH + ch is contiguous:
+//   mode 0 (forward): Wp[o][tap][c] = W[o][c][tap]
+//   mode 1 (dgrad):   Wp[c][tap][o] = W[o][c][tap]
+__global__ void permute_weights(float* wp, const float* w, int O, int C, int KK, int mode) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= O * C * KK) return;
+  int a, tap, b;
+  if (mode == 0) {
+    b = i % C; tap = (i / C) % KK; a = i / (C * KK);
+    wp[i] = w[((size_t)a * C + b) * KK + tap];
+  } else {
+    b = i % O; tap = (i / O) % KK; a = i / (O * KK);
+    wp[i] = w[((size_t)b * C + a) * KK + tap];
+  }
+}
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
 struct ConvCfg {
@@ -77,14 +94,28 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, rsrc_t rx, rsrc_t r
     PlainKC<BM, FLAG> la;            // FLAG: 128-bit loads of W rows (CKK % 4 == 0)
     ConvFwdB<BN> lb;
     la.init(rw, p.K, m0, p.M, p.K);
-    lb.init(rx, p.g, p.tab, n0, p.Ncols);
+    lb.init(rx, p.g, p.tab, n0, p.Ncols, kbeg);
     om.nchw = 1; om.ld = p.g.OHW; om.mtot = p.g.O; om.dHW = p.g.dOHW;
+    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
+  } else if constexpr (PASS == PASS_FWD_TAP) {
+    PlainKC<BM, true> la;            // permuted weights [O][KK*C]
+    ConvFwdBTap<BN> lb;
+    la.init(rw, p.K, m0, p.M, p.K);
+    lb.init(rx, p.g, n0, p.Ncols, kbeg);
+    om.nchw = 1; om.ld = p.g.OHW; om.mtot = p.g.O; om.dHW = p.g.dOHW;
+    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
+  } else if constexpr (PASS == PASS_DGRAD_TAP) {
+    PlainKC<BM, true> la;            // permuted weights [C][KK*O]
+    ConvDgradBTap<BN, FLAG> lb;      // FLAG: stride == 1
+    la.init(rw, p.K, m0, p.M, p.K);
+    lb.init(rx, p.g, n0, p.Ncols, kbeg);
+    om.nchw = 1; om.ld = p.g.IHW; om.mtot = p.g.C; om.dHW = p.g.dIHW;
     run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
   } else if constexpr (PASS == PASS_DGRAD) {
     ConvDgradA<BM> la;
     ConvDgradB<BN, FLAG> lb;         // FLAG: stride == 1
-    la.init(rw, p.g, p.tab, m0);
-    lb.init(rx, p.g, p.tab, n0, p.Ncols);
+    la.init(rw, p.g, p.tab, m0, kbeg);
+    lb.init(rx, p.g, p.tab, n0, p.Ncols, kbeg);
     om.nchw = 1; om.ld = p.g.IHW; om.mtot = p.g.C; om.dHW = p.g.dIHW;
     run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
   } else {
@@ -100,7 +131,8 @@ __device__ __forceinline__ void conv_tile(const ConvArgs& p, rsrc_t rx, rsrc_t r
 template <int PASS, int WM, int NTMAX, bool FLAG>
 __global__ __launch_bounds__(256, 2) void conv_kernel(ConvArgs p) {
   using Cfg = ConvCfg<PASS, WM, NTMAX, FLAG>;
-  __shared__ __attribute__((aligned(16))) float lds[2 * (Cfg::SA + Cfg::SB)];
+  // at least 56 KB so that exactly two workgroups share a compute unit's 160 KB of LDS
+  __shared__ __attribute__((aligned(16))) float lds[(2 * (Cfg::SA + Cfg::SB) > 14336) ? 2 * (Cfg::SA + Cfg::SB) : 14336];
   const rsrc_t rx = make_rsrc(p.X, p.bytesX);
   const rsrc_t rw = make_rsrc(p.W, p.bytesW);
   int kbeg = 0, kend = p.K;
@@ -186,6 +218,19 @@ static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const KEntry**
   return LNN_OK;
 }
 
+// Channel-permuted copy of the weights in the library's scratch buffer (valid
+// until the next call that uses scratch; the stream orders it before its reader).
+static int permuted_weights(DeviceCtx* ctx, const ConvGeom& g, const float* W, int mode, const float** out) {
+  const int n = g.O * g.C * g.KK;
+  int st = ensure_workspace(ctx, (size_t)n * sizeof(float));
+  if (st != LNN_OK) return st;
+  hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, static_cast<float*>(ctx->ws), W,
+                     g.O, g.C, g.KK, mode);
+  LNN_HIP(hipGetLastError());
+  *out = static_cast<const float*>(ctx->ws);
+  return LNN_OK;
+}
+
 template <int PASS, int WM, int NTMAX>
 static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   constexpr int WN = 4 / WM, BM = 32 * WM;
@@ -247,8 +292,7 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !W || !Y) return set_error(LNN_ERR_INVALID, "conv2d_fwd: null pointer");
-  st = get_table(ctx, a.g, 0, &a.tab);
-  if (st != LNN_OK) return st;
+  a.tab = nullptr;
   const ConvGeom& g = a.g;
   a.X = X; a.W = W; a.Out = Y;
   a.bytesX = (uint32_t)((uint64_t)g.N * g.C * g.IHW * 4);
@@ -256,6 +300,13 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   a.bytesOut = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
   a.M = g.O; a.Ncols = g.N * g.OHW; a.K = g.C * g.KK;
   a.beta = beta ? 1 : 0;
+  if (g.C % BK == 0) {
+    st = permuted_weights(ctx, g, W, 0, &a.W);
+    if (st != LNN_OK) return st;
+    return launch_by_m<PASS_FWD_TAP>(ctx, a, true);
+  }
+  st = get_table(ctx, a.g, 0, &a.tab);
+  if (st != LNN_OK) return st;
   return launch_by_m<PASS_FWD>(ctx, a, a.K % 4 == 0 && aligned16(W));
 }
 
@@ -264,8 +315,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!dY || !W || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
-  st = get_table(ctx, a.g, 1, &a.tab);
-  if (st != LNN_OK) return st;
+  a.tab = nullptr;
   const ConvGeom& g = a.g;
   a.X = dY; a.W = W; a.Out = dX;
   a.bytesX = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
@@ -273,6 +323,13 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   a.bytesOut = (uint32_t)((uint64_t)g.N * g.C * g.IHW * 4);
   a.M = g.C; a.Ncols = g.N * g.IHW; a.K = g.O * g.KK;
   a.beta = beta ? 1 : 0;
+  if (g.O % BK == 0) {
+    st = permuted_weights(ctx, g, W, 1, &a.W);
+    if (st != LNN_OK) return st;
+    return launch_by_m<PASS_DGRAD_TAP>(ctx, a, g.S == 1);
+  }
+  st = get_table(ctx, a.g, 1, &a.tab);
+  if (st != LNN_OK) return st;
   return launch_by_m<PASS_DGRAD>(ctx, a, g.S == 1);
 }
 

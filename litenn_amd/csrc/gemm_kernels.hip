@@ -47,7 +47,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, rsrc_t ra, rsrc_t r
 template <int WM, int NTMAX, bool TA, bool TB, bool VEC>
 __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs p) {
   using Cfg = GemmCfg<WM, NTMAX, TA, TB, VEC>;
-  __shared__ __attribute__((aligned(16))) float lds[2 * (Cfg::SA + Cfg::SB)];
+  // at least 56 KB so that exactly two workgroups share a compute unit's 160 KB of LDS
+  __shared__ __attribute__((aligned(16))) float lds[(2 * (Cfg::SA + Cfg::SB) > 14336) ? 2 * (Cfg::SA + Cfg::SB) : 14336];
   const long long b = blockIdx.y;
   const rsrc_t ra = make_rsrc(p.A + b * p.sA, p.bytesA);
   const rsrc_t rb = make_rsrc(p.B + b * p.sB, p.bytesB);

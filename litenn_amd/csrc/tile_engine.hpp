@@ -178,6 +178,15 @@ struct ConvGeom {
 // w = 0x20000000 (byte offset 2 GiB: out of range).
 struct __attribute__((aligned(16))) KEntry { int x, y, z, w; };
 
+// The table is read through the constant address space with wave-uniform
+// indices so that entries arrive in scalar registers (s_load), one K step
+// ahead of their use: a loader's fetch(k0) consumes the entries fetched by the
+// previous call and requests those of k0 + BK.
+typedef const __attribute__((address_space(4))) KEntry* ktab_t;
+__device__ __forceinline__ ktab_t as_ktab(const KEntry* p) {
+  return reinterpret_cast<ktab_t>(reinterpret_cast<uintptr_t>(p));
+}
+
 // Forward im2col gather: element (pixel p, k) = X[n, c, oh*S-PT+kh*D, ow*S-PL+kw*D].
 // Each wavefront fetches 4 of the 16 k rows; lanes run over pixels so that
 // global reads follow the image rows and k stays wave-uniform.
@@ -186,13 +195,23 @@ struct ConvFwdB {
   static constexpr bool KC = false;
   static constexpr int CC = (R + 63) / 64;
   rsrc_t rs;
-  const KEntry* tab;
+  ktab_t tab;
   int IH, IW;
   int base[CC], ih0[CC], iw0[CC];
+  int tx[4], ty[4], tz[4];   // table entries of the next fetch (scalar registers)
   float v[4][CC];
-  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P) {
+  __device__ __forceinline__ void load_entries(int k0) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const ktab_t t = tab + (k0 + wave + 4 * e);
+      tx[e] = t->x; ty[e] = t->y; tz[e] = t->z;
+    }
+  }
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P, int kbeg) {
     rs = r;
-    tab = tab_;
+    tab = as_ktab(tab_);
+    load_entries(kbeg);
     IH = g.IH;
     IW = g.IW;
     const int lane = threadIdx.x & 63;
@@ -209,15 +228,160 @@ struct ConvFwdB {
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const KEntry t = tab[k0 + wave + 4 * e];
 #pragma unroll
       for (int c = 0; c < CC; ++c) {
-        const bool ok = (uint32_t)(ih0[c] + t.y) < (uint32_t)IH && (uint32_t)(iw0[c] + t.z) < (uint32_t)IW;
-        v[e][c] = buf_load(rs, ok ? (uint32_t)(base[c] + t.x) * 4u : OOB);
+        const bool ok = (uint32_t)(ih0[c] + ty[e]) < (uint32_t)IH && (uint32_t)(iw0[c] + tz[e]) < (uint32_t)IW;
+        v[e][c] = buf_load(rs, ok ? (uint32_t)(base[c] + tx[e]) * 4u : OOB);
       }
+    }
+    load_entries(k0 + BK);
+  }
+  __device__ __forceinline__ void commit(float* lds) const {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int c = 0; c < CC; ++c)
+        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * R + lane + 64 * c] = v[e][c];
+  }
+};
+
+// Tap-major variants of the two pixel gathers, for channel counts that are a
+// multiple of BK.  K is ordered k = tap*CH + ch (tap = kh*KW + kw), so one K
+// step is BK consecutive channels of a single tap: the pixel part of the
+// address and its range test depend on the tap only and live in a VGPR, the
+// channel part is wave-uniform and rides in the scalar offset of the buffer
+// instruction.  No table, no per-element arithmetic.  fetch() must be called
+// with consecutive K steps starting at the kbeg given to init().
+__device__ __forceinline__ float buf_load_s(rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0));
+}
+
+template <int R>
+struct ConvFwdBTap {
+  static constexpr bool KC = false;
+  static constexpr int CC = (R + 63) / 64;
+  rsrc_t rs;
+  int IH, IW, IHW, C, D, KW;
+  int base[CC], ih0[CC], iw0[CC];
+  int c0, kh, kw;   // K position of the next fetch
+  float v[4][CC];
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int p0, int P, int kbeg) {
+    rs = r;
+    IH = g.IH; IW = g.IW; IHW = g.IHW; C = g.C; D = g.D; KW = g.KW;
+    const int tap = kbeg / g.C;
+    c0 = kbeg - tap * g.C;
+    kh = tap / g.KW;
+    kw = tap - kh * g.KW;
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int c = 0; c < CC; ++c) {
+      const int col = lane + 64 * c, p = p0 + col;
+      const bool ok = col < R && p < P;
+      const uint32_t pp = ok ? (uint32_t)p : 0u;
+      const uint32_t img = g.dOHW.div(pp), rem = pp - img * g.OHW;
+      const uint32_t oh = g.dOW.div(rem), ow = rem - oh * g.OW;
+      ih0[c] = (int)oh * g.S - g.PADT;
+      iw0[c] = ok ? (int)ow * g.S - g.PADL : -BIG;
+      base[c] = ((int)img * g.C * g.IH + ih0[c]) * g.IW + ((int)ow * g.S - g.PADL);
+    }
+  }
+  __device__ __forceinline__ void fetch(int) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int dh = kh * D, dw = kw * D, tapoff = dh * IW + dw;
+    uint32_t voff[CC];
+#pragma unroll
+    for (int c = 0; c < CC; ++c) {
+      const bool ok = (uint32_t)(ih0[c] + dh) < (uint32_t)IH && (uint32_t)(iw0[c] + dw) < (uint32_t)IW;
+      voff[c] = ok ? (uint32_t)(base[c] + tapoff) * 4u : OOB;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t soff = (uint32_t)((c0 + wave + 4 * e) * IHW) * 4u;
+#pragma unroll
+      for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
+    }
+    c0 += BK;
+    if (c0 >= C) {
+      c0 = 0;
+      ++kw;
+      if (kw == KW) { kw = 0; ++kh; }
+    }
+  }
+  __device__ __forceinline__ void commit(float* lds) const {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int c = 0; c < CC; ++c)
+        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * R + lane + 64 * c] = v[e][c];
+  }
+};
+
+template <int R, bool STRIDE1>
+struct ConvDgradBTap {
+  static constexpr bool KC = false;
+  static constexpr int CC = (R + 63) / 64;
+  rsrc_t rs;
+  int OH, OW, OHW, O, S, D, KW;
+  FastDiv dS;
+  int base[CC], a0[CC], b0[CC];
+  int o0, kh, kw;
+  float v[4][CC];
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int p0, int P, int kbeg) {
+    rs = r;
+    OH = g.OH; OW = g.OW; OHW = g.OHW; O = g.O; S = g.S; D = g.D; KW = g.KW;
+    dS = g.dS;
+    const int tap = kbeg / g.O;
+    o0 = kbeg - tap * g.O;
+    kh = tap / g.KW;
+    kw = tap - kh * g.KW;
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int c = 0; c < CC; ++c) {
+      const int col = lane + 64 * c, p = p0 + col;
+      const bool ok = col < R && p < P;
+      const uint32_t pp = ok ? (uint32_t)p : 0u;
+      const uint32_t img = g.dIHW.div(pp), rem = pp - img * g.IHW;
+      const uint32_t ih = g.dIW.div(rem), iw = rem - ih * g.IW;
+      a0[c] = (int)ih + g.PADT;
+      b0[c] = ok ? (int)iw + g.PADL : -BIG;
+      base[c] = (int)img * g.O * g.OHW;
+    }
+  }
+  __device__ __forceinline__ void fetch(int) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int dh = kh * D, dw = kw * D;
+    uint32_t voff[CC];
+#pragma unroll
+    for (int c = 0; c < CC; ++c) {
+      const int nh = a0[c] - dh, nw = b0[c] - dw;
+      bool ok;
+      int oh, ow;
+      if (STRIDE1) {
+        oh = nh;
+        ow = nw;
+        ok = (uint32_t)nh < (uint32_t)OH && (uint32_t)nw < (uint32_t)OW;
+      } else {
+        oh = (int)dS.div((uint32_t)nh & 0x7fffffffu);
+        ow = (int)dS.div((uint32_t)nw & 0x7fffffffu);
+        ok = nh >= 0 && nw >= 0 && oh * S == nh && ow * S == nw && oh < OH && ow < OW;
+      }
+      voff[c] = ok ? (uint32_t)(base[c] + oh * OW + ow) * 4u : OOB;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t soff = (uint32_t)((o0 + wave + 4 * e) * OHW) * 4u;
+#pragma unroll
+      for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
+    }
+    o0 += BK;
+    if (o0 >= O) {
+      o0 = 0;
+      ++kw;
+      if (kw == KW) { kw = 0; ++kh; }
     }
   }
   __device__ __forceinline__ void commit(float* lds) const {
@@ -238,14 +402,24 @@ struct ConvDgradB {
   static constexpr bool KC = false;
   static constexpr int CC = (R + 63) / 64;
   rsrc_t rs;
-  const KEntry* tab;
+  ktab_t tab;
   int OH, OW, S;
   FastDiv dS;
   int base[CC], a0[CC], b0[CC];
+  int tx[4], ty[4], tz[4];
   float v[4][CC];
-  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P) {
+  __device__ __forceinline__ void load_entries(int k0) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const ktab_t t = tab + (k0 + wave + 4 * e);
+      tx[e] = t->x; ty[e] = t->y; tz[e] = t->z;
+    }
+  }
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P, int kbeg) {
     rs = r;
-    tab = tab_;
+    tab = as_ktab(tab_);
+    load_entries(kbeg);
     OH = g.OH;
     OW = g.OW;
     S = g.S;
@@ -264,13 +438,12 @@ struct ConvDgradB {
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const KEntry t = tab[k0 + wave + 4 * e];
+      const int t_x = tx[e];
 #pragma unroll
       for (int c = 0; c < CC; ++c) {
-        const int nh = a0[c] - t.y, nw = b0[c] - t.z;
+        const int nh = a0[c] - ty[e], nw = b0[c] - tz[e];
         bool ok;
         int oh, ow;
         if (STRIDE1) {
@@ -282,9 +455,10 @@ struct ConvDgradB {
           ow = (int)dS.div((uint32_t)nw & 0x7fffffffu);
           ok = nh >= 0 && nw >= 0 && oh * S == nh && ow * S == nw && oh < OH && ow < OW;
         }
-        v[e][c] = buf_load(rs, ok ? (uint32_t)(base[c] + t.x + oh * OW + ow) * 4u : OOB);
+        v[e][c] = buf_load(rs, ok ? (uint32_t)(base[c] + t_x + oh * OW + ow) * 4u : OOB);
       }
     }
+    load_entries(k0 + BK);
   }
   __device__ __forceinline__ void commit(float* lds) const {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -304,12 +478,19 @@ struct ConvDgradA {
   static constexpr bool KC = true;
   static constexpr int E = (R + 63) / 64;
   rsrc_t rs;
-  const KEntry* tab;
+  ktab_t tab;
   uint32_t cb[E];
+  uint32_t tw[4];
   f32x4 v[E];
-  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int c0) {
+  __device__ __forceinline__ void load_entries(int k0) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) tw[j] = (uint32_t)(tab + (k0 + 4 * wave + j))->w;
+  }
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int c0, int kbeg) {
     rs = r;
-    tab = tab_;
+    tab = as_ktab(tab_);
+    load_entries(kbeg);
     const int lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -318,10 +499,9 @@ struct ConvDgradA {
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t w = (uint32_t)tab[k0 + 4 * wave + j].w;
+      const uint32_t w = tw[j];
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         // either term alone is >= 2^29 elements (2 GiB) when invalid; clamp the sum
@@ -329,6 +509,7 @@ struct ConvDgradA {
         v[e][j] = buf_load(rs, idx >= 0x20000000u ? OOB : idx * 4u);
       }
     }
+    load_entries(k0 + BK);
   }
   __device__ __forceinline__ void commit(float* lds) const {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -474,35 +655,46 @@ struct OutMap {
 // t-th MFMA.  A and B use the same k assignment, so any k permutation cancels.
 // ---------------------------------------------------------------------------
 template <int NT, bool A_KC, bool B_KC, int RA, int RB>
-__device__ __forceinline__ void mma_stage(const float* __restrict__ As, const float* __restrict__ Bs,
-                                          f32x16 (&acc)[NT], int arow, int brow) {
+__device__ __forceinline__ void load_frags(const float* __restrict__ As, const float* __restrict__ Bs, int arow,
+                                           int brow, int kk, float (&a)[4], float (&b)[NT][4]) {
   const int lane = threadIdx.x & 63, i = lane & 31, h = lane >> 5;
+  const int kb = kk * 8 + h * 4;
+  if (A_KC) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(&As[(arow + i) * LDK + kb]);
+    a[0] = t[0]; a[1] = t[1]; a[2] = t[2]; a[3] = t[3];
+  } else {
 #pragma unroll
-  for (int kk = 0; kk < BK / 8; ++kk) {
-    const int kb = kk * 8 + h * 4;
-    float a[4], b[NT][4];
-    if (A_KC) {
-      const f32x4 t = *reinterpret_cast<const f32x4*>(&As[(arow + i) * LDK + kb]);
-      a[0] = t[0]; a[1] = t[1]; a[2] = t[2]; a[3] = t[3];
+    for (int t = 0; t < 4; ++t) a[t] = As[(kb + t) * RA + arow + i];
+  }
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    if (B_KC) {
+      const f32x4 t = *reinterpret_cast<const f32x4*>(&Bs[(brow + 32 * j + i) * LDK + kb]);
+      b[j][0] = t[0]; b[j][1] = t[1]; b[j][2] = t[2]; b[j][3] = t[3];
     } else {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) a[t] = As[(kb + t) * RA + arow + i];
+      for (int t = 0; t < 4; ++t) b[j][t] = Bs[(kb + t) * RB + brow + 32 * j + i];
     }
+  }
+}
+
+// One LDS stage = BK/8 groups of 4*NT MFMAs.  The fragments of group kk+1 are
+// read from LDS before the MFMAs of group kk are issued, so the LDS latency is
+// covered by a full group of matrix work instead of stalling every group.
+template <int NT, bool A_KC, bool B_KC, int RA, int RB>
+__device__ __forceinline__ void mma_stage(const float* __restrict__ As, const float* __restrict__ Bs,
+                                          f32x16 (&acc)[NT], int arow, int brow) {
+  float a[2][4], b[2][NT][4];
+  load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, 0, a[0], b[0]);
 #pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      if (B_KC) {
-        const f32x4 t = *reinterpret_cast<const f32x4*>(&Bs[(brow + 32 * j + i) * LDK + kb]);
-        b[j][0] = t[0]; b[j][1] = t[1]; b[j][2] = t[2]; b[j][3] = t[3];
-      } else {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) b[j][t] = Bs[(kb + t) * RB + brow + 32 * j + i];
-      }
-    }
+  for (int kk = 0; kk < BK / 8; ++kk) {
+    const int cur = kk & 1;
+    if (kk + 1 < BK / 8) load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, kk + 1, a[cur ^ 1], b[cur ^ 1]);
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int j = 0; j < NT; ++j)
-        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[j][t], acc[j], 0, 0, 0);
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][t], b[cur][j][t], acc[j], 0, 0, 0);
   }
 }
 
@@ -532,19 +724,24 @@ __device__ __forceinline__ void run_tile(LA& la, LB& lb, float* ldsA, float* lds
     lb.commit(ldsB);
   }
   __syncthreads();
-  for (int it = 0; it < nk; ++it) {
+  // Steady state: the global loads of K step it+1 are issued first, so that
+  // they (and their address arithmetic) share one scheduling region with the
+  // MFMAs of step it; the data is parked in LDS after the MFMAs.
+  for (int it = 0; it + 1 < nk; ++it) {
     const int cur = it & 1;
-    const bool more = it + 1 < nk;
-    if (more) {
-      la.fetch(kbeg + (it + 1) * BK);
-      lb.fetch(kbeg + (it + 1) * BK);
-    }
+    la.fetch(kbeg + (it + 1) * BK);
+    lb.fetch(kbeg + (it + 1) * BK);
+    __builtin_amdgcn_sched_barrier(0);   // keep the loads ahead of the matrix work
     mma_stage<NT, LA::KC, LB::KC, BM, BN>(ldsA + cur * strideA, ldsB + cur * strideB, acc, wm * 32, wn * NT * 32);
-    if (more) {
-      la.commit(ldsA + (cur ^ 1) * strideA);
-      lb.commit(ldsB + (cur ^ 1) * strideB);
-    }
+    __builtin_amdgcn_sched_barrier(0);
+    la.commit(ldsA + (cur ^ 1) * strideA);
+    lb.commit(ldsB + (cur ^ 1) * strideB);
     __syncthreads();
+  }
+  if (nk > 0) {
+    const int cur = (nk - 1) & 1;
+    mma_stage<NT, LA::KC, LB::KC, BM, BN>(ldsA + cur * strideA, ldsB + cur * strideB, acc, wm * 32, wn * NT * 32);
+    __syncthreads();   // the next sub-tile's prologue overwrites stage 0
   }
 
   // epilogue: acc[j][r] is C[m0 + wm*32 + 8*(r/4) + 4*(lane/32) + r%4][n0 + (wn*NT + j)*32 + lane%32]

@@ -176,6 +176,33 @@ def test_conv_odd_corners_integer_exact(hip):
             assert np.array_equal(dw - off, rdw), ('dW', xs, ws)
 
 
+def test_conv_channel_multiples_of_16_integer_exact(hip):
+    """Channel counts that are multiples of 16 take the tap-major kernels
+    (permuted weights, address arithmetic in the scalar offset); everything
+    else about the geometry varies."""
+    rs = np.random.RandomState(11)
+    cnt = 0
+    for (ic, oc), s, d, ks, padding in itertools.product([(16, 16), (32, 48), (48, 16), (16, 5), (6, 32)], [1, 2, 3],
+                                                         [1, 2], [1, 2, 3, 5], ['same', 'valid', 1]):
+        n, h, w_ = 2, 11, 9
+        if padding == 'valid' and min(h, w_) < (ks - 1) * d + 1:
+            continue
+        if cnt % 40 == 0:
+            say(f'conv c16 case {cnt}: ic={ic} oc={oc} s={s} d={d} ks={ks} pad={padding}')
+        x = rs.randint(8, size=(n, ic, h, w_)).astype(np.float32)
+        w = rs.randint(8, size=(oc, ic, ks, ks)).astype(np.float32)
+        ci = info_conv2d(h, w_, ks, ks, s, d, padding)
+        dy = rs.randint(8, size=(n, oc, ci.OH, ci.OW)).astype(np.float32)
+        y, dx, dw = _run_conv(hip, x, w, dy, s, d, padding, prefill=1.0)
+        ry, rdx, rdw = conv2d_all(x, w, dy, s, d, padding)
+        tag = (ic, oc, s, d, ks, padding)
+        assert np.array_equal(y, ry), ('fwd', tag)
+        assert np.array_equal(dx - 1.0, rdx), ('dX', tag)
+        assert np.array_equal(dw - 1.0, rdw), ('dW', tag)
+        cnt += 1
+    assert cnt > 250
+
+
 # benchmark geometries at a reduced batch (the oracle materialises im2col in fp64)
 _BENCH = {
     'cfg1': ((8, 3, 64, 64), (32, 3, 3, 3), 1, 1, 'same', 0),
