@@ -76,91 +76,94 @@ __global__ void permute_weights(float* wp, const float* w, int O, int C, int KK,
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
 struct ConvCfg {
-  static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * NTMAX;
-  // A side is K-contiguous in LDS for all three passes.
+  static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
+  // A side is K-contiguous in LDS for all passes.
   static constexpr int SA = LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
   static constexpr int SB = LdsSize<PASS == PASS_WGRAD, BNMAX>::value;
 };
 
-template <int PASS, class Cfg, int WM, int NT, bool FLAG>
-__device__ __forceinline__ void conv_tile(const ConvArgs& p, rsrc_t rx, rsrc_t rw, rsrc_t ro, float* lds, int mt,
-                                          int un, int kbeg, int kend) {
-  constexpr int WN = 4 / WM, BM = 32 * WM, BN = 32 * WN * NT;
-  const int m0 = mt * BM, n0 = un * 32 * WN;
+// Loader selection and initialisation per pass.  FLAG:
+//   PASS_FWD        128-bit loads of W rows (CKK % 4 == 0)
+//   PASS_DGRAD(_TAP) stride == 1
+//   PASS_WGRAD      128-bit loads of dY (OHW % 4 == 0)
+template <int PASS, bool FLAG>
+struct ConvProblem;
+
+struct ConvProblemBase {
+  ConvGeom g;
+  const KEntry* tab;
+  rsrc_t rx, rw, rc;
+  int M, Ncols, K, kbeg, kend, beta;
   OutMap om;
-  float* ldsB = lds + 2 * Cfg::SA;
-  if constexpr (PASS == PASS_FWD) {
-    PlainKC<BM, FLAG> la;            // FLAG: 128-bit loads of W rows (CKK % 4 == 0)
-    ConvFwdB<BN> lb;
-    la.init(rw, p.K, m0, p.M, p.K);
-    lb.init(rx, p.g, p.tab, n0, p.Ncols, kbeg);
-    om.nchw = 1; om.ld = p.g.OHW; om.mtot = p.g.O; om.dHW = p.g.dOHW;
-    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
-  } else if constexpr (PASS == PASS_FWD_TAP) {
-    PlainKC<BM, true> la;            // permuted weights [O][KK*C]
-    ConvFwdBTap<BN> lb;
-    la.init(rw, p.K, m0, p.M, p.K);
-    lb.init(rx, p.g, n0, p.Ncols, kbeg);
-    om.nchw = 1; om.ld = p.g.OHW; om.mtot = p.g.O; om.dHW = p.g.dOHW;
-    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
-  } else if constexpr (PASS == PASS_DGRAD_TAP) {
-    PlainKC<BM, true> la;            // permuted weights [C][KK*O]
-    ConvDgradBTap<BN, FLAG> lb;      // FLAG: stride == 1
-    la.init(rw, p.K, m0, p.M, p.K);
-    lb.init(rx, p.g, n0, p.Ncols, kbeg);
-    om.nchw = 1; om.ld = p.g.IHW; om.mtot = p.g.C; om.dHW = p.g.dIHW;
-    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
-  } else if constexpr (PASS == PASS_DGRAD) {
-    ConvDgradA<BM> la;
-    ConvDgradB<BN, FLAG> lb;         // FLAG: stride == 1
-    la.init(rw, p.g, p.tab, m0, kbeg);
-    lb.init(rx, p.g, p.tab, n0, p.Ncols, kbeg);
-    om.nchw = 1; om.ld = p.g.IHW; om.mtot = p.g.C; om.dHW = p.g.dIHW;
-    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
-  } else {
-    ConvWgradA<BM, FLAG> la;         // FLAG: 128-bit loads of dY (OHW % 4 == 0)
-    ConvWgradB<BN> lb;
-    la.init(rw, p.g, m0, kend);
-    lb.init(rx, p.g, p.tab, n0, p.Ncols, kend);
-    om.nchw = 0; om.ld = p.Ncols; om.mtot = 0; om.dHW = FastDiv{0, 0, 1};
-    run_tile<WM, NT>(la, lb, lds, ldsB, Cfg::SA, Cfg::SB, kbeg, kend, ro, om, m0, n0, p.M, p.Ncols, p.beta);
-  }
-}
+};
+
+template <bool FLAG>
+struct ConvProblem<PASS_FWD, FLAG> : ConvProblemBase {
+  template <int R> using LA = PlainKC<R, FLAG>;
+  template <int R> using LB = ConvFwdB<R>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
+  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
+};
+template <bool FLAG>
+struct ConvProblem<PASS_FWD_TAP, FLAG> : ConvProblemBase {
+  template <int R> using LA = PlainKC<R, true>;          // permuted weights [O][KK*C]
+  template <int R> using LB = ConvFwdBTap<R>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
+  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, col0, Ncols, kbeg); }
+};
+template <bool FLAG>
+struct ConvProblem<PASS_DGRAD, FLAG> : ConvProblemBase {
+  template <int R> using LA = ConvDgradA<R>;
+  template <int R> using LB = ConvDgradB<R, FLAG>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, tab, row0, kbeg); }
+  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
+};
+template <bool FLAG>
+struct ConvProblem<PASS_DGRAD_TAP, FLAG> : ConvProblemBase {
+  template <int R> using LA = PlainKC<R, true>;          // permuted weights [C][KK*O]
+  template <int R> using LB = ConvDgradBTap<R, FLAG>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
+  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, col0, Ncols, kbeg); }
+};
+template <bool FLAG>
+struct ConvProblem<PASS_WGRAD, FLAG> : ConvProblemBase {
+  template <int R> using LA = ConvWgradA<R, FLAG>;
+  template <int R> using LB = ConvWgradB<R>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend); }
+  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, tab, col0, Ncols, kend); }
+};
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
-__global__ __launch_bounds__(256, 2) void conv_kernel(ConvArgs p) {
+__global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
   using Cfg = ConvCfg<PASS, WM, NTMAX, FLAG>;
-  // at least 56 KB so that exactly two workgroups share a compute unit's 160 KB of LDS
-  __shared__ __attribute__((aligned(16))) float lds[(2 * (Cfg::SA + Cfg::SB) > 14336) ? 2 * (Cfg::SA + Cfg::SB) : 14336];
-  const rsrc_t rx = make_rsrc(p.X, p.bytesX);
-  const rsrc_t rw = make_rsrc(p.W, p.bytesW);
-  int kbeg = 0, kend = p.K;
-  float* out = p.Out;
-  if (PASS == PASS_WGRAD && p.ksplit > 1) {
-    const int nkt = (p.K + BK - 1) / BK;
-    const int t0 = (int)((long long)nkt * blockIdx.y / p.ksplit);
-    const int t1 = (int)((long long)nkt * (blockIdx.y + 1) / p.ksplit);
-    kbeg = t0 * BK;
-    kend = t1 * BK < p.K ? t1 * BK : p.K;
-    out += (size_t)blockIdx.y * p.M * p.Ncols;
+  __shared__ __attribute__((aligned(16))) float lds[2 * (Cfg::SA + Cfg::SB)];
+  ConvProblem<PASS, FLAG> p;
+  p.g = a.g;
+  p.tab = a.tab;
+  p.rx = make_rsrc(a.X, a.bytesX);
+  p.rw = make_rsrc(a.W, a.bytesW);
+  p.M = a.M; p.Ncols = a.Ncols; p.K = a.K; p.beta = a.beta;
+  p.kbeg = 0;
+  p.kend = a.K;
+  float* out = a.Out;
+  if (PASS == PASS_WGRAD && a.ksplit > 1) {
+    const int nkt = (a.K + BK - 1) / BK;
+    const int t0 = (int)((long long)nkt * blockIdx.y / a.ksplit);
+    const int t1 = (int)((long long)nkt * (blockIdx.y + 1) / a.ksplit);
+    p.kbeg = t0 * BK;
+    p.kend = t1 * BK < a.K ? t1 * BK : a.K;
+    out += (size_t)blockIdx.y * a.M * a.Ncols;
   }
-  const rsrc_t ro = make_rsrc(out, p.bytesOut);
-  long long u0 = (long long)p.total_units * blockIdx.x / gridDim.x;
-  const long long u1 = (long long)p.total_units * (blockIdx.x + 1) / gridDim.x;
-  while (u0 < u1) {
-    const int mt = (int)(u0 / p.n_units), un = (int)(u0 - (long long)mt * p.n_units);
-    long long cnt = u1 - u0;
-    if (cnt > p.n_units - un) cnt = p.n_units - un;
-    const int nt = pick_units<NTMAX>((int)cnt);
-    switch (nt) {
-      case 1: conv_tile<PASS, Cfg, WM, 1, FLAG>(p, rx, rw, ro, lds, mt, un, kbeg, kend); break;
-      case 2: conv_tile<PASS, Cfg, WM, (NTMAX >= 2 ? 2 : 1), FLAG>(p, rx, rw, ro, lds, mt, un, kbeg, kend); break;
-      case 3: conv_tile<PASS, Cfg, WM, (NTMAX >= 3 ? 3 : 1), FLAG>(p, rx, rw, ro, lds, mt, un, kbeg, kend); break;
-      default: conv_tile<PASS, Cfg, WM, (NTMAX >= 4 ? 4 : 1), FLAG>(p, rx, rw, ro, lds, mt, un, kbeg, kend); break;
-    }
-    u0 += nt;
+  p.rc = make_rsrc(out, a.bytesOut);
+  if (PASS == PASS_FWD || PASS == PASS_FWD_TAP) {
+    p.om.nchw = 1; p.om.ld = a.g.OHW; p.om.mtot = a.g.O; p.om.dHW = a.g.dOHW;
+  } else if (PASS == PASS_DGRAD || PASS == PASS_DGRAD_TAP) {
+    p.om.nchw = 1; p.om.ld = a.g.IHW; p.om.mtot = a.g.C; p.om.dHW = a.g.dIHW;
+  } else {
+    p.om.nchw = 0; p.om.ld = a.Ncols; p.om.mtot = 0; p.om.dHW = FastDiv{0, 0, 1};
   }
+  walk_units<WM, NTMAX>(p, lds, lds + 2 * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
 }
 
 // ---------------------------------------------------------------------------
@@ -239,13 +242,13 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   const long long total = (long long)m_tiles * a.n_units;
   if (total > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
   a.total_units = (int)total;
-  const long long slots = 2ll * ctx->cus;
+  const long long slots = ctx->cus;   // one 512-thread workgroup per compute unit
   int grid, ksplit = 1;
   float* final_out = a.Out;
   const int final_beta = a.beta;
   if (PASS == PASS_WGRAD) {
     // one full-width sub-tile per workgroup, then as many K slices as fill the chip
-    grid = (int)((total + NTMAX - 1) / NTMAX);
+    grid = (int)((total + 2 * NTMAX - 1) / (2 * NTMAX));
     const int nkt = (a.K + BK - 1) / BK;
     long long s = slots / grid;
     if (s > nkt / 4) s = nkt / 4;
@@ -263,7 +266,7 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     grid = (int)(total < slots ? total : slots);
   }
   a.ksplit = ksplit;
-  dim3 g(grid, ksplit, 1), b(256, 1, 1);
+  dim3 g(grid, ksplit, 1), b(512, 1, 1);
   if (flag)
     hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, true>), g, b, 0, ctx->stream, a);
   else
@@ -281,8 +284,8 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
 template <int PASS>
 static int launch_by_m(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   if (a.M > 64) return launch_pass<PASS, 4, 4>(ctx, a, flag);
-  if (a.M > 32) return launch_pass<PASS, 2, 4>(ctx, a, flag);
-  return launch_pass<PASS, 1, 2>(ctx, a, flag);
+  if (a.M > 32) return launch_pass<PASS, 2, 2>(ctx, a, flag);
+  return launch_pass<PASS, 1, 1>(ctx, a, flag);
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }

@@ -20,54 +20,37 @@ struct GemmArgs {
 
 template <int WM, int NTMAX, bool TA, bool TB, bool VEC>
 struct GemmCfg {
-  static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * NTMAX;
+  static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
   static constexpr int SA = LdsSize<!TA, BM>::value;
   static constexpr int SB = LdsSize<TB, BNMAX>::value;
 };
 
-template <class Cfg, int WM, int NT, bool TA, bool TB, bool VEC>
-__device__ __forceinline__ void gemm_tile(const GemmArgs& p, rsrc_t ra, rsrc_t rb, rsrc_t rc, float* lds,
-                                          int mt, int un) {
-  constexpr int WN = 4 / WM, BM = 32 * WM, BN = 32 * WN * NT;
-  using LA = typename std::conditional<TA, PlainMC<BM, VEC>, PlainKC<BM, VEC>>::type;
-  using LB = typename std::conditional<TB, PlainKC<BN, VEC>, PlainMC<BN, VEC>>::type;
-  const int m0 = mt * BM, n0 = un * 32 * WN;
-  LA la;
-  LB lb;
-  la.init(ra, p.lda, m0, p.M, p.K);
-  lb.init(rb, p.ldb, n0, p.N, p.K);
+// A operand: !TA -> A[M][K] row-major, K-contiguous; TA -> stored [K][M].
+// B operand: !TB -> B[K][N], row(n)-contiguous;      TB -> stored [N][K].
+template <bool TA, bool TB, bool VEC>
+struct GemmProblem {
+  template <int R> using LA = typename std::conditional<TA, PlainMC<R, VEC>, PlainKC<R, VEC>>::type;
+  template <int R> using LB = typename std::conditional<TB, PlainKC<R, VEC>, PlainMC<R, VEC>>::type;
+  rsrc_t ra, rb, rc;
+  int lda, ldb, M, Ncols, K, kbeg, kend, beta;
   OutMap om;
-  om.nchw = 0;
-  om.ld = p.ldc;
-  om.mtot = 0;
-  om.dHW = FastDiv{0, 0, 1};
-  run_tile<WM, NT>(la, lb, lds, lds + 2 * Cfg::SA, Cfg::SA, Cfg::SB, 0, p.K, rc, om, m0, n0, p.M, p.N, p.beta);
-}
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(ra, lda, row0, M, K); }
+  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rb, ldb, col0, Ncols, K); }
+};
 
 template <int WM, int NTMAX, bool TA, bool TB, bool VEC>
-__global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs p) {
+__global__ __launch_bounds__(512, 2) void gemm_kernel(GemmArgs a) {
   using Cfg = GemmCfg<WM, NTMAX, TA, TB, VEC>;
-  // at least 56 KB so that exactly two workgroups share a compute unit's 160 KB of LDS
-  __shared__ __attribute__((aligned(16))) float lds[(2 * (Cfg::SA + Cfg::SB) > 14336) ? 2 * (Cfg::SA + Cfg::SB) : 14336];
+  __shared__ __attribute__((aligned(16))) float lds[2 * (Cfg::SA + Cfg::SB)];
   const long long b = blockIdx.y;
-  const rsrc_t ra = make_rsrc(p.A + b * p.sA, p.bytesA);
-  const rsrc_t rb = make_rsrc(p.B + b * p.sB, p.bytesB);
-  const rsrc_t rc = make_rsrc(p.C + b * p.sC, p.bytesC);
-  long long u0 = (long long)p.total_units * blockIdx.x / gridDim.x;
-  const long long u1 = (long long)p.total_units * (blockIdx.x + 1) / gridDim.x;
-  while (u0 < u1) {
-    const int mt = (int)(u0 / p.n_units), un = (int)(u0 - (long long)mt * p.n_units);
-    long long cnt = u1 - u0;
-    if (cnt > p.n_units - un) cnt = p.n_units - un;
-    const int nt = pick_units<NTMAX>((int)cnt);
-    switch (nt) {
-      case 1: gemm_tile<Cfg, WM, 1, TA, TB, VEC>(p, ra, rb, rc, lds, mt, un); break;
-      case 2: gemm_tile<Cfg, WM, (NTMAX >= 2 ? 2 : 1), TA, TB, VEC>(p, ra, rb, rc, lds, mt, un); break;
-      case 3: gemm_tile<Cfg, WM, (NTMAX >= 3 ? 3 : 1), TA, TB, VEC>(p, ra, rb, rc, lds, mt, un); break;
-      default: gemm_tile<Cfg, WM, (NTMAX >= 4 ? 4 : 1), TA, TB, VEC>(p, ra, rb, rc, lds, mt, un); break;
-    }
-    u0 += nt;
-  }
+  GemmProblem<TA, TB, VEC> p;
+  p.ra = make_rsrc(a.A + b * a.sA, a.bytesA);
+  p.rb = make_rsrc(a.B + b * a.sB, a.bytesB);
+  p.rc = make_rsrc(a.C + b * a.sC, a.bytesC);
+  p.lda = a.lda; p.ldb = a.ldb; p.M = a.M; p.Ncols = a.N; p.K = a.K;
+  p.kbeg = 0; p.kend = a.K; p.beta = a.beta;
+  p.om.nchw = 0; p.om.ld = a.ldc; p.om.mtot = 0; p.om.dHW = FastDiv{0, 0, 1};
+  walk_units<WM, NTMAX>(p, lds, lds + 2 * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
 }
 
 template <int WM, int NTMAX, bool TA, bool TB>
@@ -78,10 +61,10 @@ static int launch_cfg(DeviceCtx* ctx, GemmArgs& a, int batch, bool vec) {
   const long long total = (long long)m_tiles * a.n_units;
   if (total > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "gemm: too many tiles");
   a.total_units = (int)total;
-  long long slots = 2ll * ctx->cus / (batch > 1 ? (batch > 8 ? 8 : batch) : 1);
+  long long slots = (long long)ctx->cus / (batch > 1 ? (batch > 8 ? 8 : batch) : 1);
   if (slots < 1) slots = 1;
   const int grid = (int)(total < slots ? total : slots);
-  dim3 g(grid, batch, 1), b(256, 1, 1);
+  dim3 g(grid, batch, 1), b(512, 1, 1);
   if (vec)
     hipLaunchKernelGGL((gemm_kernel<WM, NTMAX, TA, TB, true>), g, b, 0, ctx->stream, a);
   else
@@ -93,8 +76,8 @@ static int launch_cfg(DeviceCtx* ctx, GemmArgs& a, int batch, bool vec) {
 template <bool TA, bool TB>
 static int launch_layout(DeviceCtx* ctx, GemmArgs& a, int batch, bool vec) {
   if (a.M > 64) return launch_cfg<4, 4, TA, TB>(ctx, a, batch, vec);
-  if (a.M > 32) return launch_cfg<2, 4, TA, TB>(ctx, a, batch, vec);
-  return launch_cfg<1, 2, TA, TB>(ctx, a, batch, vec);
+  if (a.M > 32) return launch_cfg<2, 2, TA, TB>(ctx, a, batch, vec);
+  return launch_cfg<1, 1, TA, TB>(ctx, a, batch, vec);
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }

@@ -3,20 +3,27 @@
 //
 //   C[m, n] (+)= sum_k A(m, k) * B(k, n)
 //
-// A workgroup has 256 threads = 4 wavefronts of 64 lanes arranged WM x WN.
-// Each wavefront owns a 32 x (32*NT) slab of the output held in NT
-// v_mfma_f32_32x32x2_f32 accumulators.  Operand tiles are staged through LDS
-// (double buffered, one barrier per K step of BK) by "loader" objects which
-// differ only in how they turn (row, k) into a global address: plain strided
-// matrices or on-the-fly im2col gathers.  All global traffic uses raw buffer
-// instructions so that an out-of-range or masked element is a hardware zero
-// (loads) or a dropped write (stores) instead of a branch or a fault.
+// A workgroup has 512 threads: two groups of 4 wavefronts (arranged WM x WN
+// inside a group).  The two groups share one compute unit's four SIMDs, one
+// wavefront of each group per SIMD, and run in opposite phases separated by
+// workgroup barriers ("ping-pong"): while one group issues the MFMAs of a K
+// step, the other parks its previously fetched operands in LDS and issues the
+// global loads of a later step, so the matrix pipe of every SIMD always has
+// one wavefront feeding it.  Both groups work on the same M tile and K step
+// (they share the A operand tile in LDS) and on adjacent column ranges: group
+// g owns NT_g accumulators of v_mfma_f32_32x32x2_f32 per wavefront, i.e. a
+// 32 x (32*NT_g) slab.  Operand tiles are double buffered in LDS and filled by
+// "loader" objects which differ only in how they turn (row, k) into a global
+// address: plain strided matrices or on-the-fly im2col gathers.  All global
+// traffic uses raw buffer instructions so that an out-of-range or masked
+// element is a hardware zero (loads) or a dropped write (stores) instead of a
+// branch or a fault.
 //
 // Work distribution: the output is cut into "units" of 32*WN columns per
 // M-tile; the launch gives every workgroup a contiguous, nearly equal range of
 // units (so all compute units finish together regardless of how the problem
 // size divides into tiles) and the workgroup walks its range in sub-tiles of
-// 1..NTMAX units.
+// 1..2*NTMAX units, split between the two groups.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -33,6 +40,10 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 using rsrc_t = __amdgpu_buffer_rsrc_t;
 
+// thread / wavefront index inside a group of 256 threads
+__device__ __forceinline__ int gtid() { return threadIdx.x & 255; }
+__device__ __forceinline__ int gwave() { return (threadIdx.x >> 6) & 3; }
+
 __device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
 }
@@ -41,6 +52,14 @@ __device__ __forceinline__ float buf_load(rsrc_t r, uint32_t off) {
 }
 __device__ __forceinline__ f32x4 buf_load4(rsrc_t r, uint32_t off) {
   return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0));
+}
+// voff is per lane; soff is wave-uniform and travels in a scalar register, so
+// a K step can advance the address without any vector arithmetic.
+__device__ __forceinline__ float buf_load_s(rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0));
+}
+__device__ __forceinline__ f32x4 buf_load4_s(rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
 }
 __device__ __forceinline__ void buf_store(rsrc_t r, uint32_t off, float v) {
   __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, (int)off, 0, 0);
@@ -88,13 +107,26 @@ struct PlainKC {
     kend = kend_;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = threadIdx.x + 256 * e, row = s >> 2, kg = s & 3;
+      const int s = gtid() + 256 * e, row = s >> 2, kg = s & 3;
       const bool ok = row < R && row0 + row < rows_total;
       base[e] = ok ? (uint32_t)((row0 + row) * ld + 4 * kg) * 4u : OOB;
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
-    const int kg = threadIdx.x & 3;
+    if (k0 + BK <= kend) {   // whole K step in range (wave-uniform): no per-lane arithmetic
+      const uint32_t soff = (uint32_t)k0 * 4u;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        if (VEC) {
+          v[e] = buf_load4_s(rs, base[e], soff);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[e][j] = buf_load_s(rs, base[e] + 4u * j, soff);
+        }
+      }
+      return;
+    }
+    const int kg = gtid() & 3;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       if (VEC) {
@@ -109,11 +141,11 @@ struct PlainKC {
       }
     }
   }
-  __device__ __forceinline__ void commit(float* lds) const {
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = threadIdx.x + 256 * e, row = s >> 2, kg = s & 3;
-      if (R * 4 % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[row * LDK + 4 * kg]) = v[e];
+      const int s = gtid() + 256 * e, row = s >> 2, kg = s & 3;
+      if (R * 4 % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
     }
   }
 };
@@ -135,16 +167,29 @@ struct PlainMC {
     kend = kend_;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = threadIdx.x + 256 * e, ks = s / G, rg = s - ks * G;
+      const int s = gtid() + 256 * e, ks = s / G, rg = s - ks * G;
       const int left = rows_total - (row0 + 4 * rg);
       nval[e] = ks < BK ? (left < 0 ? 0 : (left > 4 ? 4 : left)) : 0;
       base[e] = nval[e] > 0 ? (uint32_t)(ks * ld + row0 + 4 * rg) * 4u : OOB;
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
+    if (k0 + BK <= kend) {   // whole K step in range (wave-uniform)
+      const uint32_t soff = (uint32_t)(k0 * ld) * 4u;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        if (VEC) {
+          v[e] = buf_load4_s(rs, base[e], soff);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[e][j] = buf_load_s(rs, j < nval[e] ? base[e] + 4u * j : OOB, soff);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = threadIdx.x + 256 * e, ks = s / G;
+      const int s = gtid() + 256 * e, ks = s / G;
       const uint32_t off = (k0 + ks < kend) ? base[e] + (uint32_t)(k0 * ld) * 4u : OOB;
       if (VEC) {
         v[e] = buf_load4(rs, off);
@@ -154,11 +199,11 @@ struct PlainMC {
       }
     }
   }
-  __device__ __forceinline__ void commit(float* lds) const {
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = threadIdx.x + 256 * e, ks = s / G, rg = s - ks * G;
-      if (BK * G % 256 == 0 || ks < BK) *reinterpret_cast<f32x4*>(&lds[ks * R + 4 * rg]) = v[e];
+      const int s = gtid() + 256 * e, ks = s / G, rg = s - ks * G;
+      if (BK * G % 256 == 0 || ks < BK) *reinterpret_cast<f32x4*>(&lds[ks * ld + off + 4 * rg]) = v[e];
     }
   }
 };
@@ -201,7 +246,7 @@ struct ConvFwdB {
   int tx[4], ty[4], tz[4];   // table entries of the next fetch (scalar registers)
   float v[4][CC];
   __device__ __forceinline__ void load_entries(int k0) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const ktab_t t = tab + (k0 + wave + 4 * e);
@@ -238,13 +283,13 @@ struct ConvFwdB {
     }
     load_entries(k0 + BK);
   }
-  __device__ __forceinline__ void commit(float* lds) const {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
+    const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
       for (int c = 0; c < CC; ++c)
-        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * R + lane + 64 * c] = v[e][c];
+        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
   }
 };
 
@@ -255,10 +300,6 @@ struct ConvFwdB {
 // channel part is wave-uniform and rides in the scalar offset of the buffer
 // instruction.  No table, no per-element arithmetic.  fetch() must be called
 // with consecutive K steps starting at the kbeg given to init().
-__device__ __forceinline__ float buf_load_s(rsrc_t r, uint32_t voff, uint32_t soff) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0));
-}
-
 template <int R>
 struct ConvFwdBTap {
   static constexpr bool KC = false;
@@ -266,8 +307,17 @@ struct ConvFwdBTap {
   rsrc_t rs;
   int IH, IW, IHW, C, D, KW;
   int base[CC], ih0[CC], iw0[CC];
+  uint32_t voff[CC];   // per-pixel byte offset for the current tap, or OOB
   int c0, kh, kw;   // K position of the next fetch
   float v[4][CC];
+  __device__ __forceinline__ void set_tap() {
+    const int dh = kh * D, dw = kw * D, tapoff = dh * IW + dw;
+#pragma unroll
+    for (int c = 0; c < CC; ++c) {
+      const bool ok = (uint32_t)(ih0[c] + dh) < (uint32_t)IH && (uint32_t)(iw0[c] + dw) < (uint32_t)IW;
+      voff[c] = ok ? (uint32_t)(base[c] + tapoff) * 4u : OOB;
+    }
+  }
   __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int p0, int P, int kbeg) {
     rs = r;
     IH = g.IH; IW = g.IW; IHW = g.IHW; C = g.C; D = g.D; KW = g.KW;
@@ -287,16 +337,10 @@ struct ConvFwdBTap {
       iw0[c] = ok ? (int)ow * g.S - g.PADL : -BIG;
       base[c] = ((int)img * g.C * g.IH + ih0[c]) * g.IW + ((int)ow * g.S - g.PADL);
     }
+    set_tap();
   }
   __device__ __forceinline__ void fetch(int) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int dh = kh * D, dw = kw * D, tapoff = dh * IW + dw;
-    uint32_t voff[CC];
-#pragma unroll
-    for (int c = 0; c < CC; ++c) {
-      const bool ok = (uint32_t)(ih0[c] + dh) < (uint32_t)IH && (uint32_t)(iw0[c] + dw) < (uint32_t)IW;
-      voff[c] = ok ? (uint32_t)(base[c] + tapoff) * 4u : OOB;
-    }
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const uint32_t soff = (uint32_t)((c0 + wave + 4 * e) * IHW) * 4u;
@@ -304,19 +348,20 @@ struct ConvFwdBTap {
       for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
     }
     c0 += BK;
-    if (c0 >= C) {
+    if (c0 >= C) {   // wave-uniform: next tap
       c0 = 0;
       ++kw;
       if (kw == KW) { kw = 0; ++kh; }
+      set_tap();
     }
   }
-  __device__ __forceinline__ void commit(float* lds) const {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
+    const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
       for (int c = 0; c < CC; ++c)
-        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * R + lane + 64 * c] = v[e][c];
+        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
   }
 };
 
@@ -328,8 +373,28 @@ struct ConvDgradBTap {
   int OH, OW, OHW, O, S, D, KW;
   FastDiv dS;
   int base[CC], a0[CC], b0[CC];
+  uint32_t voff[CC];
   int o0, kh, kw;
   float v[4][CC];
+  __device__ __forceinline__ void set_tap() {
+    const int dh = kh * D, dw = kw * D;
+#pragma unroll
+    for (int c = 0; c < CC; ++c) {
+      const int nh = a0[c] - dh, nw = b0[c] - dw;
+      bool ok;
+      int oh, ow;
+      if (STRIDE1) {
+        oh = nh;
+        ow = nw;
+        ok = (uint32_t)nh < (uint32_t)OH && (uint32_t)nw < (uint32_t)OW;
+      } else {
+        oh = (int)dS.div((uint32_t)nh & 0x7fffffffu);
+        ow = (int)dS.div((uint32_t)nw & 0x7fffffffu);
+        ok = nh >= 0 && nw >= 0 && oh * S == nh && ow * S == nw && oh < OH && ow < OW;
+      }
+      voff[c] = ok ? (uint32_t)(base[c] + oh * OW + ow) * 4u : OOB;
+    }
+  }
   __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int p0, int P, int kbeg) {
     rs = r;
     OH = g.OH; OW = g.OW; OHW = g.OHW; O = g.O; S = g.S; D = g.D; KW = g.KW;
@@ -350,27 +415,10 @@ struct ConvDgradBTap {
       b0[c] = ok ? (int)iw + g.PADL : -BIG;
       base[c] = (int)img * g.O * g.OHW;
     }
+    set_tap();
   }
   __device__ __forceinline__ void fetch(int) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int dh = kh * D, dw = kw * D;
-    uint32_t voff[CC];
-#pragma unroll
-    for (int c = 0; c < CC; ++c) {
-      const int nh = a0[c] - dh, nw = b0[c] - dw;
-      bool ok;
-      int oh, ow;
-      if (STRIDE1) {
-        oh = nh;
-        ow = nw;
-        ok = (uint32_t)nh < (uint32_t)OH && (uint32_t)nw < (uint32_t)OW;
-      } else {
-        oh = (int)dS.div((uint32_t)nh & 0x7fffffffu);
-        ow = (int)dS.div((uint32_t)nw & 0x7fffffffu);
-        ok = nh >= 0 && nw >= 0 && oh * S == nh && ow * S == nw && oh < OH && ow < OW;
-      }
-      voff[c] = ok ? (uint32_t)(base[c] + oh * OW + ow) * 4u : OOB;
-    }
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const uint32_t soff = (uint32_t)((o0 + wave + 4 * e) * OHW) * 4u;
@@ -378,19 +426,20 @@ struct ConvDgradBTap {
       for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
     }
     o0 += BK;
-    if (o0 >= O) {
+    if (o0 >= O) {   // wave-uniform: next tap
       o0 = 0;
       ++kw;
       if (kw == KW) { kw = 0; ++kh; }
+      set_tap();
     }
   }
-  __device__ __forceinline__ void commit(float* lds) const {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
+    const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
       for (int c = 0; c < CC; ++c)
-        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * R + lane + 64 * c] = v[e][c];
+        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
   }
 };
 
@@ -409,7 +458,7 @@ struct ConvDgradB {
   int tx[4], ty[4], tz[4];
   float v[4][CC];
   __device__ __forceinline__ void load_entries(int k0) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const ktab_t t = tab + (k0 + wave + 4 * e);
@@ -460,13 +509,13 @@ struct ConvDgradB {
     }
     load_entries(k0 + BK);
   }
-  __device__ __forceinline__ void commit(float* lds) const {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
+    const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
       for (int c = 0; c < CC; ++c)
-        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * R + lane + 64 * c] = v[e][c];
+        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
   }
 };
 
@@ -483,7 +532,7 @@ struct ConvDgradA {
   uint32_t tw[4];
   f32x4 v[E];
   __device__ __forceinline__ void load_entries(int k0) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
     for (int j = 0; j < 4; ++j) tw[j] = (uint32_t)(tab + (k0 + 4 * wave + j))->w;
   }
@@ -511,12 +560,12 @@ struct ConvDgradA {
     }
     load_entries(k0 + BK);
   }
-  __device__ __forceinline__ void commit(float* lds) const {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
+    const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < E; ++e)
       if (R % 64 == 0 || lane + 64 * e < R)
-        *reinterpret_cast<f32x4*>(&lds[(lane + 64 * e) * LDK + 4 * wave]) = v[e];
+        *reinterpret_cast<f32x4*>(&lds[(off + lane + 64 * e) * LDK + 4 * wave]) = v[e];
   }
 };
 
@@ -539,12 +588,12 @@ struct ConvWgradA {
     kend = kend_;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = threadIdx.x + 256 * e, row = s >> 2;
+      const int s = gtid() + 256 * e, row = s >> 2;
       rb[e] = (row < R && o0 + row < g.O) ? (uint32_t)((o0 + row) * g.OHW) : 0x20000000u;
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
-    const int kg = threadIdx.x & 3;
+    const int kg = gtid() & 3;
     if (VEC) {
       const uint32_t p = (uint32_t)(k0 + 4 * kg);
       const uint32_t img = dOHW.div(p), rem = p - img * OHW;
@@ -568,11 +617,11 @@ struct ConvWgradA {
       }
     }
   }
-  __device__ __forceinline__ void commit(float* lds) const {
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = threadIdx.x + 256 * e, row = s >> 2, kg = s & 3;
-      if (R * 4 % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[row * LDK + 4 * kg]) = v[e];
+      const int s = gtid() + 256 * e, row = s >> 2, kg = s & 3;
+      if (R * 4 % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
     }
   }
 };
@@ -596,7 +645,7 @@ struct ConvWgradB {
     kend = kend_;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = threadIdx.x + 256 * e, row = s >> 2;
+      const int s = gtid() + 256 * e, row = s >> 2;
       const bool ok = row < R && q0 + row < Q;
       const KEntry t = tab[ok ? q0 + row : 0];
       xo[e] = t.x;
@@ -605,7 +654,7 @@ struct ConvWgradB {
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
-    const int kg = threadIdx.x & 3;
+    const int kg = gtid() & 3;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t p = (uint32_t)(k0 + 4 * kg + j);
@@ -623,11 +672,11 @@ struct ConvWgradB {
       }
     }
   }
-  __device__ __forceinline__ void commit(float* lds) const {
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = threadIdx.x + 256 * e, row = s >> 2, kg = s & 3;
-      if (R * 4 % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[row * LDK + 4 * kg]) = v[e];
+      const int s = gtid() + 256 * e, row = s >> 2, kg = s & 3;
+      if (R * 4 % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
     }
   }
 };
@@ -678,96 +727,191 @@ __device__ __forceinline__ void load_frags(const float* __restrict__ As, const f
   }
 }
 
-// One LDS stage = BK/8 groups of 4*NT MFMAs.  The fragments of group kk+1 are
-// read from LDS before the MFMAs of group kk are issued, so the LDS latency is
-// covered by a full group of matrix work instead of stalling every group.
+// One LDS stage = BK/8 = 2 groups of 4*NT MFMAs.  The fragments of the first
+// group are read up front; the reads of the second group are slotted one by
+// one between the MFMAs of the first, so the matrix pipe starts after a single
+// LDS latency and never waits for LDS again within the stage.
 template <int NT, bool A_KC, bool B_KC, int RA, int RB>
 __device__ __forceinline__ void mma_stage(const float* __restrict__ As, const float* __restrict__ Bs,
                                           f32x16 (&acc)[NT], int arow, int brow) {
+  static_assert(BK == 16, "two MFMA groups per stage");
   float a[2][4], b[2][NT][4];
   load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, 0, a[0], b[0]);
+  load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, 1, a[1], b[1]);
 #pragma unroll
-  for (int kk = 0; kk < BK / 8; ++kk) {
-    const int cur = kk & 1;
-    if (kk + 1 < BK / 8) load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, kk + 1, a[cur ^ 1], b[cur ^ 1]);
+  for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int j = 0; j < NT; ++j)
-        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][t], b[cur][j][t], acc[j], 0, 0, 0);
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk][t], b[kk][j][t], acc[j], 0, 0, 0);
+  // LDS read instructions per group: A is one b128 or four b32; B is NT b128 or 4*NT b32 (paired into read2)
+  constexpr int RD = (A_KC ? 1 : 2) + (B_KC ? NT : 2 * NT);
+  __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);          // DS reads of group 0
+#pragma unroll
+  for (int i = 0; i < RD; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);         // one MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);         // one DS read of group 1
   }
+  __builtin_amdgcn_sched_group_barrier(0x008, 8 * NT - RD, 0);  // the remaining MFMAs
 }
 
 template <bool KC, int R>
 struct LdsSize { static constexpr int value = KC ? R * LDK : BK * R; };
 
-// One output sub-tile: BM x BN with BM = 32*WM, BN = 32*WN*NT.
-// The loaders must already be initialised for this tile.
-template <int WM, int NT, class LA, class LB>
-__device__ __forceinline__ void run_tile(LA& la, LB& lb, float* ldsA, float* ldsB, int strideA, int strideB,
-                                         int kbeg, int kend, rsrc_t rc, const OutMap& om, int m0, int n0,
-                                         int M, int Ncols, int beta) {
-  constexpr int WN = 4 / WM, BM = 32 * WM, BN = 32 * WN * NT;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+// What a kernel hands to the engine: loader types (templates over the row
+// count) and how to initialise them for one sub-tile.
+//
+//   struct Problem {
+//     template <int R> using LA = ...;   template <int R> using LB = ...;
+//     template <int R> void init_a(LA<R>&, int row0) const;
+//     template <int R> void init_b(LB<R>&, int col0) const;
+//     int kbeg, kend, M, Ncols, beta;  rsrc_t rc;  OutMap om;
+//   };
+
+// Body of one group (G = 0 or 1) for one sub-tile: BM = 32*WM rows shared by
+// both groups, 32*WN*NT columns of its own starting at column offset COFF of
+// the sub-tile; BNTOT is the column count of both groups together.
+template <int WM, int NT, int G, int COFF, int BNTOT, class P>
+__device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB, int strideA, int strideB, int m0,
+                                           int n0) {
+  constexpr int WN = 4 / WM, BM = 32 * WM, HALF = BM / 2, BN = 32 * WN * (NT > 0 ? NT : 1);
+  using LA = typename P::template LA<HALF>;
+  using LB = typename P::template LB<BN>;
+  constexpr bool A_KC = LA::KC, B_KC = LB::KC;
+  constexpr int LDA = A_KC ? LDK : BM, LDB = B_KC ? LDK : BNTOT;
+  const int wave = gwave(), lane = threadIdx.x & 63;
   const int wm = wave % WM, wn = wave / WM;
-  f32x16 acc[NT];
+  LA la;
+  LB lb;
+  p.template init_a<HALF>(la, m0 + G * HALF);
+  if (NT > 0) p.template init_b<BN>(lb, n0 + COFF);
+  f32x16 acc[NT > 0 ? NT : 1];
 #pragma unroll
-  for (int j = 0; j < NT; ++j)
+  for (int j = 0; j < (NT > 0 ? NT : 1); ++j)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
 
-  const int nk = (kend - kbeg + BK - 1) / BK;
+  const int kbeg = p.kbeg;
+  const int nk = (p.kend - kbeg + BK - 1) / BK;
+  // prologue: K step 0 into stage 0, K step 1 into registers
   if (nk > 0) {
     la.fetch(kbeg);
-    lb.fetch(kbeg);
-    la.commit(ldsA);
-    lb.commit(ldsB);
+    if (NT > 0) lb.fetch(kbeg);
+    la.commit(ldsA, LDA, G * HALF);
+    if (NT > 0) lb.commit(ldsB, LDB, COFF);
+  }
+  if (nk > 1) {
+    la.fetch(kbeg + BK);
+    if (NT > 0) lb.fetch(kbeg + BK);
   }
   __syncthreads();
-  // Steady state: the global loads of K step it+1 are issued first, so that
-  // they (and their address arithmetic) share one scheduling region with the
-  // MFMAs of step it; the data is parked in LDS after the MFMAs.
-  for (int it = 0; it + 1 < nk; ++it) {
-    const int cur = it & 1;
-    la.fetch(kbeg + (it + 1) * BK);
-    lb.fetch(kbeg + (it + 1) * BK);
-    __builtin_amdgcn_sched_barrier(0);   // keep the loads ahead of the matrix work
-    mma_stage<NT, LA::KC, LB::KC, BM, BN>(ldsA + cur * strideA, ldsB + cur * strideB, acc, wm * 32, wn * NT * 32);
-    __builtin_amdgcn_sched_barrier(0);
-    la.commit(ldsA + (cur ^ 1) * strideA);
-    lb.commit(ldsB + (cur ^ 1) * strideB);
-    __syncthreads();
-  }
-  if (nk > 0) {
-    const int cur = (nk - 1) & 1;
-    mma_stage<NT, LA::KC, LB::KC, BM, BN>(ldsA + cur * strideA, ldsB + cur * strideB, acc, wm * 32, wn * NT * 32);
-    __syncthreads();   // the next sub-tile's prologue overwrites stage 0
+  // Each K step t has two phases separated by barriers.  Group 0 computes in
+  // the first and moves data in the second; group 1 the other way round.
+  // "Moving data" for step t = park K step t+1 (fetched one step earlier) in
+  // the other LDS stage, then fetch K step t+2 into registers.  Stage (t+1)&1
+  // was last read for step t-1, which both groups finished before this step.
+  for (int t = 0; t < nk; ++t) {
+    const int cur = t & 1;
+#pragma unroll
+    for (int phase = 0; phase < 2; ++phase) {
+      if (phase == G) {
+        if (NT > 0)
+          mma_stage<(NT > 0 ? NT : 1), A_KC, B_KC, BM, BNTOT>(ldsA + cur * strideA, ldsB + cur * strideB, acc, wm * 32,
+                                                            COFF + wn * NT * 32);
+      } else {
+        if (t + 1 < nk) {
+          la.commit(ldsA + (cur ^ 1) * strideA, LDA, G * HALF);
+          if (NT > 0) lb.commit(ldsB + (cur ^ 1) * strideB, LDB, COFF);
+        }
+        if (t + 2 < nk) {
+          la.fetch(kbeg + (t + 2) * BK);
+          if (NT > 0) lb.fetch(kbeg + (t + 2) * BK);
+        }
+      }
+      // the phase ends only when all of its MFMAs have been issued: do not let
+      // the scheduler sink them below the barrier into the other group's phase
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 
-  // epilogue: acc[j][r] is C[m0 + wm*32 + 8*(r/4) + 4*(lane/32) + r%4][n0 + (wn*NT + j)*32 + lane%32]
-  const int i = lane & 31, h = lane >> 5;
+  // epilogue: acc[j][r] is C[m0 + wm*32 + 8*(r/4) + 4*(lane/32) + r%4][n0 + COFF + (wn*NT + j)*32 + lane%32]
+  if (NT > 0) {
+    const int i = lane & 31, h = lane >> 5;
 #pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    const int n = n0 + (wn * NT + j) * 32 + i;
-    const bool nok = n < Ncols;
-    const uint32_t cb = om.col(nok ? (uint32_t)n : 0u);
+    for (int j = 0; j < (NT > 0 ? NT : 1); ++j) {
+      const int n = n0 + COFF + (wn * NT + j) * 32 + i;
+      const bool nok = n < p.Ncols;
+      const uint32_t cb = p.om.col(nok ? (uint32_t)n : 0u);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-      const uint32_t off = (nok && m < M) ? (cb + (uint32_t)(m * om.ld)) * 4u : OOB;
-      float val = acc[j][r];
-      if (beta) val += buf_load(rc, off);
-      buf_store(rc, off, val);
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+        const uint32_t off = (nok && m < p.M) ? (cb + (uint32_t)(m * p.om.ld)) * 4u : OOB;
+        float val = acc[j][r];
+        if (p.beta) val += buf_load(p.rc, off);
+        buf_store(p.rc, off, val);
+      }
     }
   }
 }
 
-// Sub-tile width policy for a remaining run of cnt units.
-template <int NTMAX>
+// One output sub-tile of NT0 + NT1 units: rows [m0, m0 + 32*WM), columns
+// [n0, n0 + 32*WN*(NT0+NT1)).  Must be called by all 512 threads.
+template <int WM, int NT0, int NT1, class P>
+__device__ __forceinline__ void run_tile(const P& p, float* ldsA, float* ldsB, int strideA, int strideB, int m0,
+                                         int n0) {
+  constexpr int WN = 4 / WM, BNTOT = 32 * WN * (NT0 + NT1);
+  // wave-uniform by construction; read through a scalar so the two bodies are
+  // separate uniform branches (each wavefront executes exactly one of them)
+  if (__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) == 0)
+    group_body<WM, NT0, 0, 0, BNTOT>(p, ldsA, ldsB, strideA, strideB, m0, n0);
+  else
+    group_body<WM, NT1, 1, 32 * WN * NT0, BNTOT>(p, ldsA, ldsB, strideA, strideB, m0, n0);
+  __syncthreads();   // the next sub-tile's prologue overwrites stage 0
+}
+
+// Dispatch on the number of units (1 .. 2*NTMAX) of a sub-tile: group 0 takes
+// the larger half.
+template <int WM, int NTMAX, class P>
+__device__ __forceinline__ void run_units(int units, const P& p, float* ldsA, float* ldsB, int strideA, int strideB,
+                                          int m0, int n0) {
+  switch (units) {
+    case 1: run_tile<WM, 1, 0>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
+    case 2: run_tile<WM, 1, 1>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
+    case 3: run_tile<WM, (NTMAX >= 2 ? 2 : 1), (NTMAX >= 2 ? 1 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
+    case 4: run_tile<WM, (NTMAX >= 2 ? 2 : 1), (NTMAX >= 2 ? 2 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
+    case 5: run_tile<WM, (NTMAX >= 3 ? 3 : 1), (NTMAX >= 3 ? 2 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
+    case 6: run_tile<WM, (NTMAX >= 3 ? 3 : 1), (NTMAX >= 3 ? 3 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
+    case 7: run_tile<WM, (NTMAX >= 4 ? 4 : 1), (NTMAX >= 4 ? 3 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
+    default: run_tile<WM, (NTMAX >= 4 ? 4 : 1), (NTMAX >= 4 ? 4 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
+  }
+}
+
+// Sub-tile width policy for a remaining run of cnt units (at most MAXU per sub-tile).
+template <int MAXU>
 __device__ __forceinline__ int pick_units(int cnt) {
-  if (cnt <= NTMAX) return cnt;
-  if (cnt >= 2 * NTMAX) return NTMAX;
+  if (cnt <= MAXU) return cnt;
+  if (cnt >= 2 * MAXU) return MAXU;
   return (cnt + 1) >> 1;
+}
+
+// The walk of one workgroup over its share of the (M tile, unit) space.
+template <int WM, int NTMAX, class P>
+__device__ __forceinline__ void walk_units(const P& p, float* ldsA, float* ldsB, int strideA, int strideB,
+                                           int n_units, int total_units) {
+  constexpr int WN = 4 / WM;
+  long long u0 = (long long)total_units * blockIdx.x / gridDim.x;
+  const long long u1 = (long long)total_units * (blockIdx.x + 1) / gridDim.x;
+  while (u0 < u1) {
+    const int mt = (int)(u0 / n_units), un = (int)(u0 - (long long)mt * n_units);
+    long long cnt = u1 - u0;
+    if (cnt > n_units - un) cnt = n_units - un;
+    const int nt = pick_units<2 * NTMAX>((int)cnt);
+    run_units<WM, NTMAX>(nt, p, ldsA, ldsB, strideA, strideB, mt * 32 * WM, un * 32 * WN);
+    u0 += nt;
+  }
 }
 
 }  // namespace lnn
