@@ -30,7 +30,9 @@
 
 namespace lnn {
 
-constexpr int BK = 16;            // K extent of one LDS stage
+constexpr int BK = 32;            // K extent of one LDS stage
+constexpr int KG = BK / 4;        // float4 groups along K
+constexpr int KR = BK / 4;        // K rows fetched per wavefront of a group in the pixel-major gathers
 constexpr int LDK = BK + 4;       // row stride (floats) of a K-contiguous LDS tile
 constexpr uint32_t OOB = 0x80000000u;  // byte offset beyond every buffer (< 2 GiB each)
 constexpr int BIG = 0x40000000;   // coordinate that fails every range test
@@ -97,7 +99,7 @@ inline FastDiv make_fastdiv(uint32_t d) {
 template <int R, bool VEC>
 struct PlainKC {
   static constexpr bool KC = true;
-  static constexpr int E = (R * 4 + 255) / 256;
+  static constexpr int E = (R * KG + 255) / 256;
   rsrc_t rs;
   uint32_t base[E];
   int kend;
@@ -107,7 +109,7 @@ struct PlainKC {
     kend = kend_;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = gtid() + 256 * e, row = s >> 2, kg = s & 3;
+      const int s = gtid() + 256 * e, row = s / KG, kg = s % KG;
       const bool ok = row < R && row0 + row < rows_total;
       base[e] = ok ? (uint32_t)((row0 + row) * ld + 4 * kg) * 4u : OOB;
     }
@@ -126,7 +128,7 @@ struct PlainKC {
       }
       return;
     }
-    const int kg = gtid() & 3;
+    const int kg = gtid() % KG;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       if (VEC) {
@@ -144,8 +146,8 @@ struct PlainKC {
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = gtid() + 256 * e, row = s >> 2, kg = s & 3;
-      if (R * 4 % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
+      const int s = gtid() + 256 * e, row = s / KG, kg = s % KG;
+      if (R * KG % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
     }
   }
 };
@@ -243,12 +245,12 @@ struct ConvFwdB {
   ktab_t tab;
   int IH, IW;
   int base[CC], ih0[CC], iw0[CC];
-  int tx[4], ty[4], tz[4];   // table entries of the next fetch (scalar registers)
-  float v[4][CC];
+  int tx[KR], ty[KR], tz[KR];   // table entries of the next fetch (scalar registers)
+  float v[KR][CC];
   __device__ __forceinline__ void load_entries(int k0) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < KR; ++e) {
       const ktab_t t = tab + (k0 + wave + 4 * e);
       tx[e] = t->x; ty[e] = t->y; tz[e] = t->z;
     }
@@ -274,7 +276,7 @@ struct ConvFwdB {
   }
   __device__ __forceinline__ void fetch(int k0) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < KR; ++e) {
 #pragma unroll
       for (int c = 0; c < CC; ++c) {
         const bool ok = (uint32_t)(ih0[c] + ty[e]) < (uint32_t)IH && (uint32_t)(iw0[c] + tz[e]) < (uint32_t)IW;
@@ -286,7 +288,7 @@ struct ConvFwdB {
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
+    for (int e = 0; e < KR; ++e)
 #pragma unroll
       for (int c = 0; c < CC; ++c)
         if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
@@ -309,7 +311,7 @@ struct ConvFwdBTap {
   int base[CC], ih0[CC], iw0[CC];
   uint32_t voff[CC];   // per-pixel byte offset for the current tap, or OOB
   int c0, kh, kw;   // K position of the next fetch
-  float v[4][CC];
+  float v[KR][CC];
   __device__ __forceinline__ void set_tap() {
     const int dh = kh * D, dw = kw * D, tapoff = dh * IW + dw;
 #pragma unroll
@@ -342,7 +344,7 @@ struct ConvFwdBTap {
   __device__ __forceinline__ void fetch(int) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < KR; ++e) {
       const uint32_t soff = (uint32_t)((c0 + wave + 4 * e) * IHW) * 4u;
 #pragma unroll
       for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
@@ -358,7 +360,7 @@ struct ConvFwdBTap {
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
+    for (int e = 0; e < KR; ++e)
 #pragma unroll
       for (int c = 0; c < CC; ++c)
         if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
@@ -375,7 +377,7 @@ struct ConvDgradBTap {
   int base[CC], a0[CC], b0[CC];
   uint32_t voff[CC];
   int o0, kh, kw;
-  float v[4][CC];
+  float v[KR][CC];
   __device__ __forceinline__ void set_tap() {
     const int dh = kh * D, dw = kw * D;
 #pragma unroll
@@ -420,7 +422,7 @@ struct ConvDgradBTap {
   __device__ __forceinline__ void fetch(int) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < KR; ++e) {
       const uint32_t soff = (uint32_t)((o0 + wave + 4 * e) * OHW) * 4u;
 #pragma unroll
       for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
@@ -436,7 +438,7 @@ struct ConvDgradBTap {
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
+    for (int e = 0; e < KR; ++e)
 #pragma unroll
       for (int c = 0; c < CC; ++c)
         if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
@@ -455,12 +457,12 @@ struct ConvDgradB {
   int OH, OW, S;
   FastDiv dS;
   int base[CC], a0[CC], b0[CC];
-  int tx[4], ty[4], tz[4];
-  float v[4][CC];
+  int tx[KR], ty[KR], tz[KR];
+  float v[KR][CC];
   __device__ __forceinline__ void load_entries(int k0) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < KR; ++e) {
       const ktab_t t = tab + (k0 + wave + 4 * e);
       tx[e] = t->x; ty[e] = t->y; tz[e] = t->z;
     }
@@ -488,7 +490,7 @@ struct ConvDgradB {
   }
   __device__ __forceinline__ void fetch(int k0) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < KR; ++e) {
       const int t_x = tx[e];
 #pragma unroll
       for (int c = 0; c < CC; ++c) {
@@ -512,7 +514,7 @@ struct ConvDgradB {
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
+    for (int e = 0; e < KR; ++e)
 #pragma unroll
       for (int c = 0; c < CC; ++c)
         if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
@@ -520,21 +522,24 @@ struct ConvDgradB {
 };
 
 // dgrad weight gather: element (c, k = (o, kh, kw)) = W[o, c, kh, kw].
-// Wavefront w fetches k columns 4w..4w+3 (wave-uniform table entries); lanes
-// run over the channel rows.
+// Wavefront w fetches the k groups w, w+4, ... (four k each, wave-uniform table
+// entries); lanes run over the channel rows.
 template <int R>
 struct ConvDgradA {
   static constexpr bool KC = true;
   static constexpr int E = (R + 63) / 64;
+  static constexpr int NG = KG / 4;     // k groups per wavefront
   rsrc_t rs;
   ktab_t tab;
   uint32_t cb[E];
-  uint32_t tw[4];
-  f32x4 v[E];
+  uint32_t tw[NG][4];
+  f32x4 v[E][NG];
   __device__ __forceinline__ void load_entries(int k0) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
-    for (int j = 0; j < 4; ++j) tw[j] = (uint32_t)(tab + (k0 + 4 * wave + j))->w;
+    for (int q = 0; q < NG; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) tw[q][j] = (uint32_t)(tab + (k0 + 4 * (wave + 4 * q) + j))->w;
   }
   __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int c0, int kbeg) {
     rs = r;
@@ -549,23 +554,27 @@ struct ConvDgradA {
   }
   __device__ __forceinline__ void fetch(int k0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t w = tw[j];
+    for (int q = 0; q < NG; ++q)
 #pragma unroll
-      for (int e = 0; e < E; ++e) {
-        // either term alone is >= 2^29 elements (2 GiB) when invalid; clamp the sum
-        const uint32_t idx = cb[e] + w;
-        v[e][j] = buf_load(rs, idx >= 0x20000000u ? OOB : idx * 4u);
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t w = tw[q][j];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          // either term alone is >= 2^29 elements (2 GiB) when invalid; clamp the sum
+          const uint32_t idx = cb[e] + w;
+          v[e][q][j] = buf_load(rs, idx >= 0x20000000u ? OOB : idx * 4u);
+        }
       }
-    }
     load_entries(k0 + BK);
   }
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < E; ++e)
-      if (R % 64 == 0 || lane + 64 * e < R)
-        *reinterpret_cast<f32x4*>(&lds[(off + lane + 64 * e) * LDK + 4 * wave]) = v[e];
+#pragma unroll
+      for (int q = 0; q < NG; ++q)
+        if (R % 64 == 0 || lane + 64 * e < R)
+          *reinterpret_cast<f32x4*>(&lds[(off + lane + 64 * e) * LDK + 4 * (wave + 4 * q)]) = v[e][q];
   }
 };
 
@@ -574,7 +583,7 @@ struct ConvDgradA {
 template <int R, bool VEC>
 struct ConvWgradA {
   static constexpr bool KC = true;
-  static constexpr int E = (R * 4 + 255) / 256;
+  static constexpr int E = (R * KG + 255) / 256;
   rsrc_t rs;
   uint32_t rb[E];
   int O, OHW, kend;
@@ -588,12 +597,12 @@ struct ConvWgradA {
     kend = kend_;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = gtid() + 256 * e, row = s >> 2;
+      const int s = gtid() + 256 * e, row = s / KG;
       rb[e] = (row < R && o0 + row < g.O) ? (uint32_t)((o0 + row) * g.OHW) : 0x20000000u;
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
-    const int kg = gtid() & 3;
+    const int kg = gtid() % KG;
     if (VEC) {
       const uint32_t p = (uint32_t)(k0 + 4 * kg);
       const uint32_t img = dOHW.div(p), rem = p - img * OHW;
@@ -620,8 +629,8 @@ struct ConvWgradA {
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = gtid() + 256 * e, row = s >> 2, kg = s & 3;
-      if (R * 4 % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
+      const int s = gtid() + 256 * e, row = s / KG, kg = s % KG;
+      if (R * KG % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
     }
   }
 };
@@ -631,7 +640,7 @@ struct ConvWgradA {
 template <int R>
 struct ConvWgradB {
   static constexpr bool KC = true;
-  static constexpr int E = (R * 4 + 255) / 256;
+  static constexpr int E = (R * KG + 255) / 256;
   rsrc_t rs;
   int xo[E], dh[E], dw[E];
   int C, IH, IW, IHW, OHW, OW, S, PADL, PADT, kend;
@@ -645,7 +654,7 @@ struct ConvWgradB {
     kend = kend_;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = gtid() + 256 * e, row = s >> 2;
+      const int s = gtid() + 256 * e, row = s / KG;
       const bool ok = row < R && q0 + row < Q;
       const KEntry t = tab[ok ? q0 + row : 0];
       xo[e] = t.x;
@@ -654,7 +663,7 @@ struct ConvWgradB {
     }
   }
   __device__ __forceinline__ void fetch(int k0) {
-    const int kg = gtid() & 3;
+    const int kg = gtid() % KG;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t p = (uint32_t)(k0 + 4 * kg + j);
@@ -675,8 +684,8 @@ struct ConvWgradB {
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int s = gtid() + 256 * e, row = s >> 2, kg = s & 3;
-      if (R * 4 % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
+      const int s = gtid() + 256 * e, row = s / KG, kg = s % KG;
+      if (R * KG % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
     }
   }
 };
@@ -727,33 +736,39 @@ __device__ __forceinline__ void load_frags(const float* __restrict__ As, const f
   }
 }
 
-// One LDS stage = BK/8 = 2 groups of 4*NT MFMAs.  The fragments of the first
-// group are read up front; the reads of the second group are slotted one by
-// one between the MFMAs of the first, so the matrix pipe starts after a single
-// LDS latency and never waits for LDS again within the stage.
+// One LDS stage = BK/8 groups of 4*NT MFMAs.  The fragments of the first
+// group are read up front; the reads of each following group are slotted one
+// by one between the MFMAs of the group before it, so the matrix pipe starts
+// after a single LDS latency and does not wait for LDS again within the stage.
 template <int NT, bool A_KC, bool B_KC, int RA, int RB>
 __device__ __forceinline__ void mma_stage(const float* __restrict__ As, const float* __restrict__ Bs,
                                           f32x16 (&acc)[NT], int arow, int brow) {
-  static_assert(BK == 16, "two MFMA groups per stage");
-  float a[2][4], b[2][NT][4];
+  constexpr int NG = BK / 8;
+  // LDS read instructions per group: A is one b128 or four b32; B is NT b128 or 4*NT b32 (paired into read2)
+  constexpr int RD = (A_KC ? 1 : 2) + (B_KC ? NT : 2 * NT);
+  float a[2][4], b[2][NT][4];   // fragment double buffer
   load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, 0, a[0], b[0]);
-  load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, 1, a[1], b[1]);
+  __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);              // DS reads of group 0
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk)
+  for (int kk = 0; kk < NG; ++kk) {
+    const int cur = kk & 1;
+    if (kk + 1 < NG) load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, kk + 1, a[cur ^ 1], b[cur ^ 1]);
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int j = 0; j < NT; ++j)
-        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk][t], b[kk][j][t], acc[j], 0, 0, 0);
-  // LDS read instructions per group: A is one b128 or four b32; B is NT b128 or 4*NT b32 (paired into read2)
-  constexpr int RD = (A_KC ? 1 : 2) + (B_KC ? NT : 2 * NT);
-  __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);          // DS reads of group 0
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][t], b[cur][j][t], acc[j], 0, 0, 0);
+    if (kk + 1 < NG) {
 #pragma unroll
-  for (int i = 0; i < RD; ++i) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);         // one MFMA
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);         // one DS read of group 1
+      for (int i = 0; i < RD; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);         // one MFMA of group kk
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);         // one DS read of group kk+1
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * NT - RD, 0);  // the remaining MFMAs of group kk
+    } else {
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * NT, 0);       // last group
+    }
   }
-  __builtin_amdgcn_sched_group_barrier(0x008, 8 * NT - RD, 0);  // the remaining MFMAs
 }
 
 template <bool KC, int R>
