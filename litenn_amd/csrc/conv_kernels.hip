@@ -20,6 +20,8 @@ struct ConvArgs {
   int beta;
   int n_units, total_units;
   int ksplit;        // wgrad: number of K slices (gridDim.y)
+  FastDiv dC;        // tap-major wgrad: divide a column index by the channel count
+  int chunk_units;   // tap-major wgrad: units per workgroup
 };
 
 // mode 0: k = (c, kh, kw) for forward / wgrad; mode 1: k = (o, kh, kw) for dgrad.
@@ -56,7 +58,7 @@ __global__ void reduce_partials(float* out, const float* part, int n, int slices
 }
 
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
-enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4 };
+enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5 };
 
 // Wp[a][tap][b] = W[..] so that the tap-major K index tap*CH + ch is contiguous:
 //   mode 0 (forward): Wp[o][tap][c] = W[o][c][tap]
@@ -80,7 +82,7 @@ struct ConvCfg {
   // A side is K-contiguous in LDS for all passes.
   static constexpr int SA = LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
-  static constexpr int SB = LdsSize<PASS == PASS_WGRAD, BNMAX>::value;
+  static constexpr int SB = LdsSize<PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP, BNMAX>::value;
 };
 
 // Loader selection and initialisation per pass.  FLAG:
@@ -103,35 +105,43 @@ struct ConvProblem<PASS_FWD, FLAG> : ConvProblemBase {
   template <int R> using LA = PlainKC<R, FLAG>;
   template <int R> using LB = ConvFwdB<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
-  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
 template <bool FLAG>
 struct ConvProblem<PASS_FWD_TAP, FLAG> : ConvProblemBase {
   template <int R> using LA = PlainKC<R, true>;          // permuted weights [O][KK*C]
   template <int R> using LB = ConvFwdBTap<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
-  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, col0, Ncols, kbeg); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, col0, Ncols, kbeg); }
 };
 template <bool FLAG>
 struct ConvProblem<PASS_DGRAD, FLAG> : ConvProblemBase {
   template <int R> using LA = ConvDgradA<R>;
   template <int R> using LB = ConvDgradB<R, FLAG>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, tab, row0, kbeg); }
-  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
 template <bool FLAG>
 struct ConvProblem<PASS_DGRAD_TAP, FLAG> : ConvProblemBase {
   template <int R> using LA = PlainKC<R, true>;          // permuted weights [C][KK*O]
   template <int R> using LB = ConvDgradBTap<R, FLAG>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
-  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, col0, Ncols, kbeg); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, col0, Ncols, kbeg); }
 };
 template <bool FLAG>
 struct ConvProblem<PASS_WGRAD, FLAG> : ConvProblemBase {
   template <int R> using LA = ConvWgradA<R, FLAG>;
   template <int R> using LB = ConvWgradB<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend); }
-  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rx, g, tab, col0, Ncols, kend); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kend); }
+};
+
+template <bool FLAG>
+struct ConvProblem<PASS_WGRAD_TAP, FLAG> : ConvProblemBase {
+  template <int R> using LA = ConvWgradTapA<R>;
+  template <int R> using LB = ConvWgradTapB<R>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A& la) const { l.init(rx, g, col0, la); }
 };
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
@@ -147,7 +157,7 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
   p.kbeg = 0;
   p.kend = a.K;
   float* out = a.Out;
-  if (PASS == PASS_WGRAD && a.ksplit > 1) {
+  if ((PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP) && a.ksplit > 1) {
     const int nkt = (a.K + BK - 1) / BK;
     const int t0 = (int)((long long)nkt * blockIdx.y / a.ksplit);
     const int t1 = (int)((long long)nkt * (blockIdx.y + 1) / a.ksplit);
@@ -160,10 +170,17 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
     p.om.nchw = 1; p.om.ld = a.g.OHW; p.om.mtot = a.g.O; p.om.dHW = a.g.dOHW;
   } else if (PASS == PASS_DGRAD || PASS == PASS_DGRAD_TAP) {
     p.om.nchw = 1; p.om.ld = a.g.IHW; p.om.mtot = a.g.C; p.om.dHW = a.g.dIHW;
+  } else if (PASS == PASS_WGRAD_TAP) {
+    // GEMM column tap*C + c lands in dW[o][c][tap]
+    p.om.nchw = 2; p.om.ld = a.Ncols; p.om.mtot = a.g.KK; p.om.dHW = a.dC;
   } else {
     p.om.nchw = 0; p.om.ld = a.Ncols; p.om.mtot = 0; p.om.dHW = FastDiv{0, 0, 1};
   }
-  walk_units<WM, NTMAX>(p, lds, lds + 2 * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
+  if (PASS == PASS_WGRAD_TAP)
+    walk_units_seg<WM, NTMAX>(p, lds, lds + 2 * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.g.KK, a.total_units,
+                              a.chunk_units);
+  else
+    walk_units<WM, NTMAX>(p, lds, lds + 2 * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
 }
 
 // ---------------------------------------------------------------------------
@@ -239,16 +256,27 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   constexpr int WN = 4 / WM, BM = 32 * WM;
   const int m_tiles = (a.M + BM - 1) / BM;
   a.n_units = (a.Ncols + 32 * WN - 1) / (32 * WN);
-  const long long total = (long long)m_tiles * a.n_units;
+  long long total = (long long)m_tiles * a.n_units;
+  a.chunk_units = 0;
+  if (PASS == PASS_WGRAD_TAP) {
+    // columns are tap-major: KK segments of C / (32*WN) units per M tile; a workgroup
+    // takes one sub-tile's worth of whole segments (or of one segment's halves)
+    a.n_units = a.g.C / (32 * WN);
+    const int per_group = a.n_units < NTMAX ? a.n_units : NTMAX;
+    a.chunk_units = 2 * per_group;
+    total = (long long)m_tiles * a.g.KK * a.n_units;
+    a.dC = make_fastdiv((uint32_t)a.g.C);
+  }
   if (total > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
   a.total_units = (int)total;
   const long long slots = ctx->cus;   // one 512-thread workgroup per compute unit
   int grid, ksplit = 1;
   float* final_out = a.Out;
   const int final_beta = a.beta;
-  if (PASS == PASS_WGRAD) {
+  if (PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP) {
     // one full-width sub-tile per workgroup, then as many K slices as fill the chip
-    grid = (int)((total + 2 * NTMAX - 1) / (2 * NTMAX));
+    const int chunk = PASS == PASS_WGRAD_TAP ? a.chunk_units : 2 * NTMAX;
+    grid = (int)((total + chunk - 1) / chunk);
     const int nkt = (a.K + BK - 1) / BK;
     long long s = slots / grid;
     if (s > nkt / 4) s = nkt / 4;
@@ -350,6 +378,9 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   a.bytesOut = (uint32_t)((uint64_t)g.O * g.C * g.KK * 4);
   a.M = g.O; a.Ncols = g.C * g.KK; a.K = g.N * g.OHW;
   a.beta = beta ? 1 : 0;
+  // pixel-major loaders when the channels fill whole units of the tile shape chosen for O
+  const int unit = g.O > 64 ? 32 : (g.O > 32 ? 64 : 128);
+  if (g.C % unit == 0) return launch_by_m<PASS_WGRAD_TAP>(ctx, a, false);
   return launch_by_m<PASS_WGRAD>(ctx, a, g.OHW % 4 == 0 && aligned16(dY));
 }
 

@@ -35,7 +35,7 @@ struct GemmProblem {
   int lda, ldb, M, Ncols, K, kbeg, kend, beta;
   OutMap om;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(ra, lda, row0, M, K); }
-  template <int R> __device__ __forceinline__ void init_b(LB<R>& l, int col0) const { l.init(rb, ldb, col0, Ncols, K); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rb, ldb, col0, Ncols, K); }
 };
 
 template <int WM, int NTMAX, bool TA, bool TB, bool VEC>

@@ -28,6 +28,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace lnn {
 
 constexpr int BK = 32;            // K extent of one LDS stage
@@ -690,19 +692,101 @@ struct ConvWgradB {
   }
 };
 
+// Pixel-major wgrad loaders for channel counts that fill whole units: K = the
+// output pixel p, and the GEMM columns are ordered tap-major (column = tap*C + c)
+// so that all columns of a group belong to one tap.  Lane (tid % 32) owns one
+// pixel of the K step, tid / 32 selects a row subgroup; the rows of a thread
+// are sub + 8*e and differ only by a wave-uniform multiple of the plane size,
+// which rides in the scalar offset.  Per K step a thread decomposes its pixel
+// once (shared by both loaders), tests the padding once, and issues its loads.
+template <int R>
+struct ConvWgradTapA {
+  static constexpr bool KC = true;
+  static constexpr int E = R / 8;       // rows per thread (R is a multiple of 8)
+  rsrc_t rs;
+  int OHW, OOHW, kend;
+  FastDiv dOHW;
+  uint32_t rowoff;          // (first row of this thread) * OHW
+  uint32_t img, rem;        // decomposition of this thread's pixel in the last fetch
+  bool pok;
+  float v[E];
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int o0, int kend_) {
+    rs = r;
+    OHW = g.OHW;
+    OOHW = g.O * g.OHW;
+    dOHW = g.dOHW;
+    kend = kend_;
+    rowoff = (uint32_t)((o0 + (gtid() >> 5)) * g.OHW);
+  }
+  __device__ __forceinline__ void fetch(int k0) {
+    const uint32_t p = (uint32_t)(k0 + (gtid() & 31));
+    pok = p < (uint32_t)kend;
+    img = dOHW.div(p);
+    rem = p - img * OHW;
+    // rows past the last output channel are never stored, so they need no mask
+    const uint32_t voff = pok ? (img * (uint32_t)OOHW + rem + rowoff) * 4u : OOB;
+#pragma unroll
+    for (int e = 0; e < E; ++e) v[e] = buf_load_s(rs, voff, (uint32_t)(8 * e * OHW) * 4u);
+  }
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
+    const int l = gtid() & 31, sub = gtid() >> 5;
+#pragma unroll
+    for (int e = 0; e < E; ++e) lds[(off + sub + 8 * e) * LDK + l] = v[e];
+  }
+};
+
+template <int R>
+struct ConvWgradTapB {
+  static constexpr bool KC = true;
+  static constexpr bool NEEDS_A = true;
+  static constexpr int E = R / 8;
+  rsrc_t rs;
+  int C, IH, IW, IHW, OW, S;
+  FastDiv dOW;
+  int dh, dw;               // kh*D - PADT, kw*D - PADL of this group's tap
+  uint32_t chanoff;         // (first channel of this thread) * IHW
+  float v[E];
+  template <class LA>
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int col0, const LA&) {
+    rs = r;
+    C = g.C; IH = g.IH; IW = g.IW; IHW = g.IHW; OW = g.OW; S = g.S;
+    dOW = g.dOW;
+    const int tap = col0 / g.C, c0 = col0 - tap * g.C;
+    const int kh = tap / g.KW, kw = tap - kh * g.KW;
+    dh = kh * g.D - g.PADT;
+    dw = kw * g.D - g.PADL;
+    chanoff = (uint32_t)((c0 + (gtid() >> 5)) * g.IHW);
+  }
+  template <class LA>
+  __device__ __forceinline__ void fetch(int, const LA& la) {
+    const uint32_t oh = dOW.div(la.rem), ow = la.rem - oh * OW;
+    const int ih = (int)oh * S + dh, iw = (int)ow * S + dw;
+    const bool ok = la.pok && (uint32_t)ih < (uint32_t)IH && (uint32_t)iw < (uint32_t)IW;
+    const uint32_t voff = ok ? (la.img * (uint32_t)(C * IHW) + (uint32_t)(ih * IW + iw) + chanoff) * 4u : OOB;
+#pragma unroll
+    for (int e = 0; e < E; ++e) v[e] = buf_load_s(rs, voff, (uint32_t)(8 * e * IHW) * 4u);
+  }
+  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
+    const int l = gtid() & 31, sub = gtid() >> 5;
+#pragma unroll
+    for (int e = 0; e < E; ++e) lds[(off + sub + 8 * e) * LDK + l] = v[e];
+  }
+};
+
 // ---------------------------------------------------------------------------
 // Output mapping.  plain: off = m*ld + n.  NCHW image tensor with the GEMM
 // column n = (img, pixel): off = (img*Mtot + m)*HW + pixel.
 // ---------------------------------------------------------------------------
 struct OutMap {
-  int nchw;    // 0 plain, 1 image layout
-  int ld;      // plain: leading dimension; nchw: HW
-  int mtot;    // nchw: channel count
-  FastDiv dHW;
+  int nchw;    // 0 plain, 1 image layout, 2 tap-major weight columns
+  int ld;      // plain / tap-major: leading dimension; nchw: HW
+  int mtot;    // nchw: channel count; tap-major: KK
+  FastDiv dHW; // nchw: divide by HW; tap-major: divide by the channel count C
   __device__ __forceinline__ uint32_t col(uint32_t n) const {
-    if (!nchw) return n;
-    const uint32_t img = dHW.div(n);
-    return img * (uint32_t)(mtot * ld) + (n - img * ld);
+    if (nchw == 0) return n;
+    const uint32_t q = dHW.div(n);
+    if (nchw == 1) return q * (uint32_t)(mtot * ld) + (n - q * ld);   // q = image
+    return (n - q * dHW.d) * (uint32_t)mtot + q;                      // q = tap: column tap*C + c -> c*KK + tap
   }
 };
 
@@ -780,16 +864,30 @@ struct LdsSize { static constexpr int value = KC ? R * LDK : BK * R; };
 //   struct Problem {
 //     template <int R> using LA = ...;   template <int R> using LB = ...;
 //     template <int R> void init_a(LA<R>&, int row0) const;
-//     template <int R> void init_b(LB<R>&, int col0) const;
+//     template <int R, class A> void init_b(LB<R>&, int col0, A& la) const;   (la: this group's A loader)
 //     int kbeg, kend, M, Ncols, beta;  rsrc_t rc;  OutMap om;
 //   };
+
+// A B-side loader that shares per-step state with its group's A loader
+// declares `static constexpr bool NEEDS_A = true` and takes the A loader in fetch().
+template <class T, class = void>
+struct needs_a : std::false_type {};
+template <class T>
+struct needs_a<T, std::void_t<decltype(T::NEEDS_A)>> : std::true_type {};
+template <class LB, class LA>
+__device__ __forceinline__ void fetch_b(LB& lb, int k0, const LA& la) {
+  if constexpr (needs_a<LB>::value)
+    lb.fetch(k0, la);
+  else
+    lb.fetch(k0);
+}
 
 // Body of one group (G = 0 or 1) for one sub-tile: BM = 32*WM rows shared by
 // both groups, 32*WN*NT columns of its own starting at column offset COFF of
 // the sub-tile; BNTOT is the column count of both groups together.
 template <int WM, int NT, int G, int COFF, int BNTOT, class P>
 __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB, int strideA, int strideB, int m0,
-                                           int n0) {
+                                           int ng) {   // ng: first global column of this group
   constexpr int WN = 4 / WM, BM = 32 * WM, HALF = BM / 2, BN = 32 * WN * (NT > 0 ? NT : 1);
   using LA = typename P::template LA<HALF>;
   using LB = typename P::template LB<BN>;
@@ -800,7 +898,7 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
   LA la;
   LB lb;
   p.template init_a<HALF>(la, m0 + G * HALF);
-  if (NT > 0) p.template init_b<BN>(lb, n0 + COFF);
+  if (NT > 0) p.template init_b<BN>(lb, ng, la);
   f32x16 acc[NT > 0 ? NT : 1];
 #pragma unroll
   for (int j = 0; j < (NT > 0 ? NT : 1); ++j)
@@ -812,13 +910,13 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
   // prologue: K step 0 into stage 0, K step 1 into registers
   if (nk > 0) {
     la.fetch(kbeg);
-    if (NT > 0) lb.fetch(kbeg);
+    if (NT > 0) fetch_b(lb, kbeg, la);
     la.commit(ldsA, LDA, G * HALF);
     if (NT > 0) lb.commit(ldsB, LDB, COFF);
   }
   if (nk > 1) {
     la.fetch(kbeg + BK);
-    if (NT > 0) lb.fetch(kbeg + BK);
+    if (NT > 0) fetch_b(lb, kbeg + BK, la);
   }
   __syncthreads();
   // Each K step t has two phases separated by barriers.  Group 0 computes in
@@ -841,7 +939,7 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
         }
         if (t + 2 < nk) {
           la.fetch(kbeg + (t + 2) * BK);
-          if (NT > 0) lb.fetch(kbeg + (t + 2) * BK);
+          if (NT > 0) fetch_b(lb, kbeg + (t + 2) * BK, la);
         }
       }
       // the phase ends only when all of its MFMAs have been issued: do not let
@@ -852,12 +950,12 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
     }
   }
 
-  // epilogue: acc[j][r] is C[m0 + wm*32 + 8*(r/4) + 4*(lane/32) + r%4][n0 + COFF + (wn*NT + j)*32 + lane%32]
+  // epilogue: acc[j][r] is C[m0 + wm*32 + 8*(r/4) + 4*(lane/32) + r%4][ng + (wn*NT + j)*32 + lane%32]
   if (NT > 0) {
     const int i = lane & 31, h = lane >> 5;
 #pragma unroll
     for (int j = 0; j < (NT > 0 ? NT : 1); ++j) {
-      const int n = n0 + COFF + (wn * NT + j) * 32 + i;
+      const int n = ng + (wn * NT + j) * 32 + i;
       const bool nok = n < p.Ncols;
       const uint32_t cb = p.om.col(nok ? (uint32_t)n : 0u);
 #pragma unroll
@@ -872,36 +970,36 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
   }
 }
 
-// One output sub-tile of NT0 + NT1 units: rows [m0, m0 + 32*WM), columns
-// [n0, n0 + 32*WN*(NT0+NT1)).  Must be called by all 512 threads.
+// One output sub-tile: rows [m0, m0 + 32*WM); group 0 owns NT0 units of columns
+// starting at global column n0a, group 1 owns NT1 units starting at n0b
+// (normally n0a + 32*WN*NT0).  Must be called by all 512 threads.
 template <int WM, int NT0, int NT1, class P>
 __device__ __forceinline__ void run_tile(const P& p, float* ldsA, float* ldsB, int strideA, int strideB, int m0,
-                                         int n0) {
+                                         int n0a, int n0b) {
   constexpr int WN = 4 / WM, BNTOT = 32 * WN * (NT0 + NT1);
   // wave-uniform by construction; read through a scalar so the two bodies are
   // separate uniform branches (each wavefront executes exactly one of them)
   if (__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) == 0)
-    group_body<WM, NT0, 0, 0, BNTOT>(p, ldsA, ldsB, strideA, strideB, m0, n0);
+    group_body<WM, NT0, 0, 0, BNTOT>(p, ldsA, ldsB, strideA, strideB, m0, n0a);
   else
-    group_body<WM, NT1, 1, 32 * WN * NT0, BNTOT>(p, ldsA, ldsB, strideA, strideB, m0, n0);
+    group_body<WM, NT1, 1, 32 * WN * NT0, BNTOT>(p, ldsA, ldsB, strideA, strideB, m0, n0b);
   __syncthreads();   // the next sub-tile's prologue overwrites stage 0
 }
 
-// Dispatch on the number of units (1 .. 2*NTMAX) of a sub-tile: group 0 takes
-// the larger half.
-template <int WM, int NTMAX, class P>
-__device__ __forceinline__ void run_units(int units, const P& p, float* ldsA, float* ldsB, int strideA, int strideB,
-                                          int m0, int n0) {
-  switch (units) {
-    case 1: run_tile<WM, 1, 0>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
-    case 2: run_tile<WM, 1, 1>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
-    case 3: run_tile<WM, (NTMAX >= 2 ? 2 : 1), (NTMAX >= 2 ? 1 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
-    case 4: run_tile<WM, (NTMAX >= 2 ? 2 : 1), (NTMAX >= 2 ? 2 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
-    case 5: run_tile<WM, (NTMAX >= 3 ? 3 : 1), (NTMAX >= 3 ? 2 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
-    case 6: run_tile<WM, (NTMAX >= 3 ? 3 : 1), (NTMAX >= 3 ? 3 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
-    case 7: run_tile<WM, (NTMAX >= 4 ? 4 : 1), (NTMAX >= 4 ? 3 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
-    default: run_tile<WM, (NTMAX >= 4 ? 4 : 1), (NTMAX >= 4 ? 4 : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0); break;
+// Dispatch on the unit counts of the two groups (nt0 >= nt1, 1 <= nt0 <= NTMAX).
+template <int WM, int NTMAX, bool ANYPAIR, class P>
+__device__ __forceinline__ void run_pair(int nt0, int nt1, const P& p, float* ldsA, float* ldsB, int strideA,
+                                         int strideB, int m0, int n0a, int n0b) {
+#define LNN_PAIR(A, B)                                                                                   \
+  if (nt0 == A && nt1 == B) {                                                                            \
+    run_tile<WM, (A <= NTMAX ? A : 1), (A <= NTMAX ? B : 0)>(p, ldsA, ldsB, strideA, strideB, m0, n0a, n0b); \
+    return;                                                                                              \
   }
+  LNN_PAIR(1, 0) LNN_PAIR(1, 1)
+  if (NTMAX >= 2) { LNN_PAIR(2, 1) LNN_PAIR(2, 2) if (ANYPAIR) { LNN_PAIR(2, 0) } }
+  if (NTMAX >= 3) { LNN_PAIR(3, 2) LNN_PAIR(3, 3) if (ANYPAIR) { LNN_PAIR(3, 0) LNN_PAIR(3, 1) } }
+  if (NTMAX >= 4) { LNN_PAIR(4, 3) LNN_PAIR(4, 4) if (ANYPAIR) { LNN_PAIR(4, 0) LNN_PAIR(4, 1) LNN_PAIR(4, 2) } }
+#undef LNN_PAIR
 }
 
 // Sub-tile width policy for a remaining run of cnt units (at most MAXU per sub-tile).
@@ -924,8 +1022,39 @@ __device__ __forceinline__ void walk_units(const P& p, float* ldsA, float* ldsB,
     long long cnt = u1 - u0;
     if (cnt > n_units - un) cnt = n_units - un;
     const int nt = pick_units<2 * NTMAX>((int)cnt);
-    run_units<WM, NTMAX>(nt, p, ldsA, ldsB, strideA, strideB, mt * 32 * WM, un * 32 * WN);
+    const int nt0 = (nt + 1) >> 1, n0 = un * 32 * WN;
+    run_pair<WM, NTMAX, false>(nt0, nt - nt0, p, ldsA, ldsB, strideA, strideB, mt * 32 * WM, n0, n0 + 32 * WN * nt0);
     u0 += nt;
+  }
+}
+
+// Walk for column spaces made of segments of seg_units units (one segment per
+// convolution tap): a group's columns never cross a segment, the two groups
+// of a sub-tile may sit in different segments of the same M tile.
+// Units are numbered (mt * segs_per_mt + segment) * seg_units + unit; workgroup
+// b takes units [b*chunk, (b+1)*chunk).
+template <int WM, int NTMAX, class P>
+__device__ __forceinline__ void walk_units_seg(const P& p, float* ldsA, float* ldsB, int strideA, int strideB,
+                                               int seg_units, int segs_per_mt, int total_units, int chunk) {
+  constexpr int WN = 4 / WM;
+  const int per_mt = seg_units * segs_per_mt;
+  int pos = (int)blockIdx.x * chunk;
+  const int end = pos + chunk < total_units ? pos + chunk : total_units;
+  while (pos < end) {
+    const int mt = pos / per_mt;
+    int nt0 = seg_units - pos % seg_units;
+    if (nt0 > NTMAX) nt0 = NTMAX;
+    if (nt0 > end - pos) nt0 = end - pos;
+    const int p1 = pos + nt0;
+    int nt1 = 0;
+    if (p1 < end && p1 / per_mt == mt) {
+      nt1 = seg_units - p1 % seg_units;
+      if (nt1 > nt0) nt1 = nt0;
+      if (nt1 > end - p1) nt1 = end - p1;
+    }
+    run_pair<WM, NTMAX, true>(nt0, nt1, p, ldsA, ldsB, strideA, strideB, mt * 32 * WM, (pos - mt * per_mt) * 32 * WN,
+                              (p1 - mt * per_mt) * 32 * WN);
+    pos = p1 + nt1;
   }
 }
 

@@ -176,14 +176,17 @@ def test_conv_odd_corners_integer_exact(hip):
             assert np.array_equal(dw - off, rdw), ('dW', xs, ws)
 
 
-def test_conv_channel_multiples_of_16_integer_exact(hip):
-    """Channel counts that are multiples of 16 take the tap-major kernels
-    (permuted weights, address arithmetic in the scalar offset); everything
-    else about the geometry varies."""
+def test_conv_channel_multiples_of_32_integer_exact(hip):
+    """Channel counts that are multiples of 32 take the tap-major kernels
+    (forward / dgrad: permuted weights, address arithmetic in the scalar
+    offset; wgrad: pixel-major loaders with tap-major columns, for every tile
+    shape the output-channel count selects); everything else about the
+    geometry varies, and some pairs stay on the generic kernels."""
     rs = np.random.RandomState(11)
     cnt = 0
-    for (ic, oc), s, d, ks, padding in itertools.product([(16, 16), (32, 48), (48, 16), (16, 5), (6, 32)], [1, 2, 3],
-                                                         [1, 2], [1, 2, 3, 5], ['same', 'valid', 1]):
+    for (ic, oc), s, d, ks, padding in itertools.product([(16, 16), (32, 48), (48, 16), (16, 5), (6, 32), (32, 96),
+                                                          (64, 40), (128, 8), (64, 130), (96, 70), (160, 66)],
+                                                         [1, 2, 3], [1, 2], [1, 2, 3, 5], ['same', 'valid', 1]):
         n, h, w_ = 2, 11, 9
         if padding == 'valid' and min(h, w_) < (ks - 1) * d + 1:
             continue
@@ -200,7 +203,7 @@ def test_conv_channel_multiples_of_16_integer_exact(hip):
         assert np.array_equal(dx - 1.0, rdx), ('dX', tag)
         assert np.array_equal(dw - 1.0, rdw), ('dW', tag)
         cnt += 1
-    assert cnt > 250
+    assert cnt > 600
 
 
 # benchmark geometries at a reduced batch (the oracle materialises im2col in fp64)
