@@ -49,12 +49,31 @@ __global__ void build_ktable(KEntry* tab, int K, int Kpad, int mode, ConvGeom g)
   tab[k] = e;
 }
 
-__global__ void reduce_partials(float* out, const float* part, int n, int slices, int beta) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  float s = beta ? out[i] : 0.0f;
-  for (int k = 0; k < slices; ++k) s += part[(size_t)k * n + i];
-  out[i] = s;
+// out[f(i)] (+)= sum over slices of part[slice][i], slices added in a fixed order.
+// A block covers 32 consecutive i (one 128-byte line per slice row) with 8
+// lanes per i striding over the slices.  permute: partial column tap*C + c of
+// row m goes to out[m][c][tap] (tap-major wgrad columns back to OIHW).
+__global__ __launch_bounds__(256) void reduce_partials(float* out, const float* part, int n, int slices, int beta,
+                                                       int ncols, FastDiv dN, FastDiv dC, int KK, int permute) {
+  __shared__ float red[8][33];
+  const int li = threadIdx.x & 31, ls = threadIdx.x >> 5;
+  const int i = blockIdx.x * 32 + li;
+  float s = 0.0f;
+  if (i < n)
+    for (int k = ls; k < slices; k += 8) s += part[(size_t)k * n + i];
+  red[ls][li] = s;
+  __syncthreads();
+  if (ls == 0 && i < n) {
+#pragma unroll
+    for (int k = 1; k < 8; ++k) s += red[k][li];
+    uint32_t o = (uint32_t)i;
+    if (permute) {
+      const uint32_t m = dN.div(o), col = o - m * (uint32_t)ncols;
+      const uint32_t tap = dC.div(col), ch = col - tap * dC.d;
+      o = m * (uint32_t)ncols + ch * (uint32_t)KK + tap;
+    }
+    out[o] = beta ? out[o] + s : s;
+  }
 }
 
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
@@ -83,13 +102,14 @@ struct ConvCfg {
   static constexpr int SA = LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
   static constexpr int SB = LdsSize<PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP, BNMAX>::value;
+  static constexpr int STAGES = 2;   // 3 (fragments read ahead of the phase barrier) measured no faster
 };
 
 // Loader selection and initialisation per pass.  FLAG:
 //   PASS_FWD        128-bit loads of W rows (CKK % 4 == 0)
 //   PASS_DGRAD(_TAP) stride == 1
 //   PASS_WGRAD      128-bit loads of dY (OHW % 4 == 0)
-template <int PASS, bool FLAG>
+template <int PASS, bool FLAG, int ST>
 struct ConvProblem;
 
 struct ConvProblemBase {
@@ -100,44 +120,50 @@ struct ConvProblemBase {
   OutMap om;
 };
 
-template <bool FLAG>
-struct ConvProblem<PASS_FWD, FLAG> : ConvProblemBase {
+template <bool FLAG, int ST>
+struct ConvProblem<PASS_FWD, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
   template <int R> using LA = PlainKC<R, FLAG>;
   template <int R> using LB = ConvFwdB<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
-template <bool FLAG>
-struct ConvProblem<PASS_FWD_TAP, FLAG> : ConvProblemBase {
+template <bool FLAG, int ST>
+struct ConvProblem<PASS_FWD_TAP, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
   template <int R> using LA = PlainKC<R, true>;          // permuted weights [O][KK*C]
   template <int R> using LB = ConvFwdBTap<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, col0, Ncols, kbeg); }
 };
-template <bool FLAG>
-struct ConvProblem<PASS_DGRAD, FLAG> : ConvProblemBase {
+template <bool FLAG, int ST>
+struct ConvProblem<PASS_DGRAD, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
   template <int R> using LA = ConvDgradA<R>;
   template <int R> using LB = ConvDgradB<R, FLAG>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, tab, row0, kbeg); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
-template <bool FLAG>
-struct ConvProblem<PASS_DGRAD_TAP, FLAG> : ConvProblemBase {
+template <bool FLAG, int ST>
+struct ConvProblem<PASS_DGRAD_TAP, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
   template <int R> using LA = PlainKC<R, true>;          // permuted weights [C][KK*O]
   template <int R> using LB = ConvDgradBTap<R, FLAG>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, col0, Ncols, kbeg); }
 };
-template <bool FLAG>
-struct ConvProblem<PASS_WGRAD, FLAG> : ConvProblemBase {
+template <bool FLAG, int ST>
+struct ConvProblem<PASS_WGRAD, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
   template <int R> using LA = ConvWgradA<R, FLAG>;
   template <int R> using LB = ConvWgradB<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kend); }
 };
 
-template <bool FLAG>
-struct ConvProblem<PASS_WGRAD_TAP, FLAG> : ConvProblemBase {
+template <bool FLAG, int ST>
+struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
   template <int R> using LA = ConvWgradTapA<R>;
   template <int R> using LB = ConvWgradTapB<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend); }
@@ -147,8 +173,8 @@ struct ConvProblem<PASS_WGRAD_TAP, FLAG> : ConvProblemBase {
 template <int PASS, int WM, int NTMAX, bool FLAG>
 __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
   using Cfg = ConvCfg<PASS, WM, NTMAX, FLAG>;
-  __shared__ __attribute__((aligned(16))) float lds[2 * (Cfg::SA + Cfg::SB)];
-  ConvProblem<PASS, FLAG> p;
+  __shared__ __attribute__((aligned(16))) float lds[Cfg::STAGES * (Cfg::SA + Cfg::SB)];
+  ConvProblem<PASS, FLAG, Cfg::STAGES> p;
   p.g = a.g;
   p.tab = a.tab;
   p.rx = make_rsrc(a.X, a.bytesX);
@@ -170,17 +196,18 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
     p.om.nchw = 1; p.om.ld = a.g.OHW; p.om.mtot = a.g.O; p.om.dHW = a.g.dOHW;
   } else if (PASS == PASS_DGRAD || PASS == PASS_DGRAD_TAP) {
     p.om.nchw = 1; p.om.ld = a.g.IHW; p.om.mtot = a.g.C; p.om.dHW = a.g.dIHW;
-  } else if (PASS == PASS_WGRAD_TAP) {
-    // GEMM column tap*C + c lands in dW[o][c][tap]
+  } else if (PASS == PASS_WGRAD_TAP && a.ksplit <= 1) {
+    // GEMM column tap*C + c lands in dW[o][c][tap]; split-K partials stay in
+    // GEMM order (coalesced) and the slice reduction does this permutation
     p.om.nchw = 2; p.om.ld = a.Ncols; p.om.mtot = a.g.KK; p.om.dHW = a.dC;
   } else {
     p.om.nchw = 0; p.om.ld = a.Ncols; p.om.mtot = 0; p.om.dHW = FastDiv{0, 0, 1};
   }
   if (PASS == PASS_WGRAD_TAP)
-    walk_units_seg<WM, NTMAX>(p, lds, lds + 2 * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.g.KK, a.total_units,
+    walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.g.KK, a.total_units,
                               a.chunk_units);
   else
-    walk_units<WM, NTMAX>(p, lds, lds + 2 * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
+    walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
 }
 
 // ---------------------------------------------------------------------------
@@ -302,8 +329,10 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   LNN_HIP(hipGetLastError());
   if (ksplit > 1) {
     const int n = a.M * a.Ncols;
-    hipLaunchKernelGGL(reduce_partials, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, final_out,
-                       static_cast<const float*>(ctx->ws), n, ksplit, final_beta);
+    hipLaunchKernelGGL(reduce_partials, dim3((n + 31) / 32), dim3(256), 0, ctx->stream, final_out,
+                       static_cast<const float*>(ctx->ws), n, ksplit, final_beta, a.Ncols,
+                       make_fastdiv((uint32_t)a.Ncols), make_fastdiv((uint32_t)a.g.C), a.g.KK,
+                       PASS == PASS_WGRAD_TAP ? 1 : 0);
     LNN_HIP(hipGetLastError());
   }
   return LNN_OK;

@@ -23,12 +23,14 @@ struct GemmCfg {
   static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
   static constexpr int SA = LdsSize<!TA, BM>::value;
   static constexpr int SB = LdsSize<TB, BNMAX>::value;
+  static constexpr int STAGES = 2;   // 3 (fragments read ahead of the phase barrier) measured no faster
 };
 
 // A operand: !TA -> A[M][K] row-major, K-contiguous; TA -> stored [K][M].
 // B operand: !TB -> B[K][N], row(n)-contiguous;      TB -> stored [N][K].
-template <bool TA, bool TB, bool VEC>
+template <bool TA, bool TB, bool VEC, int ST>
 struct GemmProblem {
+  static constexpr int STAGES = ST;
   template <int R> using LA = typename std::conditional<TA, PlainMC<R, VEC>, PlainKC<R, VEC>>::type;
   template <int R> using LB = typename std::conditional<TB, PlainKC<R, VEC>, PlainMC<R, VEC>>::type;
   rsrc_t ra, rb, rc;
@@ -41,16 +43,16 @@ struct GemmProblem {
 template <int WM, int NTMAX, bool TA, bool TB, bool VEC>
 __global__ __launch_bounds__(512, 2) void gemm_kernel(GemmArgs a) {
   using Cfg = GemmCfg<WM, NTMAX, TA, TB, VEC>;
-  __shared__ __attribute__((aligned(16))) float lds[2 * (Cfg::SA + Cfg::SB)];
+  __shared__ __attribute__((aligned(16))) float lds[Cfg::STAGES * (Cfg::SA + Cfg::SB)];
   const long long b = blockIdx.y;
-  GemmProblem<TA, TB, VEC> p;
+  GemmProblem<TA, TB, VEC, Cfg::STAGES> p;
   p.ra = make_rsrc(a.A + b * a.sA, a.bytesA);
   p.rb = make_rsrc(a.B + b * a.sB, a.bytesB);
   p.rc = make_rsrc(a.C + b * a.sC, a.bytesC);
   p.lda = a.lda; p.ldb = a.ldb; p.M = a.M; p.Ncols = a.N; p.K = a.K;
   p.kbeg = 0; p.kend = a.K; p.beta = a.beta;
   p.om.nchw = 0; p.om.ld = a.ldc; p.om.mtot = 0; p.om.dHW = FastDiv{0, 0, 1};
-  walk_units<WM, NTMAX>(p, lds, lds + 2 * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
+  walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
 }
 
 template <int WM, int NTMAX, bool TA, bool TB>

@@ -821,27 +821,31 @@ __device__ __forceinline__ void load_frags(const float* __restrict__ As, const f
 }
 
 // One LDS stage = BK/8 groups of 4*NT MFMAs.  The fragments of the first
-// group are read up front; the reads of each following group are slotted one
-// by one between the MFMAs of the group before it, so the matrix pipe starts
-// after a single LDS latency and does not wait for LDS again within the stage.
-template <int NT, bool A_KC, bool B_KC, int RA, int RB>
+// group are either already in fa[0] / fb[0] (PRE: read before the phase barrier)
+// or read up front; the reads of each following group are slotted one by one
+// between the MFMAs of the group before it, so the matrix pipe does not wait
+// for LDS within the stage.
+template <int NT, bool A_KC, bool B_KC, int RA, int RB, bool PRE>
 __device__ __forceinline__ void mma_stage(const float* __restrict__ As, const float* __restrict__ Bs,
-                                          f32x16 (&acc)[NT], int arow, int brow) {
+                                          f32x16 (&acc)[NT], int arow, int brow, float (&fa)[2][4],
+                                          float (&fb)[2][NT][4]) {
   constexpr int NG = BK / 8;
+  static_assert(NG % 2 == 0, "the pre-loaded fragments live in buffer 0");
   // LDS read instructions per group: A is one b128 or four b32; B is NT b128 or 4*NT b32 (paired into read2)
   constexpr int RD = (A_KC ? 1 : 2) + (B_KC ? NT : 2 * NT);
-  float a[2][4], b[2][NT][4];   // fragment double buffer
-  load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, 0, a[0], b[0]);
-  __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);              // DS reads of group 0
+  if (!PRE) {
+    load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, 0, fa[0], fb[0]);
+    __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);              // DS reads of group 0
+  }
 #pragma unroll
   for (int kk = 0; kk < NG; ++kk) {
     const int cur = kk & 1;
-    if (kk + 1 < NG) load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, kk + 1, a[cur ^ 1], b[cur ^ 1]);
+    if (kk + 1 < NG) load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, kk + 1, fa[cur ^ 1], fb[cur ^ 1]);
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int j = 0; j < NT; ++j)
-        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][t], b[cur][j][t], acc[j], 0, 0, 0);
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][t], fb[cur][j][t], acc[j], 0, 0, 0);
     if (kk + 1 < NG) {
 #pragma unroll
       for (int i = 0; i < RD; ++i) {
@@ -885,61 +889,83 @@ __device__ __forceinline__ void fetch_b(LB& lb, int k0, const LA& la) {
 // Body of one group (G = 0 or 1) for one sub-tile: BM = 32*WM rows shared by
 // both groups, 32*WN*NT columns of its own starting at column offset COFF of
 // the sub-tile; BNTOT is the column count of both groups together.
+//
+// P::STAGES LDS stages.  With 2, K step t+1 is parked while step t is computed
+// and a compute phase starts by reading its first fragments.  With 3, step t+2
+// is parked during step t, so step t+1 is complete a whole step early and each
+// group reads the first fragments of its next compute phase *before* the
+// barrier that starts it: the matrix pipe restarts right at the barrier.
 template <int WM, int NT, int G, int COFF, int BNTOT, class P>
 __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB, int strideA, int strideB, int m0,
                                            int ng) {   // ng: first global column of this group
-  constexpr int WN = 4 / WM, BM = 32 * WM, HALF = BM / 2, BN = 32 * WN * (NT > 0 ? NT : 1);
+  constexpr int WN = 4 / WM, BM = 32 * WM, HALF = BM / 2, NTC = NT > 0 ? NT : 1, BN = 32 * WN * NTC;
+  constexpr int ST = P::STAGES;
+  constexpr bool PRE = ST == 3;
   using LA = typename P::template LA<HALF>;
   using LB = typename P::template LB<BN>;
   constexpr bool A_KC = LA::KC, B_KC = LB::KC;
   constexpr int LDA = A_KC ? LDK : BM, LDB = B_KC ? LDK : BNTOT;
   const int wave = gwave(), lane = threadIdx.x & 63;
   const int wm = wave % WM, wn = wave / WM;
+  const int arow = wm * 32, brow = COFF + wn * NT * 32;
   LA la;
   LB lb;
   p.template init_a<HALF>(la, m0 + G * HALF);
   if (NT > 0) p.template init_b<BN>(lb, ng, la);
-  f32x16 acc[NT > 0 ? NT : 1];
+  f32x16 acc[NTC];
+  float fa[2][4], fb[2][NTC][4];
 #pragma unroll
-  for (int j = 0; j < (NT > 0 ? NT : 1); ++j)
+  for (int j = 0; j < NTC; ++j)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
 
   const int kbeg = p.kbeg;
   const int nk = (p.kend - kbeg + BK - 1) / BK;
-  // prologue: K step 0 into stage 0, K step 1 into registers
-  if (nk > 0) {
-    la.fetch(kbeg);
-    if (NT > 0) fetch_b(lb, kbeg, la);
-    la.commit(ldsA, LDA, G * HALF);
-    if (NT > 0) lb.commit(ldsB, LDB, COFF);
-  }
-  if (nk > 1) {
-    la.fetch(kbeg + BK);
-    if (NT > 0) fetch_b(lb, kbeg + BK, la);
+  // prologue: K steps 0 .. ST-2 into their stages, step ST-1 into registers
+#pragma unroll
+  for (int q = 0; q < ST - 1; ++q)
+    if (q < nk) {
+      la.fetch(kbeg + q * BK);
+      if (NT > 0) fetch_b(lb, kbeg + q * BK, la);
+      la.commit(ldsA + q * strideA, LDA, G * HALF);
+      if (NT > 0) lb.commit(ldsB + q * strideB, LDB, COFF);
+    }
+  if (ST - 1 < nk) {
+    la.fetch(kbeg + (ST - 1) * BK);
+    if (NT > 0) fetch_b(lb, kbeg + (ST - 1) * BK, la);
   }
   __syncthreads();
+  if (PRE && G == 0 && NT > 0 && nk > 0)
+    load_frags<NTC, A_KC, B_KC, BM, BNTOT>(ldsA, ldsB, arow, brow, 0, fa[0], fb[0]);
+
   // Each K step t has two phases separated by barriers.  Group 0 computes in
   // the first and moves data in the second; group 1 the other way round.
-  // "Moving data" for step t = park K step t+1 (fetched one step earlier) in
-  // the other LDS stage, then fetch K step t+2 into registers.  Stage (t+1)&1
-  // was last read for step t-1, which both groups finished before this step.
+  // "Moving data" in step t = park K step t+ST-1 (fetched one step earlier) in
+  // its stage, which was last read for step t-1, then fetch K step t+ST.
+  int cur = 0;        // stage of K step t
   for (int t = 0; t < nk; ++t) {
-    const int cur = t & 1;
+    const int park = cur == 0 ? ST - 1 : cur - 1;           // stage of K step t+ST-1 == stage of step t-1
+    const int nxt = cur + 1 == ST ? 0 : cur + 1;            // stage of K step t+1
 #pragma unroll
     for (int phase = 0; phase < 2; ++phase) {
       if (phase == G) {
         if (NT > 0)
-          mma_stage<(NT > 0 ? NT : 1), A_KC, B_KC, BM, BNTOT>(ldsA + cur * strideA, ldsB + cur * strideB, acc, wm * 32,
-                                                            COFF + wn * NT * 32);
+          mma_stage<NTC, A_KC, B_KC, BM, BNTOT, PRE>(ldsA + cur * strideA, ldsB + cur * strideB, acc, arow, brow, fa, fb);
       } else {
-        if (t + 1 < nk) {
-          la.commit(ldsA + (cur ^ 1) * strideA, LDA, G * HALF);
-          if (NT > 0) lb.commit(ldsB + (cur ^ 1) * strideB, LDB, COFF);
+        if (t + ST - 1 < nk) {
+          la.commit(ldsA + park * strideA, LDA, G * HALF);
+          if (NT > 0) lb.commit(ldsB + park * strideB, LDB, COFF);
         }
-        if (t + 2 < nk) {
-          la.fetch(kbeg + (t + 2) * BK);
-          if (NT > 0) fetch_b(lb, kbeg + (t + 2) * BK, la);
+        if (t + ST < nk) {
+          la.fetch(kbeg + (t + ST) * BK);
+          if (NT > 0) fetch_b(lb, kbeg + (t + ST) * BK, la);
+        }
+        if (PRE && NT > 0) {
+          // first fragments of this group's next compute phase: group 0 computes
+          // step t+1 next, group 1 computes step t in the coming phase
+          const int st = G == 0 ? nxt : cur;
+          if (G == 1 || t + 1 < nk)
+            load_frags<NTC, A_KC, B_KC, BM, BNTOT>(ldsA + st * strideA, ldsB + st * strideB, arow, brow, 0, fa[0], fb[0]);
         }
       }
       // the phase ends only when all of its MFMAs have been issued: do not let
@@ -948,23 +974,47 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
       __syncthreads();
       __builtin_amdgcn_sched_barrier(0);
     }
+    cur = nxt;
   }
 
   // epilogue: acc[j][r] is C[m0 + wm*32 + 8*(r/4) + 4*(lane/32) + r%4][ng + (wn*NT + j)*32 + lane%32]
   if (NT > 0) {
     const int i = lane & 31, h = lane >> 5;
+    uint32_t roff[16];   // row part of the element offset, OOB for rows past M
 #pragma unroll
-    for (int j = 0; j < (NT > 0 ? NT : 1); ++j) {
+    for (int r = 0; r < 16; ++r) {
+      const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+      roff[r] = m < p.M ? (uint32_t)(m * p.om.ld) : OOB;
+    }
+    auto col_off = [&](int j) -> uint32_t {
       const int n = ng + (wn * NT + j) * 32 + i;
-      const bool nok = n < p.Ncols;
-      const uint32_t cb = p.om.col(nok ? (uint32_t)n : 0u);
+      return n < p.Ncols ? p.om.col((uint32_t)n) : OOB;
+    };
+    auto elem = [](uint32_t cb, uint32_t ro) -> uint32_t { return ((cb | ro) & OOB) ? OOB : (cb + ro) * 4u; };
+    if (p.beta) {
+      // accumulate: the old values of fragment j+1 are in flight while fragment j is added and stored
+      float old[2][16];
+      uint32_t cb = col_off(0);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-        const uint32_t off = (nok && m < p.M) ? (cb + (uint32_t)(m * p.om.ld)) * 4u : OOB;
-        float val = acc[j][r];
-        if (p.beta) val += buf_load(p.rc, off);
-        buf_store(p.rc, off, val);
+      for (int r = 0; r < 16; ++r) old[0][r] = buf_load(p.rc, elem(cb, roff[r]));
+#pragma unroll
+      for (int j = 0; j < NTC; ++j) {
+        uint32_t cbn = 0;
+        if (j + 1 < NTC) {
+          cbn = col_off(j + 1);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) old[(j + 1) & 1][r] = buf_load(p.rc, elem(cbn, roff[r]));
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) buf_store(p.rc, elem(cb, roff[r]), acc[j][r] + old[j & 1][r]);
+        cb = cbn;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NTC; ++j) {
+        const uint32_t cb = col_off(j);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) buf_store(p.rc, elem(cb, roff[r]), acc[j][r]);
       }
     }
   }
