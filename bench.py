@@ -245,7 +245,10 @@ def bench_matmul(api, steps, warmup, n=4096, cpu=True):
 def bench_encoder(steps, warmup):
     """cfg5: full training step (forward, backward, SGD) of the 4-layer 5x5
     stride-2 encoder through the litenn-compatible Python API."""
-    import litenn_amd as nn
+    import contextlib
+    with contextlib.redirect_stdout(sys.stderr):   # the device banner must not share stdout with the JSON line
+        import litenn_amd as nn
+        nn.devices.get_current()
     rs = np.random.RandomState(0)
     x_n = rs.uniform(-1, 1, (16, 3, 128, 128)).astype(np.float32)
     chans = [3, 64, 128, 256, 512]

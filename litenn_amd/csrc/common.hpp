@@ -22,7 +22,7 @@ struct DeviceCtx {
   void* ws = nullptr;
   size_t ws_bytes = 0;
   // gather tables, one per (geometry, kind)
-  std::map<std::array<int, 12>, KEntry*> tables;
+  std::map<std::array<int, 16>, KEntry*> tables;
 };
 
 int set_error(int code, const std::string& msg);

@@ -22,29 +22,49 @@ struct ConvArgs {
   int ksplit;        // wgrad: number of K slices (gridDim.y)
   FastDiv dC;        // tap-major wgrad: divide a column index by the channel count
   int chunk_units;   // tap-major wgrad: units per workgroup
+  // dgrad: g describes one pixel class (g.IH, g.IW = class grid); the plane it is cut from:
+  int full_IW, full_IHW, cls_org, cls_s;
 };
 
-// mode 0: k = (c, kh, kw) for forward / wgrad; mode 1: k = (o, kh, kw) for dgrad.
-__global__ void build_ktable(KEntry* tab, int K, int Kpad, int mode, ConvGeom g) {
+// One class of input pixels of a strided dgrad: pixels (h0 + S*i, w0 + S*j),
+// fed by the taps with kh*D = rh (mod S) and kw*D = rw (mod S).
+struct PixelClass {
+  int rh, rw, h0, w0, nkh, nkw;
+};
+// the j-th k in [0, n) with k*D = r (mod S)
+__host__ __device__ inline int nth_tap(int n, int D, int S, int r, int j) {
+  for (int k = 0; k < n; ++k)
+    if (k * D % S == r && j-- == 0) return k;
+  return -1;
+}
+
+// mode 0: k = (c, kh, kw) for forward / wgrad.
+// mode 1: dgrad, k = (o, tap of the class); mode 2: dgrad, one entry per tap of the class (tap-major K).
+__global__ void build_ktable(KEntry* tab, int K, int Kpad, int mode, ConvGeom g, PixelClass pc) {
   const int k = blockIdx.x * blockDim.x + threadIdx.x;
   if (k >= Kpad) return;
   KEntry e;
+  e.x = 0;
+  e.y = BIG;
+  e.z = 0;
+  e.w = 0x20000000;
   if (k < K) {
-    const int ch = k / g.KK, tap = k - ch * g.KK, kh = tap / g.KW, kw = tap - kh * g.KW;
-    e.y = kh * g.D;
-    e.z = kw * g.D;
     if (mode == 0) {
+      const int ch = k / g.KK, tap = k - ch * g.KK, kh = tap / g.KW, kw = tap - kh * g.KW;
+      e.y = kh * g.D;
+      e.z = kw * g.D;
       e.x = ch * g.IHW + kh * g.D * g.IW + kw * g.D;
       e.w = 0;
     } else {
+      const int nt = pc.nkh * pc.nkw;
+      const int ch = mode == 1 ? k / nt : 0, t = mode == 1 ? k - ch * nt : k;
+      const int jh = t / pc.nkw, jw = t - jh * pc.nkw;
+      const int kh = nth_tap(g.KH, g.D, g.S, pc.rh, jh), kw = nth_tap(g.KW, g.D, g.S, pc.rw, jw);
+      e.y = (kh * g.D - g.PADT - pc.h0) / g.S;   // exact by the definition of the class
+      e.z = (kw * g.D - g.PADL - pc.w0) / g.S;
       e.x = ch * g.OHW;
-      e.w = ch * g.C * g.KK + tap;
+      e.w = ch * g.C * g.KK + kh * g.KW + kw;
     }
-  } else {
-    e.x = 0;
-    e.y = BIG;
-    e.z = 0;
-    e.w = 0x20000000;
   }
   tab[k] = e;
 }
@@ -81,16 +101,19 @@ enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRA
 
 // Wp[a][tap][b] = W[..] so that the tap-major K index tap*CH + ch is contiguous:
 //   mode 0 (forward): Wp[o][tap][c] = W[o][c][tap]
-//   mode 1 (dgrad):   Wp[c][tap][o] = W[o][c][tap]
-__global__ void permute_weights(float* wp, const float* w, int O, int C, int KK, int mode) {
+//   mode 1 (dgrad):   Wp[c][t][o] = W[o][c][tap_t], t over the taps of the pixel class
+__global__ void permute_weights(float* wp, const float* w, int O, int C, int KK, int mode, ConvGeom g, PixelClass pc) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= O * C * KK) return;
-  int a, tap, b;
   if (mode == 0) {
-    b = i % C; tap = (i / C) % KK; a = i / (C * KK);
+    if (i >= O * C * KK) return;
+    const int b = i % C, tap = (i / C) % KK, a = i / (C * KK);
     wp[i] = w[((size_t)a * C + b) * KK + tap];
   } else {
-    b = i % O; tap = (i / O) % KK; a = i / (O * KK);
+    const int nt = pc.nkh * pc.nkw;
+    if (i >= O * C * nt) return;
+    const int b = i % O, t = (i / O) % nt, a = i / (O * nt);
+    const int jh = t / pc.nkw, jw = t - jh * pc.nkw;
+    const int tap = nth_tap(g.KH, g.D, g.S, pc.rh, jh) * g.KW + nth_tap(g.KW, g.D, g.S, pc.rw, jw);
     wp[i] = w[((size_t)b * C + a) * KK + tap];
   }
 }
@@ -107,7 +130,6 @@ struct ConvCfg {
 
 // Loader selection and initialisation per pass.  FLAG:
 //   PASS_FWD        128-bit loads of W rows (CKK % 4 == 0)
-//   PASS_DGRAD(_TAP) stride == 1
 //   PASS_WGRAD      128-bit loads of dY (OHW % 4 == 0)
 template <int PASS, bool FLAG, int ST>
 struct ConvProblem;
@@ -140,7 +162,7 @@ template <bool FLAG, int ST>
 struct ConvProblem<PASS_DGRAD, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = ConvDgradA<R>;
-  template <int R> using LB = ConvDgradB<R, FLAG>;
+  template <int R> using LB = ConvDgradB<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, tab, row0, kbeg); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
@@ -148,9 +170,9 @@ template <bool FLAG, int ST>
 struct ConvProblem<PASS_DGRAD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = PlainKC<R, true>;          // permuted weights [C][KK*O]
-  template <int R> using LB = ConvDgradBTap<R, FLAG>;
+  template <int R> using LB = ConvDgradBTap<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
-  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, col0, Ncols, kbeg); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD, FLAG, ST> : ConvProblemBase {
@@ -195,7 +217,8 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
   if (PASS == PASS_FWD || PASS == PASS_FWD_TAP) {
     p.om.nchw = 1; p.om.ld = a.g.OHW; p.om.mtot = a.g.O; p.om.dHW = a.g.dOHW;
   } else if (PASS == PASS_DGRAD || PASS == PASS_DGRAD_TAP) {
-    p.om.nchw = 1; p.om.ld = a.g.IHW; p.om.mtot = a.g.C; p.om.dHW = a.g.dIHW;
+    p.om.nchw = 3; p.om.ld = a.full_IHW; p.om.mtot = a.g.C; p.om.dHW = a.g.dIHW;
+    p.om.dCW = a.g.dIW; p.om.s = a.cls_s; p.om.iw = a.full_IW; p.om.org = a.cls_org;
   } else if (PASS == PASS_WGRAD_TAP && a.ksplit <= 1) {
     // GEMM column tap*C + c lands in dW[o][c][tap]; split-K partials stay in
     // GEMM order (coalesced) and the slice reduction does this permutation
@@ -237,10 +260,14 @@ static int fill_geom(const lnn_conv2d_desc* d, ConvGeom& g) {
   return LNN_OK;
 }
 
-static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const KEntry** out) {
-  const int K = (mode == 0 ? g.C : g.O) * g.KK;
-  const int Kpad = ((K + BK - 1) / BK) * BK + BK;
-  const std::array<int, 12> key = {mode, g.C, g.O, g.KH, g.KW, g.D, g.IH, g.IW, g.OH, g.OW, 0, 0};
+// mode 0: forward / wgrad table; 1, 2: dgrad tables of pixel class pc (per k / per tap)
+static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const PixelClass& pc, const KEntry** out) {
+  const int nt = pc.nkh * pc.nkw;
+  const int K = mode == 0 ? g.C * g.KK : (mode == 1 ? g.O * nt : nt);
+  // readers prefetch one K step (mode 2: one tap) past the end
+  const int Kpad = mode == 2 ? K + 2 : ((K + BK - 1) / BK) * BK + BK;
+  const std::array<int, 16> key = {mode, g.C,  g.O,  g.KH, g.KW,   g.D,    g.IH,  g.IW,
+                                   g.OH, g.OW, g.S, g.PADT, g.PADL, pc.rh, pc.rw, 0};
   auto it = ctx->tables.find(key);
   if (it != ctx->tables.end()) {
     *out = it->second;
@@ -258,7 +285,7 @@ static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const KEntry**
     return set_error(LNN_ERR_OOM, "conv2d: out of device memory for the gather table");
   }
   LNN_HIP(e);
-  hipLaunchKernelGGL(build_ktable, dim3((Kpad + 255) / 256), dim3(256), 0, ctx->stream, tab, K, Kpad, mode, g);
+  hipLaunchKernelGGL(build_ktable, dim3((Kpad + 255) / 256), dim3(256), 0, ctx->stream, tab, K, Kpad, mode, g, pc);
   LNN_HIP(hipGetLastError());
   ctx->tables[key] = tab;
   *out = tab;
@@ -267,13 +294,16 @@ static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const KEntry**
 
 // Channel-permuted copy of the weights in the library's scratch buffer (valid
 // until the next call that uses scratch; the stream orders it before its reader).
-static int permuted_weights(DeviceCtx* ctx, const ConvGeom& g, const float* W, int mode, const float** out) {
-  const int n = g.O * g.C * g.KK;
-  int st = ensure_workspace(ctx, (size_t)n * sizeof(float));
+static int permuted_weights(DeviceCtx* ctx, const ConvGeom& g, const float* W, int mode, const PixelClass& pc,
+                            const float** out) {
+  const int n = g.O * g.C * (mode == 0 ? g.KK : pc.nkh * pc.nkw);
+  int st = ensure_workspace(ctx, (size_t)(n > 0 ? n : 1) * sizeof(float));
   if (st != LNN_OK) return st;
-  hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, static_cast<float*>(ctx->ws), W,
-                     g.O, g.C, g.KK, mode);
-  LNN_HIP(hipGetLastError());
+  if (n > 0) {
+    hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream,
+                       static_cast<float*>(ctx->ws), W, g.O, g.C, g.KK, mode, g, pc);
+    LNN_HIP(hipGetLastError());
+  }
   *out = static_cast<const float*>(ctx->ws);
   return LNN_OK;
 }
@@ -322,10 +352,12 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   }
   a.ksplit = ksplit;
   dim3 g(grid, ksplit, 1), b(512, 1, 1);
-  if (flag)
+  constexpr bool kUsesFlag = PASS == PASS_FWD || PASS == PASS_WGRAD;   // the other passes have one variant
+  if (flag || !kUsesFlag) {
     hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, true>), g, b, 0, ctx->stream, a);
-  else
+  } else if constexpr (kUsesFlag) {
     hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, false>), g, b, 0, ctx->stream, a);
+  }
   LNN_HIP(hipGetLastError());
   if (ksplit > 1) {
     const int n = a.M * a.Ncols;
@@ -361,36 +393,64 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   a.M = g.O; a.Ncols = g.N * g.OHW; a.K = g.C * g.KK;
   a.beta = beta ? 1 : 0;
   if (g.C % BK == 0) {
-    st = permuted_weights(ctx, g, W, 0, &a.W);
+    st = permuted_weights(ctx, g, W, 0, PixelClass{}, &a.W);
     if (st != LNN_OK) return st;
     return launch_by_m<PASS_FWD_TAP>(ctx, a, true);
   }
-  st = get_table(ctx, a.g, 0, &a.tab);
+  st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);
   if (st != LNN_OK) return st;
   return launch_by_m<PASS_FWD>(ctx, a, a.K % 4 == 0 && aligned16(W));
 }
 
 int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta) {
-  ConvArgs a;
-  int st = fill_geom(d, a.g);
+  ConvGeom full;
+  int st = fill_geom(d, full);
   if (st != LNN_OK) return st;
   if (!dY || !W || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
-  a.tab = nullptr;
-  const ConvGeom& g = a.g;
-  a.X = dY; a.W = W; a.Out = dX;
-  a.bytesX = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
-  a.bytesW = (uint32_t)((uint64_t)g.O * g.C * g.KK * 4);
-  a.bytesOut = (uint32_t)((uint64_t)g.N * g.C * g.IHW * 4);
-  a.M = g.C; a.Ncols = g.N * g.IHW; a.K = g.O * g.KK;
-  a.beta = beta ? 1 : 0;
-  if (g.O % BK == 0) {
-    st = permuted_weights(ctx, g, W, 1, &a.W);
-    if (st != LNN_OK) return st;
-    return launch_by_m<PASS_DGRAD_TAP>(ctx, a, g.S == 1);
-  }
-  st = get_table(ctx, a.g, 1, &a.tab);
-  if (st != LNN_OK) return st;
-  return launch_by_m<PASS_DGRAD>(ctx, a, g.S == 1);
+  const int S = full.S;
+  // one stride-1 problem per class of input pixels (see ConvDgradB)
+  for (int rh = 0; rh < S; ++rh)
+    for (int rw = 0; rw < S; ++rw) {
+      PixelClass pc;
+      pc.rh = rh; pc.rw = rw;
+      pc.h0 = ((rh - full.PADT) % S + S) % S;
+      pc.w0 = ((rw - full.PADL) % S + S) % S;
+      if (pc.h0 >= full.IH || pc.w0 >= full.IW) continue;   // no such pixels
+      pc.nkh = pc.nkw = 0;
+      for (int k = 0; k < full.KH; ++k) pc.nkh += k * full.D % S == rh;
+      for (int k = 0; k < full.KW; ++k) pc.nkw += k * full.D % S == rw;
+      const int nt = pc.nkh * pc.nkw;
+      if (nt == 0 && beta) continue;                        // nothing to add; without beta the class is zero-filled
+      ConvArgs a;
+      a.g = full;
+      ConvGeom& g = a.g;
+      g.IH = (full.IH - pc.h0 + S - 1) / S;
+      g.IW = (full.IW - pc.w0 + S - 1) / S;
+      g.IHW = g.IH * g.IW;
+      g.dIW = make_fastdiv(g.IW); g.dIHW = make_fastdiv(g.IHW);
+      a.full_IW = full.IW; a.full_IHW = full.IHW; a.cls_s = S; a.cls_org = pc.h0 * full.IW + pc.w0;
+      a.tab = nullptr;
+      a.X = dY; a.W = W; a.Out = dX;
+      a.bytesX = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
+      a.bytesW = (uint32_t)((uint64_t)g.O * g.C * g.KK * 4);
+      a.bytesOut = (uint32_t)((uint64_t)g.N * g.C * full.IHW * 4);
+      a.M = g.C; a.Ncols = g.N * g.IHW; a.K = g.O * nt;
+      a.beta = beta ? 1 : 0;
+      if (g.O % BK == 0) {
+        st = permuted_weights(ctx, full, W, 1, pc, &a.W);
+        if (st != LNN_OK) return st;
+        a.bytesW = (uint32_t)((uint64_t)g.O * g.C * nt * 4);
+        st = get_table(ctx, full, 2, pc, &a.tab);
+        if (st != LNN_OK) return st;
+        st = launch_by_m<PASS_DGRAD_TAP>(ctx, a, true);
+      } else {
+        st = get_table(ctx, full, 1, pc, &a.tab);
+        if (st != LNN_OK) return st;
+        st = launch_by_m<PASS_DGRAD>(ctx, a, true);
+      }
+      if (st != LNN_OK) return st;
+    }
+  return LNN_OK;
 }
 
 int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
@@ -398,7 +458,7 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");
-  st = get_table(ctx, a.g, 0, &a.tab);
+  st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);
   if (st != LNN_OK) return st;
   const ConvGeom& g = a.g;
   a.X = X; a.W = dY; a.Out = dW;

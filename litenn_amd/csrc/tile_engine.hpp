@@ -369,44 +369,34 @@ struct ConvFwdBTap {
   }
 };
 
-template <int R, bool STRIDE1>
+template <int R>
 struct ConvDgradBTap {
   static constexpr bool KC = false;
   static constexpr int CC = (R + 63) / 64;
   rsrc_t rs;
-  int OH, OW, OHW, O, S, D, KW;
-  FastDiv dS;
+  ktab_t tab;           // one entry per tap of the pixel class: y, z (see ConvDgradB)
+  int OH, OW, OHW, O;
   int base[CC], a0[CC], b0[CC];
   uint32_t voff[CC];
-  int o0, kh, kw;
-  float v[KR][CC];
+  int o0, tap;          // K position of the next fetch
+  int cy, cz, ny, nz;   // (y, z) of the current tap and of the one after it
   __device__ __forceinline__ void set_tap() {
-    const int dh = kh * D, dw = kw * D;
 #pragma unroll
     for (int c = 0; c < CC; ++c) {
-      const int nh = a0[c] - dh, nw = b0[c] - dw;
-      bool ok;
-      int oh, ow;
-      if (STRIDE1) {
-        oh = nh;
-        ow = nw;
-        ok = (uint32_t)nh < (uint32_t)OH && (uint32_t)nw < (uint32_t)OW;
-      } else {
-        oh = (int)dS.div((uint32_t)nh & 0x7fffffffu);
-        ow = (int)dS.div((uint32_t)nw & 0x7fffffffu);
-        ok = nh >= 0 && nw >= 0 && oh * S == nh && ow * S == nw && oh < OH && ow < OW;
-      }
+      const int oh = a0[c] - cy, ow = b0[c] - cz;
+      const bool ok = (uint32_t)oh < (uint32_t)OH && (uint32_t)ow < (uint32_t)OW;
       voff[c] = ok ? (uint32_t)(base[c] + oh * OW + ow) * 4u : OOB;
     }
   }
-  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int p0, int P, int kbeg) {
+  float v[KR][CC];
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P, int kbeg) {
     rs = r;
-    OH = g.OH; OW = g.OW; OHW = g.OHW; O = g.O; S = g.S; D = g.D; KW = g.KW;
-    dS = g.dS;
-    const int tap = kbeg / g.O;
+    tab = as_ktab(tab_);
+    OH = g.OH; OW = g.OW; OHW = g.OHW; O = g.O;
+    tap = kbeg / g.O;
     o0 = kbeg - tap * g.O;
-    kh = tap / g.KW;
-    kw = tap - kh * g.KW;
+    cy = (tab + tap)->y; cz = (tab + tap)->z;
+    ny = (tab + tap + 1)->y; nz = (tab + tap + 1)->z;
     const int lane = threadIdx.x & 63;
 #pragma unroll
     for (int c = 0; c < CC; ++c) {
@@ -415,8 +405,8 @@ struct ConvDgradBTap {
       const uint32_t pp = ok ? (uint32_t)p : 0u;
       const uint32_t img = g.dIHW.div(pp), rem = pp - img * g.IHW;
       const uint32_t ih = g.dIW.div(rem), iw = rem - ih * g.IW;
-      a0[c] = (int)ih + g.PADT;
-      b0[c] = ok ? (int)iw + g.PADL : -BIG;
+      a0[c] = (int)ih;
+      b0[c] = ok ? (int)iw : -BIG;
       base[c] = (int)img * g.O * g.OHW;
     }
     set_tap();
@@ -432,9 +422,10 @@ struct ConvDgradBTap {
     o0 += BK;
     if (o0 >= O) {   // wave-uniform: next tap
       o0 = 0;
-      ++kw;
-      if (kw == KW) { kw = 0; ++kh; }
+      ++tap;
+      cy = ny; cz = nz;
       set_tap();
+      ny = (tab + tap + 1)->y; nz = (tab + tap + 1)->z;
     }
   }
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
@@ -447,17 +438,22 @@ struct ConvDgradBTap {
   }
 };
 
-// dgrad gather of dY: element (input pixel (n, ih, iw), k = (o, kh, kw)) =
-// dY[n, o, (ih+PT-kh*D)/S, (iw+PL-kw*D)/S] when both quotients are exact and
-// in range, else 0.
-template <int R, bool STRIDE1>
+// dgrad gather of dY.  A strided convolution is handled as S*S independent
+// stride-1 problems, one per class of input pixels with equal
+// ((ih + PT) mod S, (iw + PL) mod S): inside a class only the taps with
+// kh*D = (ih + PT) (mod S) contribute, and for those
+//   oh = (ih + PT - kh*D) / S = ihc - y,   ih = h0 + S*ihc,  y = (kh*D - PT - h0) / S
+// exactly (likewise ow = iwc - z).  The geometry handed to the loader is that
+// of the class (IH, IW = class grid) and the table lists the class's taps:
+// element (class pixel (n, ihc, iwc), k = (o, tap)) = dY[n, o, ihc - y, iwc - z]
+// when in range, else 0.  Stride 1 is the single class h0 = w0 = 0.
+template <int R>
 struct ConvDgradB {
   static constexpr bool KC = false;
   static constexpr int CC = (R + 63) / 64;
   rsrc_t rs;
   ktab_t tab;
-  int OH, OW, S;
-  FastDiv dS;
+  int OH, OW;
   int base[CC], a0[CC], b0[CC];
   int tx[KR], ty[KR], tz[KR];
   float v[KR][CC];
@@ -475,8 +471,6 @@ struct ConvDgradB {
     load_entries(kbeg);
     OH = g.OH;
     OW = g.OW;
-    S = g.S;
-    dS = g.dS;
     const int lane = threadIdx.x & 63;
 #pragma unroll
     for (int c = 0; c < CC; ++c) {
@@ -485,8 +479,8 @@ struct ConvDgradB {
       const uint32_t pp = ok ? (uint32_t)p : 0u;
       const uint32_t img = g.dIHW.div(pp), rem = pp - img * g.IHW;
       const uint32_t ih = g.dIW.div(rem), iw = rem - ih * g.IW;
-      a0[c] = (int)ih + g.PADT;
-      b0[c] = ok ? (int)iw + g.PADL : -BIG;
+      a0[c] = (int)ih;
+      b0[c] = ok ? (int)iw : -BIG;
       base[c] = (int)img * g.O * g.OHW;
     }
   }
@@ -496,18 +490,8 @@ struct ConvDgradB {
       const int t_x = tx[e];
 #pragma unroll
       for (int c = 0; c < CC; ++c) {
-        const int nh = a0[c] - ty[e], nw = b0[c] - tz[e];
-        bool ok;
-        int oh, ow;
-        if (STRIDE1) {
-          oh = nh;
-          ow = nw;
-          ok = (uint32_t)nh < (uint32_t)OH && (uint32_t)nw < (uint32_t)OW;
-        } else {
-          oh = (int)dS.div((uint32_t)nh & 0x7fffffffu);
-          ow = (int)dS.div((uint32_t)nw & 0x7fffffffu);
-          ok = nh >= 0 && nw >= 0 && oh * S == nh && ow * S == nw && oh < OH && ow < OW;
-        }
+        const int oh = a0[c] - ty[e], ow = b0[c] - tz[e];
+        const bool ok = (uint32_t)oh < (uint32_t)OH && (uint32_t)ow < (uint32_t)OW;
         v[e][c] = buf_load(rs, ok ? (uint32_t)(base[c] + t_x + oh * OW + ow) * 4u : OOB);
       }
     }
@@ -778,15 +762,20 @@ struct ConvWgradTapB {
 // column n = (img, pixel): off = (img*Mtot + m)*HW + pixel.
 // ---------------------------------------------------------------------------
 struct OutMap {
-  int nchw;    // 0 plain, 1 image layout, 2 tap-major weight columns
+  int nchw;    // 0 plain, 1 image layout, 2 tap-major weight columns, 3 strided pixel class of an image layout
   int ld;      // plain / tap-major: leading dimension; nchw: HW
   int mtot;    // nchw: channel count; tap-major: KK
-  FastDiv dHW; // nchw: divide by HW; tap-major: divide by the channel count C
+  FastDiv dHW; // nchw: divide by HW (class: by the class plane); tap-major: divide by the channel count C
+  // class: column (img, ihc, iwc) is pixel (h0 + s*ihc, w0 + s*iwc) of a plane of width iw; org = h0*iw + w0
+  FastDiv dCW;
+  int s, iw, org;
   __device__ __forceinline__ uint32_t col(uint32_t n) const {
     if (nchw == 0) return n;
     const uint32_t q = dHW.div(n);
     if (nchw == 1) return q * (uint32_t)(mtot * ld) + (n - q * ld);   // q = image
-    return (n - q * dHW.d) * (uint32_t)mtot + q;                      // q = tap: column tap*C + c -> c*KK + tap
+    if (nchw == 2) return (n - q * dHW.d) * (uint32_t)mtot + q;       // q = tap: column tap*C + c -> c*KK + tap
+    const uint32_t rem = n - q * dHW.d, r = dCW.div(rem), c = rem - r * dCW.d;
+    return q * (uint32_t)(mtot * ld) + (uint32_t)org + (r * (uint32_t)iw + c) * (uint32_t)s;
   }
 };
 

@@ -176,6 +176,43 @@ def test_conv_odd_corners_integer_exact(hip):
             assert np.array_equal(dw - off, rdw), ('dW', xs, ws)
 
 
+def test_conv_strided_dgrad_pixel_classes_integer_exact(hip):
+    """dX of a strided convolution is computed per class of input pixels
+    ((ih + PADT) mod S, (iw + PADL) mod S).  Sweep strides against dilations
+    and kernel sizes so that classes with no tap, with no pixel, with one tap
+    and with uneven tap counts all occur, on the table-driven path (odd
+    channel counts) and on the tap-major path (O a multiple of 32), with and
+    without accumulation into a prefilled dX."""
+    rs = np.random.RandomState(11)
+    cnt = 0
+    for s in (2, 3, 4):
+        for d in (1, 2, 3):
+            for k in (1, 2, 3, 5):
+                for padding in ('same', 'valid', 1, (2, 0, 1, 3)):
+                    for (C, O) in ((3, 5), (6, 32), (33, 64)):
+                        H, W_ = 11 + s, 9 + 2 * s
+                        try:
+                            ci = info_conv2d(H, W_, k, k + (s == 3), s, d, padding)
+                        except ValueError:
+                            continue
+                        if ci.OH <= 0 or ci.OW <= 0:
+                            continue
+                        xs, ws = (2, C, H, W_), (O, C, k, k + (s == 3))
+                        say(f'conv classes x={xs} w={ws} s={s} d={d} pad={padding}')
+                        x = rs.randint(5, size=xs).astype(np.float32)
+                        w = rs.randint(5, size=ws).astype(np.float32)
+                        dy = rs.randint(5, size=(xs[0], O, ci.OH, ci.OW)).astype(np.float32)
+                        ry, rdx, rdw = conv2d_all(x, w, dy, s, d, padding)
+                        prefill = None if cnt % 2 else 3.0
+                        y, dx, dw = _run_conv(hip, x, w, dy, s, d, padding, prefill=prefill)
+                        off = 0.0 if prefill is None else prefill
+                        assert np.array_equal(y, ry), ('fwd', xs, ws, s, d, padding)
+                        assert np.array_equal(dx - off, rdx), ('dX', xs, ws, s, d, padding)
+                        assert np.array_equal(dw - off, rdw), ('dW', xs, ws, s, d, padding)
+                        cnt += 1
+    assert cnt > 300
+
+
 def test_conv_channel_multiples_of_32_integer_exact(hip):
     """Channel counts that are multiples of 32 take the tap-major kernels
     (forward / dgrad: permuted weights, address arithmetic in the scalar
