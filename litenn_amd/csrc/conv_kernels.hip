@@ -125,7 +125,7 @@ struct ConvCfg {
   static constexpr int SA = LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
   static constexpr int SB = LdsSize<PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP, BNMAX>::value;
-  static constexpr int STAGES = 2;   // 3 (fragments read ahead of the phase barrier) measured no faster
+  static constexpr int STAGES = 2;
 };
 
 // Loader selection and initialisation per pass.  FLAG:
@@ -153,8 +153,8 @@ struct ConvProblem<PASS_FWD, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_FWD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  template <int R> using LA = PlainKC<R, true>;          // permuted weights [O][KK*C]
-  template <int R> using LB = ConvFwdBTap<R>;
+  template <int R> using LA = DirectKC<R>;               // permuted weights [O][KK*C]
+  template <int R> using LB = ConvFwdBTap<R, true>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, col0, Ncols, kbeg); }
 };
@@ -169,8 +169,8 @@ struct ConvProblem<PASS_DGRAD, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_DGRAD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  template <int R> using LA = PlainKC<R, true>;          // permuted weights [C][KK*O]
-  template <int R> using LB = ConvDgradBTap<R>;
+  template <int R> using LA = DirectKC<R>;               // permuted weights [C][taps*O]
+  template <int R> using LB = ConvDgradBTap<R, true>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };

@@ -18,21 +18,27 @@ struct GemmArgs {
   int n_units, total_units;       // schedule: units of 32*WN columns per M tile
 };
 
-template <int WM, int NTMAX, bool TA, bool TB, bool VEC>
+// MODE: how operands travel.  0: 32-bit loads through registers (any alignment,
+// any K); 1: 128-bit loads through registers; 2: 128-bit transfers straight
+// into LDS (as 1, and K a multiple of BK).
+template <int WM, int NTMAX, bool TA, bool TB, int MODE>
 struct GemmCfg {
   static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
   static constexpr int SA = LdsSize<!TA, BM>::value;
   static constexpr int SB = LdsSize<TB, BNMAX>::value;
-  static constexpr int STAGES = 2;   // 3 (fragments read ahead of the phase barrier) measured no faster
+  static constexpr int STAGES = 2;
 };
 
 // A operand: !TA -> A[M][K] row-major, K-contiguous; TA -> stored [K][M].
 // B operand: !TB -> B[K][N], row(n)-contiguous;      TB -> stored [N][K].
-template <bool TA, bool TB, bool VEC, int ST>
+template <bool TA, bool TB, int MODE, int ST>
 struct GemmProblem {
   static constexpr int STAGES = ST;
-  template <int R> using LA = typename std::conditional<TA, PlainMC<R, VEC>, PlainKC<R, VEC>>::type;
-  template <int R> using LB = typename std::conditional<TB, PlainKC<R, VEC>, PlainMC<R, VEC>>::type;
+  static constexpr bool VEC = MODE >= 1, DIR = MODE == 2;
+  template <int R> using KCL = typename std::conditional<DIR, DirectKC<R>, PlainKC<R, VEC>>::type;
+  template <int R> using MCL = typename std::conditional<DIR, DirectMC<R>, PlainMC<R, VEC>>::type;
+  template <int R> using LA = typename std::conditional<TA, MCL<R>, KCL<R>>::type;
+  template <int R> using LB = typename std::conditional<TB, KCL<R>, MCL<R>>::type;
   rsrc_t ra, rb, rc;
   int lda, ldb, M, Ncols, K, kbeg, kend, beta;
   OutMap om;
@@ -40,12 +46,12 @@ struct GemmProblem {
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rb, ldb, col0, Ncols, K); }
 };
 
-template <int WM, int NTMAX, bool TA, bool TB, bool VEC>
+template <int WM, int NTMAX, bool TA, bool TB, int MODE>
 __global__ __launch_bounds__(512, 2) void gemm_kernel(GemmArgs a) {
-  using Cfg = GemmCfg<WM, NTMAX, TA, TB, VEC>;
+  using Cfg = GemmCfg<WM, NTMAX, TA, TB, MODE>;
   __shared__ __attribute__((aligned(16))) float lds[Cfg::STAGES * (Cfg::SA + Cfg::SB)];
   const long long b = blockIdx.y;
-  GemmProblem<TA, TB, VEC, Cfg::STAGES> p;
+  GemmProblem<TA, TB, MODE, Cfg::STAGES> p;
   p.ra = make_rsrc(a.A + b * a.sA, a.bytesA);
   p.rb = make_rsrc(a.B + b * a.sB, a.bytesB);
   p.rc = make_rsrc(a.C + b * a.sC, a.bytesC);
@@ -56,7 +62,7 @@ __global__ __launch_bounds__(512, 2) void gemm_kernel(GemmArgs a) {
 }
 
 template <int WM, int NTMAX, bool TA, bool TB>
-static int launch_cfg(DeviceCtx* ctx, GemmArgs& a, int batch, bool vec) {
+static int launch_cfg(DeviceCtx* ctx, GemmArgs& a, int batch, int mode) {
   constexpr int WN = 4 / WM, BM = 32 * WM;
   const int m_tiles = (a.M + BM - 1) / BM;
   a.n_units = (a.N + 32 * WN - 1) / (32 * WN);
@@ -67,19 +73,21 @@ static int launch_cfg(DeviceCtx* ctx, GemmArgs& a, int batch, bool vec) {
   if (slots < 1) slots = 1;
   const int grid = (int)(total < slots ? total : slots);
   dim3 g(grid, batch, 1), b(512, 1, 1);
-  if (vec)
-    hipLaunchKernelGGL((gemm_kernel<WM, NTMAX, TA, TB, true>), g, b, 0, ctx->stream, a);
+  if (mode == 2)
+    hipLaunchKernelGGL((gemm_kernel<WM, NTMAX, TA, TB, 2>), g, b, 0, ctx->stream, a);
+  else if (mode == 1)
+    hipLaunchKernelGGL((gemm_kernel<WM, NTMAX, TA, TB, 1>), g, b, 0, ctx->stream, a);
   else
-    hipLaunchKernelGGL((gemm_kernel<WM, NTMAX, TA, TB, false>), g, b, 0, ctx->stream, a);
+    hipLaunchKernelGGL((gemm_kernel<WM, NTMAX, TA, TB, 0>), g, b, 0, ctx->stream, a);
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }
 
 template <bool TA, bool TB>
-static int launch_layout(DeviceCtx* ctx, GemmArgs& a, int batch, bool vec) {
-  if (a.M > 64) return launch_cfg<4, 4, TA, TB>(ctx, a, batch, vec);
-  if (a.M > 32) return launch_cfg<2, 2, TA, TB>(ctx, a, batch, vec);
-  return launch_cfg<1, 1, TA, TB>(ctx, a, batch, vec);
+static int launch_layout(DeviceCtx* ctx, GemmArgs& a, int batch, int mode) {
+  if (a.M > 64) return launch_cfg<4, 4, TA, TB>(ctx, a, batch, mode);
+  if (a.M > 32) return launch_cfg<2, 2, TA, TB>(ctx, a, batch, mode);
+  return launch_cfg<1, 1, TA, TB>(ctx, a, batch, mode);
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -109,10 +117,10 @@ int launch_gemm(DeviceCtx* ctx, int ta, int tb, int batch, int M, int N, int K, 
   // multiples of four floats.
   const bool va = aligned16(A) && lda % 4 == 0 && sA % 4 == 0 && a_cols % 4 == 0;
   const bool vb = aligned16(B) && ldb % 4 == 0 && sB % 4 == 0 && b_cols % 4 == 0;
-  const bool vec = va && vb;
-  if (!ta && !tb) return launch_layout<false, false>(ctx, a, batch, vec);
-  if (!ta && tb) return launch_layout<false, true>(ctx, a, batch, vec);
-  if (ta && !tb) return launch_layout<true, false>(ctx, a, batch, vec);
+  const int mode = (va && vb) ? (K % BK == 0 ? 2 : 1) : 0;
+  if (!ta && !tb) return launch_layout<false, false>(ctx, a, batch, mode);
+  if (!ta && tb) return launch_layout<false, true>(ctx, a, batch, mode);
+  if (ta && !tb) return launch_layout<true, false>(ctx, a, batch, mode);
   return set_error(LNN_ERR_UNSUPPORTED, "gemm: trans_a and trans_b together are not provided");
 }
 

@@ -39,6 +39,14 @@ constexpr int LDK = BK + 4;       // row stride (floats) of a K-contiguous LDS t
 constexpr uint32_t OOB = 0x80000000u;  // byte offset beyond every buffer (< 2 GiB each)
 constexpr int BIG = 0x40000000;   // coordinate that fails every range test
 
+// LDS tile layouts.  R = rows of the tile (BM on the A side, a group's columns on the B side).
+//   LAY_KC        tile[row][LDK]: k contiguous, rows padded to LDK floats
+//   LAY_KC_SWZ    tile[row][BK]:  k contiguous, no padding, 4-float group g of row r in slot g ^ (r % 8)
+//   LAY_MC        tile[k][R]:     row contiguous, one tile shared by both groups
+//   LAY_MC_SPLIT  one tile[k][R'] per group, back to back: a group's slab of R' rows
+//                 starting at tile row `off` begins at float off*BK
+enum { LAY_KC = 0, LAY_KC_SWZ = 1, LAY_MC = 2, LAY_MC_SPLIT = 3 };
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -64,6 +72,16 @@ __device__ __forceinline__ float buf_load_s(rsrc_t r, uint32_t voff, uint32_t so
 }
 __device__ __forceinline__ f32x4 buf_load4_s(rsrc_t r, uint32_t voff, uint32_t soff) {
   return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
+}
+// Global -> LDS without passing through registers: lane l of the wavefront
+// deposits its 4 (16) bytes at lds + 4*l (16*l).  lds must be wave-uniform.
+// An out-of-range lane writes zeros, an inactive lane writes nothing.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+__device__ __forceinline__ void buf_load_lds4(rsrc_t r, float* lds, uint32_t voff, uint32_t soff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)lds, 4, (int)voff, (int)soff, 0, 0);
+}
+__device__ __forceinline__ void buf_load_lds16(rsrc_t r, float* lds, uint32_t voff, uint32_t soff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)lds, 16, (int)voff, (int)soff, 0, 0);
 }
 __device__ __forceinline__ void buf_store(rsrc_t r, uint32_t off, float v) {
   __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, (int)off, 0, 0);
@@ -150,6 +168,73 @@ struct PlainKC {
     for (int e = 0; e < E; ++e) {
       const int s = gtid() + 256 * e, row = s / KG, kg = s % KG;
       if (R * KG % 256 == 0 || row < R) *reinterpret_cast<f32x4*>(&lds[(off + row) * LDK + 4 * kg]) = v[e];
+    }
+  }
+};
+
+// Plain strided matrix, K-contiguous, straight into LDS (needs K % BK == 0 and
+// 16-byte aligned rows).  The LDS tile is [row][BK] without padding; to keep
+// the 128-bit fragment reads conflict free the k groups of a row are stored
+// XOR-swizzled: group g of row r sits in slot g ^ (r % 8).  One instruction
+// moves 8 rows (1 KiB): lane l carries slot l % 8 of row l / 8.
+template <int R>
+struct DirectKC {
+  static constexpr bool KC = true, DIRECT = true;
+  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int NB = R / 8, E = (NB + 3) / 4;
+  static_assert(R % 8 == 0, "whole 8-row blocks");
+  rsrc_t rs;
+  uint32_t voff[E];
+  __device__ __forceinline__ void init(rsrc_t r, int ld, int row0, int M, int) {
+    rs = r;
+    const int wave = gwave(), lane = threadIdx.x & 63, rb = lane >> 3, kg = (lane & 7) ^ rb;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int row = row0 + (wave + 4 * e) * 8 + rb;
+      voff[e] = row < M ? (uint32_t)(row * ld + kg * 4) * 4u : OOB;
+    }
+  }
+  // off: first tile row of this group
+  __device__ __forceinline__ void issue(int k0, float* lds, int, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int blk = wave + 4 * e;
+      if (NB % 4 == 0 || blk < NB) buf_load_lds16(rs, lds + (off + blk * 8) * BK, voff[e], (uint32_t)k0 * 4u);
+    }
+  }
+};
+
+// Plain strided matrix stored K-major (element (r, k) at k*ld + r), straight
+// into LDS with 128-bit transfers (16-byte aligned rows, row count % 4 == 0).
+// One instruction moves 256 consecutive floats of the group's [BK][R] slab.
+// K rows past the end lie beyond the buffer and arrive as zeros.
+template <int R>
+struct DirectMC {
+  static constexpr bool KC = false, DIRECT = true;
+  static constexpr int LAYOUT = LAY_MC_SPLIT;
+  static constexpr int NI = BK * R / 256, E = (NI + 3) / 4;
+  static_assert(R % 8 == 0, "whole 256-float transfers");
+  rsrc_t rs;
+  uint32_t voff[E];
+  int ld;
+  __device__ __forceinline__ void init(rsrc_t r, int ld_, int row0, int M, int) {
+    rs = r;
+    ld = ld_;
+    const int wave = gwave(), lane = threadIdx.x & 63;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int f = (wave + 4 * e) * 256 + lane * 4, k = f / R, n = f - k * R;
+      voff[e] = (k < BK && row0 + n < M) ? (uint32_t)(k * ld + row0 + n) * 4u : OOB;
+    }
+  }
+  __device__ __forceinline__ void issue(int k0, float* lds, int, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+    const uint32_t soff = (uint32_t)(k0 * ld) * 4u;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int q = wave + 4 * e;
+      if (NI % 4 == 0 || q < NI) buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff);
     }
   }
 };
@@ -304,9 +389,9 @@ struct ConvFwdB {
 // channel part is wave-uniform and rides in the scalar offset of the buffer
 // instruction.  No table, no per-element arithmetic.  fetch() must be called
 // with consecutive K steps starting at the kbeg given to init().
-template <int R>
+template <int R, bool DIR = false>
 struct ConvFwdBTap {
-  static constexpr bool KC = false;
+  static constexpr bool KC = false, DIRECT = DIR;
   static constexpr int CC = (R + 63) / 64;
   rsrc_t rs;
   int IH, IW, IHW, C, D, KW;
@@ -351,6 +436,9 @@ struct ConvFwdBTap {
 #pragma unroll
       for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
     }
+    advance();
+  }
+  __device__ __forceinline__ void advance() {
     c0 += BK;
     if (c0 >= C) {   // wave-uniform: next tap
       c0 = 0;
@@ -358,6 +446,18 @@ struct ConvFwdBTap {
       if (kw == KW) { kw = 0; ++kh; }
       set_tap();
     }
+  }
+  // straight into the LDS stage: element (k = wave + 4e, column lane + 64c)
+  __device__ __forceinline__ void issue(int, float* lds, int ld, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
+#pragma unroll
+    for (int e = 0; e < KR; ++e) {
+      const uint32_t soff = (uint32_t)((c0 + wave + 4 * e) * IHW) * 4u;
+#pragma unroll
+      for (int c = 0; c < CC; ++c)
+        if (R % 64 == 0 || lane + 64 * c < R) buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);
+    }
+    advance();
   }
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
@@ -369,9 +469,9 @@ struct ConvFwdBTap {
   }
 };
 
-template <int R>
+template <int R, bool DIR = false>
 struct ConvDgradBTap {
-  static constexpr bool KC = false;
+  static constexpr bool KC = false, DIRECT = DIR;
   static constexpr int CC = (R + 63) / 64;
   rsrc_t rs;
   ktab_t tab;           // one entry per tap of the pixel class: y, z (see ConvDgradB)
@@ -419,6 +519,9 @@ struct ConvDgradBTap {
 #pragma unroll
       for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
     }
+    advance();
+  }
+  __device__ __forceinline__ void advance() {
     o0 += BK;
     if (o0 >= O) {   // wave-uniform: next tap
       o0 = 0;
@@ -427,6 +530,18 @@ struct ConvDgradBTap {
       set_tap();
       ny = (tab + tap + 1)->y; nz = (tab + tap + 1)->z;
     }
+  }
+  // straight into the LDS stage: element (k = wave + 4e, column lane + 64c)
+  __device__ __forceinline__ void issue(int, float* lds, int ld, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
+#pragma unroll
+    for (int e = 0; e < KR; ++e) {
+      const uint32_t soff = (uint32_t)((o0 + wave + 4 * e) * OHW) * 4u;
+#pragma unroll
+      for (int c = 0; c < CC; ++c)
+        if (R % 64 == 0 || lane + 64 * c < R) buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);
+    }
+    advance();
   }
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
@@ -785,24 +900,31 @@ struct OutMap {
 // each group of 8 k values lane half h supplies k = 8*kk + 4*h + t to the
 // t-th MFMA.  A and B use the same k assignment, so any k permutation cancels.
 // ---------------------------------------------------------------------------
-template <int NT, bool A_KC, bool B_KC, int RA, int RB>
+template <int NT, int LAY_A, int LAY_B, int RA, int RB>
 __device__ __forceinline__ void load_frags(const float* __restrict__ As, const float* __restrict__ Bs, int arow,
                                            int brow, int kk, float (&a)[4], float (&b)[NT][4]) {
   const int lane = threadIdx.x & 63, i = lane & 31, h = lane >> 5;
   const int kb = kk * 8 + h * 4;
-  if (A_KC) {
-    const f32x4 t = *reinterpret_cast<const f32x4*>(&As[(arow + i) * LDK + kb]);
+  const int sw = ((2 * kk + h) ^ (i & 7)) << 2;   // swizzled position of k group 2*kk + h; row offsets are multiples of 32
+  if (LAY_A == LAY_KC || LAY_A == LAY_KC_SWZ) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(LAY_A == LAY_KC ? &As[(arow + i) * LDK + kb] : &As[(arow + i) * BK + sw]);
     a[0] = t[0]; a[1] = t[1]; a[2] = t[2]; a[3] = t[3];
-  } else {
+  } else if (LAY_A == LAY_MC) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) a[t] = As[(kb + t) * RA + arow + i];
+  } else {   // two [BK][RA/2] slabs
+    constexpr int H = RA / 2;
+    const int r = arow + i;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) a[t] = As[(r / H) * (BK * H) + (kb + t) * H + r % H];
   }
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
-    if (B_KC) {
-      const f32x4 t = *reinterpret_cast<const f32x4*>(&Bs[(brow + 32 * j + i) * LDK + kb]);
+    if (LAY_B == LAY_KC || LAY_B == LAY_KC_SWZ) {
+      const int r = brow + 32 * j + i;
+      const f32x4 t = *reinterpret_cast<const f32x4*>(LAY_B == LAY_KC ? &Bs[r * LDK + kb] : &Bs[r * BK + sw]);
       b[j][0] = t[0]; b[j][1] = t[1]; b[j][2] = t[2]; b[j][3] = t[3];
-    } else {
+    } else {   // shared tile or the group's own slab: the caller passes the matching base, pitch and brow
 #pragma unroll
       for (int t = 0; t < 4; ++t) b[j][t] = Bs[(kb + t) * RB + brow + 32 * j + i];
     }
@@ -810,26 +932,22 @@ __device__ __forceinline__ void load_frags(const float* __restrict__ As, const f
 }
 
 // One LDS stage = BK/8 groups of 4*NT MFMAs.  The fragments of the first
-// group are either already in fa[0] / fb[0] (PRE: read before the phase barrier)
-// or read up front; the reads of each following group are slotted one by one
-// between the MFMAs of the group before it, so the matrix pipe does not wait
-// for LDS within the stage.
-template <int NT, bool A_KC, bool B_KC, int RA, int RB, bool PRE>
+// group are read up front; the reads of each following group are slotted one
+// by one between the MFMAs of the group before it, so the matrix pipe does
+// not wait for LDS within the stage.
+template <int NT, int LAY_A, int LAY_B, int RA, int RB>
 __device__ __forceinline__ void mma_stage(const float* __restrict__ As, const float* __restrict__ Bs,
-                                          f32x16 (&acc)[NT], int arow, int brow, float (&fa)[2][4],
-                                          float (&fb)[2][NT][4]) {
+                                          f32x16 (&acc)[NT], int arow, int brow) {
   constexpr int NG = BK / 8;
-  static_assert(NG % 2 == 0, "the pre-loaded fragments live in buffer 0");
+  float fa[2][4], fb[2][NT][4];
   // LDS read instructions per group: A is one b128 or four b32; B is NT b128 or 4*NT b32 (paired into read2)
-  constexpr int RD = (A_KC ? 1 : 2) + (B_KC ? NT : 2 * NT);
-  if (!PRE) {
-    load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, 0, fa[0], fb[0]);
-    __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);              // DS reads of group 0
-  }
+  constexpr int RD = (LAY_A <= LAY_KC_SWZ ? 1 : 2) + (LAY_B <= LAY_KC_SWZ ? NT : 2 * NT);
+  load_frags<NT, LAY_A, LAY_B, RA, RB>(As, Bs, arow, brow, 0, fa[0], fb[0]);
+  __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);              // DS reads of group 0
 #pragma unroll
   for (int kk = 0; kk < NG; ++kk) {
     const int cur = kk & 1;
-    if (kk + 1 < NG) load_frags<NT, A_KC, B_KC, RA, RB>(As, Bs, arow, brow, kk + 1, fa[cur ^ 1], fb[cur ^ 1]);
+    if (kk + 1 < NG) load_frags<NT, LAY_A, LAY_B, RA, RB>(As, Bs, arow, brow, kk + 1, fa[cur ^ 1], fb[cur ^ 1]);
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -875,34 +993,52 @@ __device__ __forceinline__ void fetch_b(LB& lb, int k0, const LA& la) {
     lb.fetch(k0);
 }
 
+// A loader that moves global memory straight into LDS declares
+// `static constexpr bool DIRECT = true` and provides issue(k0, lds, ld, off)
+// instead of fetch() / commit().
+template <class T, class = void>
+struct is_direct : std::false_type {};
+template <class T>
+struct is_direct<T, std::void_t<decltype(T::DIRECT)>> : std::integral_constant<bool, T::DIRECT> {};
+// LDS layout a loader fills: T::LAYOUT if declared, else padded K-contiguous or shared row-contiguous by T::KC
+template <class T, class = void>
+struct layout_of : std::integral_constant<int, T::KC ? LAY_KC : LAY_MC> {};
+template <class T>
+struct layout_of<T, std::void_t<decltype(T::LAYOUT)>> : std::integral_constant<int, T::LAYOUT> {};
+
+// End of a phase.  All of this wavefront's LDS writes (lgkmcnt) and
+// global -> LDS transfers (vmcnt) have landed before it reports to the barrier.
+__device__ __forceinline__ void phase_barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 // Body of one group (G = 0 or 1) for one sub-tile: BM = 32*WM rows shared by
 // both groups, 32*WN*NT columns of its own starting at column offset COFF of
 // the sub-tile; BNTOT is the column count of both groups together.
-//
-// P::STAGES LDS stages.  With 2, K step t+1 is parked while step t is computed
-// and a compute phase starts by reading its first fragments.  With 3, step t+2
-// is parked during step t, so step t+1 is complete a whole step early and each
-// group reads the first fragments of its next compute phase *before* the
-// barrier that starts it: the matrix pipe restarts right at the barrier.
 template <int WM, int NT, int G, int COFF, int BNTOT, class P>
 __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB, int strideA, int strideB, int m0,
                                            int ng) {   // ng: first global column of this group
   constexpr int WN = 4 / WM, BM = 32 * WM, HALF = BM / 2, NTC = NT > 0 ? NT : 1, BN = 32 * WN * NTC;
-  constexpr int ST = P::STAGES;
-  constexpr bool PRE = ST == 3;
   using LA = typename P::template LA<HALF>;
   using LB = typename P::template LB<BN>;
-  constexpr bool A_KC = LA::KC, B_KC = LB::KC;
-  constexpr int LDA = A_KC ? LDK : BM, LDB = B_KC ? LDK : BNTOT;
+  constexpr int LAY_A = layout_of<LA>::value, LAY_B = layout_of<LB>::value;
+  constexpr bool DIRECT = is_direct<LA>::value;
+  static_assert(is_direct<LA>::value == is_direct<LB>::value, "both loaders of a kernel move data the same way");
+  constexpr int LDA = LAY_A == LAY_KC ? LDK : (LAY_A == LAY_KC_SWZ ? BK : BM);
+  constexpr int LDB = LAY_B == LAY_KC ? LDK : (LAY_B == LAY_KC_SWZ ? BK : BNTOT);
   const int wave = gwave(), lane = threadIdx.x & 63;
   const int wm = wave % WM, wn = wave / WM;
-  const int arow = wm * 32, brow = COFF + wn * NT * 32;
+  // fragment addressing: a split B tile is read through the group's own slab
+  constexpr int RB = LAY_B == LAY_MC_SPLIT ? BN : BNTOT;
+  const int arow = wm * 32, brow = (LAY_B == LAY_MC_SPLIT ? 0 : COFF) + wn * NT * 32;
+  const float* const ldsBr = ldsB + (LAY_B == LAY_MC_SPLIT ? COFF * BK : 0);
   LA la;
   LB lb;
   p.template init_a<HALF>(la, m0 + G * HALF);
   if (NT > 0) p.template init_b<BN>(lb, ng, la);
   f32x16 acc[NTC];
-  float fa[2][4], fb[2][NTC][4];
 #pragma unroll
   for (int j = 0; j < NTC; ++j)
 #pragma unroll
@@ -910,60 +1046,69 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
 
   const int kbeg = p.kbeg;
   const int nk = (p.kend - kbeg + BK - 1) / BK;
-  // prologue: K steps 0 .. ST-2 into their stages, step ST-1 into registers
-#pragma unroll
-  for (int q = 0; q < ST - 1; ++q)
-    if (q < nk) {
-      la.fetch(kbeg + q * BK);
-      if (NT > 0) fetch_b(lb, kbeg + q * BK, la);
-      la.commit(ldsA + q * strideA, LDA, G * HALF);
-      if (NT > 0) lb.commit(ldsB + q * strideB, LDB, COFF);
-    }
-  if (ST - 1 < nk) {
-    la.fetch(kbeg + (ST - 1) * BK);
-    if (NT > 0) fetch_b(lb, kbeg + (ST - 1) * BK, la);
-  }
-  __syncthreads();
-  if (PRE && G == 0 && NT > 0 && nk > 0)
-    load_frags<NTC, A_KC, B_KC, BM, BNTOT>(ldsA, ldsB, arow, brow, 0, fa[0], fb[0]);
 
   // Each K step t has two phases separated by barriers.  Group 0 computes in
   // the first and moves data in the second; group 1 the other way round.
-  // "Moving data" in step t = park K step t+ST-1 (fetched one step earlier) in
-  // its stage, which was last read for step t-1, then fetch K step t+ST.
-  int cur = 0;        // stage of K step t
-  for (int t = 0; t < nk; ++t) {
-    const int park = cur == 0 ? ST - 1 : cur - 1;           // stage of K step t+ST-1 == stage of step t-1
-    const int nxt = cur + 1 == ST ? 0 : cur + 1;            // stage of K step t+1
-#pragma unroll
-    for (int phase = 0; phase < 2; ++phase) {
-      if (phase == G) {
-        if (NT > 0)
-          mma_stage<NTC, A_KC, B_KC, BM, BNTOT, PRE>(ldsA + cur * strideA, ldsB + cur * strideB, acc, arow, brow, fa, fb);
-      } else {
-        if (t + ST - 1 < nk) {
-          la.commit(ldsA + park * strideA, LDA, G * HALF);
-          if (NT > 0) lb.commit(ldsB + park * strideB, LDB, COFF);
-        }
-        if (t + ST < nk) {
-          la.fetch(kbeg + (t + ST) * BK);
-          if (NT > 0) fetch_b(lb, kbeg + (t + ST) * BK, la);
-        }
-        if (PRE && NT > 0) {
-          // first fragments of this group's next compute phase: group 0 computes
-          // step t+1 next, group 1 computes step t in the coming phase
-          const int st = G == 0 ? nxt : cur;
-          if (G == 1 || t + 1 < nk)
-            load_frags<NTC, A_KC, B_KC, BM, BNTOT>(ldsA + st * strideA, ldsB + st * strideB, arow, brow, 0, fa[0], fb[0]);
-        }
-      }
-      // the phase ends only when all of its MFMAs have been issued: do not let
-      // the scheduler sink them below the barrier into the other group's phase
-      __builtin_amdgcn_sched_barrier(0);
-      __syncthreads();
-      __builtin_amdgcn_sched_barrier(0);
+  if constexpr (DIRECT) {
+    // "moving data" in step t = sending K step t+1 from global memory into the
+    // other LDS stage, which was last read for step t-1
+    if (nk > 0) {
+      la.issue(kbeg, ldsA, LDA, G * HALF);
+      if (NT > 0) lb.issue(kbeg, ldsB, LDB, COFF);
     }
-    cur = nxt;
+    phase_barrier();
+    for (int t = 0; t < nk; ++t) {
+      const int cur = t & 1;
+#pragma unroll
+      for (int phase = 0; phase < 2; ++phase) {
+        if (phase == G) {
+          if (NT > 0)
+            mma_stage<NTC, LAY_A, LAY_B, BM, RB>(ldsA + cur * strideA, ldsBr + cur * strideB, acc, arow, brow);
+        } else if (t + 1 < nk) {
+          la.issue(kbeg + (t + 1) * BK, ldsA + (cur ^ 1) * strideA, LDA, G * HALF);
+          if (NT > 0) lb.issue(kbeg + (t + 1) * BK, ldsB + (cur ^ 1) * strideB, LDB, COFF);
+        }
+        phase_barrier();
+      }
+    }
+  } else {
+    // "moving data" in step t = parking K step t+1 (in registers since step
+    // t-1) in the other LDS stage, then fetching K step t+2 into registers
+    if (nk > 0) {
+      la.fetch(kbeg);
+      if (NT > 0) fetch_b(lb, kbeg, la);
+      la.commit(ldsA, LDA, G * HALF);
+      if (NT > 0) lb.commit(ldsB, LDB, COFF);
+    }
+    if (1 < nk) {
+      la.fetch(kbeg + BK);
+      if (NT > 0) fetch_b(lb, kbeg + BK, la);
+    }
+    __syncthreads();
+    for (int t = 0; t < nk; ++t) {
+      const int cur = t & 1;
+#pragma unroll
+      for (int phase = 0; phase < 2; ++phase) {
+        if (phase == G) {
+          if (NT > 0)
+            mma_stage<NTC, LAY_A, LAY_B, BM, RB>(ldsA + cur * strideA, ldsBr + cur * strideB, acc, arow, brow);
+        } else {
+          if (t + 1 < nk) {
+            la.commit(ldsA + (cur ^ 1) * strideA, LDA, G * HALF);
+            if (NT > 0) lb.commit(ldsB + (cur ^ 1) * strideB, LDB, COFF);
+          }
+          if (t + 2 < nk) {
+            la.fetch(kbeg + (t + 2) * BK);
+            if (NT > 0) fetch_b(lb, kbeg + (t + 2) * BK, la);
+          }
+        }
+        // the phase ends only when all of its MFMAs have been issued: do not let
+        // the scheduler sink them below the barrier into the other group's phase
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
   }
 
   // epilogue: acc[j][r] is C[m0 + wm*32 + 8*(r/4) + 4*(lane/32) + r%4][ng + (wn*NT + j)*32 + lane%32]

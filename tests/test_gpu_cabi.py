@@ -47,7 +47,10 @@ def test_gemm_integer_exact(hip, ta, tb):
     rs = np.random.RandomState(10 + 2 * ta + tb)
     shapes = [(1, 1, 1, 1), (1, 5, 7, 3), (1, 33, 65, 17), (1, 128, 128, 16), (1, 130, 257, 100),
               (3, 8, 32, 16), (2, 70, 40, 24), (1, 64, 512, 48), (1, 256, 384, 160), (1, 2, 3000, 5),
-              (4, 1, 9, 1), (1, 97, 31, 1000)]
+              (4, 1, 9, 1), (1, 97, 31, 1000),
+              # 16-byte aligned rows and K a multiple of 32: operands go straight into LDS
+              (1, 128, 256, 64), (2, 36, 100, 32), (1, 20, 44, 96), (3, 132, 260, 128), (1, 68, 8, 32),
+              (1, 4, 4, 32), (1, 516, 96, 64), (1, 64, 1028, 320)]
     for batch, M, N, K in shapes:
         say(f'gemm ta={ta} tb={tb} batch={batch} M={M} N={N} K={K}')
         a = rs.randint(16, size=(batch, K, M) if ta else (batch, M, K)).astype(np.float32)
