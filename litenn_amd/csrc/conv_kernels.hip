@@ -7,6 +7,20 @@
 //   wgrad    dW[O  x CKK] = dY[O x P]        . im2row(X)[P x CKK]     (split over P)
 #include "common.hpp"
 
+#ifndef LNN_STAGES_WGRAD
+#define LNN_STAGES_WGRAD 3
+#endif
+#ifndef LNN_STAGES_FD
+#define LNN_STAGES_FD 2
+#endif
+// B-side gathers: 1 = straight into LDS, 0 = through registers (needs three stages)
+#ifndef LNN_FD_B_DIRECT
+#define LNN_FD_B_DIRECT 1
+#endif
+#ifndef LNN_WGRAD_B_DIRECT
+#define LNN_WGRAD_B_DIRECT 1
+#endif
+
 namespace lnn {
 
 struct ConvArgs {
@@ -19,7 +33,8 @@ struct ConvArgs {
   int M, Ncols, K;   // GEMM extents
   int beta;
   int n_units, total_units;
-  int ksplit;        // wgrad: number of K slices (gridDim.y)
+  int ksplit;        // wgrad: number of K slices (tap-major: of every chunk but the last)
+  int n_chunks, ks_last;   // tap-major wgrad: chunks of chunk_units units; K slices of the last, possibly shorter one
   FastDiv dC;        // tap-major wgrad: divide a column index by the channel count
   int chunk_units;   // tap-major wgrad: units per workgroup
   // dgrad: g describes one pixel class (g.IH, g.IW = class grid); the plane it is cut from:
@@ -71,28 +86,39 @@ __global__ void build_ktable(KEntry* tab, int K, int Kpad, int mode, ConvGeom g,
 
 // out[f(i)] (+)= sum over slices of part[slice][i], slices added in a fixed order.
 // A block covers 32 consecutive i (one 128-byte line per slice row) with 8
-// lanes per i striding over the slices.  permute: partial column tap*C + c of
-// row m goes to out[m][c][tap] (tap-major wgrad columns back to OIHW).
-__global__ __launch_bounds__(256) void reduce_partials(float* out, const float* part, int n, int slices, int beta,
-                                                       int ncols, FastDiv dN, FastDiv dC, int KK, int permute) {
+// lanes per i striding over the slices.  Elements of units >= last_unit0 (unit
+// = (m >> bm_log) * per_mt + (col >> uw_log)) have only slices_last slices.
+// permute: partial column tap*C + c of row m goes to out[m][c][tap]
+// (tap-major wgrad columns back to OIHW).
+struct ReduceArgs {
+  int n, slices, slices_last, beta, ncols, KK, permute;
+  int bm_log, uw_log, per_mt, last_unit0;
+  FastDiv dN, dC;
+};
+__global__ __launch_bounds__(256) void reduce_partials(float* out, const float* part, ReduceArgs a) {
   __shared__ float red[8][33];
   const int li = threadIdx.x & 31, ls = threadIdx.x >> 5;
   const int i = blockIdx.x * 32 + li;
   float s = 0.0f;
-  if (i < n)
-    for (int k = ls; k < slices; k += 8) s += part[(size_t)k * n + i];
+  uint32_t m = 0, col = 0;
+  if (i < a.n) {
+    m = a.dN.div((uint32_t)i);
+    col = (uint32_t)i - m * (uint32_t)a.ncols;
+    const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
+    const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+    for (int k = ls; k < ns; k += 8) s += part[(size_t)k * a.n + i];
+  }
   red[ls][li] = s;
   __syncthreads();
-  if (ls == 0 && i < n) {
+  if (ls == 0 && i < a.n) {
 #pragma unroll
     for (int k = 1; k < 8; ++k) s += red[k][li];
     uint32_t o = (uint32_t)i;
-    if (permute) {
-      const uint32_t m = dN.div(o), col = o - m * (uint32_t)ncols;
-      const uint32_t tap = dC.div(col), ch = col - tap * dC.d;
-      o = m * (uint32_t)ncols + ch * (uint32_t)KK + tap;
+    if (a.permute) {
+      const uint32_t tap = a.dC.div(col), ch = col - tap * a.dC.d;
+      o = m * (uint32_t)a.ncols + ch * (uint32_t)a.KK + tap;
     }
-    out[o] = beta ? out[o] + s : s;
+    out[o] = a.beta ? out[o] + s : s;
   }
 }
 
@@ -121,16 +147,18 @@ __global__ void permute_weights(float* wp, const float* w, int O, int C, int KK,
 template <int PASS, int WM, int NTMAX, bool FLAG>
 struct ConvCfg {
   static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
+  // the tap-major passes send both operands straight into unpadded LDS tiles, three stages deep
+  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || PASS == PASS_DGRAD_TAP || PASS == PASS_WGRAD_TAP;
   // A side is K-contiguous in LDS for all passes.
-  static constexpr int SA = LdsSize<true, BM>::value;
+  static constexpr int SA = DIRECT ? BM * BK : LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
-  static constexpr int SB = LdsSize<PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP, BNMAX>::value;
-  static constexpr int STAGES = 2;
+  static constexpr int SB = DIRECT ? BNMAX * BK : LdsSize<PASS == PASS_WGRAD, BNMAX>::value;
+  static constexpr int STAGES = !DIRECT ? 2 : (PASS == PASS_WGRAD_TAP ? LNN_STAGES_WGRAD : LNN_STAGES_FD);
 };
 
 // Loader selection and initialisation per pass.  FLAG:
 //   PASS_FWD        128-bit loads of W rows (CKK % 4 == 0)
-//   PASS_WGRAD      128-bit loads of dY (OHW % 4 == 0)
+//   PASS_WGRAD(_TAP) 128-bit loads of dY (OHW % 4 == 0)
 template <int PASS, bool FLAG, int ST>
 struct ConvProblem;
 
@@ -154,7 +182,7 @@ template <bool FLAG, int ST>
 struct ConvProblem<PASS_FWD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = DirectKC<R>;               // permuted weights [O][KK*C]
-  template <int R> using LB = ConvFwdBTap<R, true>;
+  template <int R> using LB = ConvFwdBTap<R, LNN_FD_B_DIRECT != 0>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, col0, Ncols, kbeg); }
 };
@@ -170,7 +198,7 @@ template <bool FLAG, int ST>
 struct ConvProblem<PASS_DGRAD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = DirectKC<R>;               // permuted weights [C][taps*O]
-  template <int R> using LB = ConvDgradBTap<R, true>;
+  template <int R> using LB = ConvDgradBTap<R, LNN_FD_B_DIRECT != 0>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
@@ -186,10 +214,10 @@ struct ConvProblem<PASS_WGRAD, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  template <int R> using LA = ConvWgradTapA<R>;
-  template <int R> using LB = ConvWgradTapB<R>;
-  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend); }
-  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A& la) const { l.init(rx, g, col0, la); }
+  template <int R> using LA = typename std::conditional<FLAG, ConvWgradTapA4Direct<R>, ConvWgradTapADirect<R>>::type;
+  template <int R> using LB = ConvWgradTapBDirect<R, LNN_WGRAD_B_DIRECT != 0>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A& la) const { l.init(rx, g, col0, la, kend, kbeg); }
 };
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
@@ -205,13 +233,28 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
   p.kbeg = 0;
   p.kend = a.K;
   float* out = a.Out;
+  int chunk_i = blockIdx.x;
   if ((PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP) && a.ksplit > 1) {
+    // K slice of this workgroup: the generic pass has slices in gridDim.y; the tap-major pass has a flat
+    // grid in which the last chunk, if it holds less work, is cut into proportionally fewer slices
+    int slice = blockIdx.y, ns = a.ksplit;
+    if (PASS == PASS_WGRAD_TAP) {
+      const int b = blockIdx.x, nfull = (a.n_chunks - 1) * a.ksplit;
+      if (b < nfull) {
+        chunk_i = b / a.ksplit;
+        slice = b - chunk_i * a.ksplit;
+      } else {
+        chunk_i = a.n_chunks - 1;
+        slice = b - nfull;
+        ns = a.ks_last;
+      }
+    }
     const int nkt = (a.K + BK - 1) / BK;
-    const int t0 = (int)((long long)nkt * blockIdx.y / a.ksplit);
-    const int t1 = (int)((long long)nkt * (blockIdx.y + 1) / a.ksplit);
+    const int t0 = (int)((long long)nkt * slice / ns);
+    const int t1 = (int)((long long)nkt * (slice + 1) / ns);
     p.kbeg = t0 * BK;
     p.kend = t1 * BK < a.K ? t1 * BK : a.K;
-    out += (size_t)blockIdx.y * a.M * a.Ncols;
+    out += (size_t)slice * a.M * a.Ncols;
   }
   p.rc = make_rsrc(out, a.bytesOut);
   if (PASS == PASS_FWD || PASS == PASS_FWD_TAP) {
@@ -228,7 +271,7 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
   }
   if (PASS == PASS_WGRAD_TAP)
     walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.g.KK, a.total_units,
-                              a.chunk_units);
+                              a.chunk_units, chunk_i);
   else
     walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
 }
@@ -327,19 +370,32 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   if (total > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
   a.total_units = (int)total;
   const long long slots = ctx->cus;   // one 512-thread workgroup per compute unit
-  int grid, ksplit = 1;
+  int grid, ksplit = 1, grid_y = 1;
   float* final_out = a.Out;
   const int final_beta = a.beta;
+  a.n_chunks = 1;
+  a.ks_last = 1;
   if (PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP) {
     // one full-width sub-tile per workgroup, then as many K slices as fill the chip
     const int chunk = PASS == PASS_WGRAD_TAP ? a.chunk_units : 2 * NTMAX;
     grid = (int)((total + chunk - 1) / chunk);
     const int nkt = (a.K + BK - 1) / BK;
-    long long s = slots / grid;
+    long long s = PASS == PASS_WGRAD_TAP ? slots * chunk / total : slots / grid;
     if (s > nkt / 4) s = nkt / 4;
     if (s > 1024) s = 1024;
     if (s < 1) s = 1;
     ksplit = (int)s;
+    grid_y = ksplit;
+    if (PASS == PASS_WGRAD_TAP) {
+      // the last chunk holds rem <= chunk units: give it that share of the slices
+      const int rem = (int)(total - (long long)(grid - 1) * chunk);
+      auto last = [&](int sf) { const int l = (sf * rem + chunk - 1) / chunk; return l < 1 ? 1 : l; };
+      while (ksplit > 1 && (long long)(grid - 1) * ksplit + last(ksplit) > slots) --ksplit;
+      a.n_chunks = grid;
+      a.ks_last = last(ksplit);
+      if (ksplit > 1) grid = (grid - 1) * ksplit + a.ks_last;
+      grid_y = 1;
+    }
     if (ksplit > 1) {
       const size_t need = (size_t)ksplit * a.M * a.Ncols * sizeof(float);
       int st = ensure_workspace(ctx, need);
@@ -351,8 +407,8 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     grid = (int)(total < slots ? total : slots);
   }
   a.ksplit = ksplit;
-  dim3 g(grid, ksplit, 1), b(512, 1, 1);
-  constexpr bool kUsesFlag = PASS == PASS_FWD || PASS == PASS_WGRAD;   // the other passes have one variant
+  dim3 g(grid, grid_y, 1), b(512, 1, 1);
+  constexpr bool kUsesFlag = PASS == PASS_FWD || PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP;   // the other passes have one variant
   if (flag || !kUsesFlag) {
     hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, true>), g, b, 0, ctx->stream, a);
   } else if constexpr (kUsesFlag) {
@@ -360,11 +416,19 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   }
   LNN_HIP(hipGetLastError());
   if (ksplit > 1) {
-    const int n = a.M * a.Ncols;
-    hipLaunchKernelGGL(reduce_partials, dim3((n + 31) / 32), dim3(256), 0, ctx->stream, final_out,
-                       static_cast<const float*>(ctx->ws), n, ksplit, final_beta, a.Ncols,
-                       make_fastdiv((uint32_t)a.Ncols), make_fastdiv((uint32_t)a.g.C), a.g.KK,
-                       PASS == PASS_WGRAD_TAP ? 1 : 0);
+    ReduceArgs r;
+    r.n = a.M * a.Ncols; r.slices = ksplit; r.slices_last = ksplit; r.beta = final_beta; r.ncols = a.Ncols;
+    r.KK = a.g.KK; r.permute = PASS == PASS_WGRAD_TAP ? 1 : 0;
+    r.bm_log = WM == 4 ? 7 : (WM == 2 ? 6 : 5); r.uw_log = WN == 4 ? 7 : (WN == 2 ? 6 : 5);
+    r.per_mt = 0; r.last_unit0 = 0x7fffffff;
+    if (PASS == PASS_WGRAD_TAP) {
+      r.slices_last = a.ks_last;
+      r.per_mt = a.g.KK * a.n_units;
+      r.last_unit0 = (a.n_chunks - 1) * a.chunk_units;
+    }
+    r.dN = make_fastdiv((uint32_t)a.Ncols); r.dC = make_fastdiv((uint32_t)a.g.C);
+    hipLaunchKernelGGL(reduce_partials, dim3((r.n + 31) / 32), dim3(256), 0, ctx->stream, final_out,
+                       static_cast<const float*>(ctx->ws), r);
     LNN_HIP(hipGetLastError());
   }
   return LNN_OK;
@@ -469,8 +533,10 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   a.beta = beta ? 1 : 0;
   // pixel-major loaders when the channels fill whole units of the tile shape chosen for O
   const int unit = g.O > 64 ? 32 : (g.O > 32 ? 64 : 128);
-  if (g.C % unit == 0) return launch_by_m<PASS_WGRAD_TAP>(ctx, a, false);
-  return launch_by_m<PASS_WGRAD>(ctx, a, g.OHW % 4 == 0 && aligned16(dY));
+  // ... and a K step of pixels never wraps around an image more than once
+  const bool vec = g.OHW % 4 == 0 && aligned16(dY);
+  if (g.C % unit == 0 && BK / g.OW + 1 <= g.OH) return launch_by_m<PASS_WGRAD_TAP>(ctx, a, vec);
+  return launch_by_m<PASS_WGRAD>(ctx, a, vec);
 }
 
 }  // namespace lnn

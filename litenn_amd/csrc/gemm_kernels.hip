@@ -5,6 +5,10 @@
 
 #include "common.hpp"
 
+#ifndef LNN_STAGES_GEMM
+#define LNN_STAGES_GEMM 2
+#endif
+
 namespace lnn {
 
 struct GemmArgs {
@@ -24,9 +28,10 @@ struct GemmArgs {
 template <int WM, int NTMAX, bool TA, bool TB, int MODE>
 struct GemmCfg {
   static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
-  static constexpr int SA = LdsSize<!TA, BM>::value;
-  static constexpr int SB = LdsSize<TB, BNMAX>::value;
-  static constexpr int STAGES = 2;
+  // direct transfers fill unpadded tiles and run three stages deep
+  static constexpr int SA = MODE == 2 ? BM * BK : LdsSize<!TA, BM>::value;
+  static constexpr int SB = MODE == 2 ? BNMAX * BK : LdsSize<TB, BNMAX>::value;
+  static constexpr int STAGES = MODE == 2 ? LNN_STAGES_GEMM : 2;
 };
 
 // A operand: !TA -> A[M][K] row-major, K-contiguous; TA -> stored [K][M].

@@ -182,6 +182,7 @@ struct DirectKC {
   static constexpr bool KC = true, DIRECT = true;
   static constexpr int LAYOUT = LAY_KC_SWZ;
   static constexpr int NB = R / 8, E = (NB + 3) / 4;
+  static constexpr int NLD = NB % 4 == 0 ? E : -1;   // transfers per wavefront and K step (-1: differs between wavefronts)
   static_assert(R % 8 == 0, "whole 8-row blocks");
   rsrc_t rs;
   uint32_t voff[E];
@@ -214,6 +215,7 @@ struct DirectMC {
   static constexpr bool KC = false, DIRECT = true;
   static constexpr int LAYOUT = LAY_MC_SPLIT;
   static constexpr int NI = BK * R / 256, E = (NI + 3) / 4;
+  static constexpr int NLD = NI % 4 == 0 ? E : -1;
   static_assert(R % 8 == 0, "whole 256-float transfers");
   rsrc_t rs;
   uint32_t voff[E];
@@ -393,6 +395,7 @@ template <int R, bool DIR = false>
 struct ConvFwdBTap {
   static constexpr bool KC = false, DIRECT = DIR;
   static constexpr int CC = (R + 63) / 64;
+  static constexpr int NLD = KR * CC;
   rsrc_t rs;
   int IH, IW, IHW, C, D, KW;
   int base[CC], ih0[CC], iw0[CC];
@@ -473,6 +476,7 @@ template <int R, bool DIR = false>
 struct ConvDgradBTap {
   static constexpr bool KC = false, DIRECT = DIR;
   static constexpr int CC = (R + 63) / 64;
+  static constexpr int NLD = KR * CC;
   rsrc_t rs;
   ktab_t tab;           // one entry per tap of the pixel class: y, z (see ConvDgradB)
   int OH, OW, OHW, O;
@@ -872,6 +876,150 @@ struct ConvWgradTapB {
   }
 };
 
+// The same two operands sent straight into swizzled K-contiguous LDS tiles
+// (LAY_KC_SWZ).  One transfer fills two adjacent tile rows: lanes 0..31 the
+// even one, lanes 32..63 the odd one.  Wavefront w owns the row pairs
+// w, w+4, w+8, ..., so every row a lane ever fills has the same r % 8 = 2w +
+// lane/32: the lane's swizzled position corresponds to one fixed k of the K
+// step, i.e. one pixel to decompose per step, and its rows differ by
+// wave-uniform multiples of 8 planes which ride in the scalar offset.
+__device__ __forceinline__ int wgrad_direct_k() {   // k (0..BK-1) whose swizzled position this lane fills
+  const int lane = threadIdx.x & 63, pos = lane & 31, key = 2 * gwave() + (lane >> 5);
+  return (((pos >> 2) ^ key) << 2) | (pos & 3);
+}
+//
+// The lane's pixel advances by BK per K step.  Its coordinates and the
+// element offsets derived from them are carried along with additions and
+// single wrap tests (which is why these loaders need BK/OW + 1 <= OH): no
+// division or multiplication in the K loop.
+template <int R>
+struct ConvWgradTapADirect {
+  static constexpr bool KC = true, DIRECT = true;
+  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int E = R / 8, NLD = E;
+  static_assert(R % 8 == 0, "whole row pairs for all four wavefronts");
+  rsrc_t rs;
+  int OHW, kend, p, rem, aoff, awrap;   // aoff = img*O*OHW + rem + (row of this lane)*OHW
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int o0, int kend_, int k0) {
+    rs = r;
+    OHW = g.OHW;
+    kend = kend_;
+    awrap = g.O * g.OHW - g.OHW;   // to the same pixel offset in the next image
+    p = k0 + wgrad_direct_k();
+    const uint32_t img = g.dOHW.div((uint32_t)p);
+    rem = p - (int)img * g.OHW;
+    aoff = (int)img * g.O * g.OHW + rem + (o0 + 2 * gwave() + (int)((threadIdx.x & 63) >> 5)) * g.OHW;
+  }
+  __device__ __forceinline__ void issue(int, float* lds, int, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+    // rows past the last output channel are never stored, so they need no mask
+    const uint32_t voff = p < kend ? (uint32_t)aoff * 4u : OOB;
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, voff, (uint32_t)(8 * e * OHW) * 4u);
+    p += BK; rem += BK; aoff += BK;
+    if (rem >= OHW) { rem -= OHW; aoff += awrap; }
+  }
+};
+
+// The same with 128-bit transfers, for OH*OW % 4 == 0 and a 16-byte aligned dY:
+// lane l carries 4-pixel group (l % 8) ^ (l / 8) of row l / 8 of an 8-row block
+// (the layout of DirectKC), wavefront w the blocks w, w+4, ...
+template <int R>
+struct ConvWgradTapA4Direct {
+  static constexpr bool KC = true, DIRECT = true;
+  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int NB = R / 8, E = (NB + 3) / 4;
+  static constexpr int NLD = NB % 4 == 0 ? E : -1;
+  static_assert(R % 8 == 0, "whole 8-row blocks");
+  rsrc_t rs;
+  int OHW, kend, p, rem, aoff, awrap;
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int o0, int kend_, int k0) {
+    rs = r;
+    OHW = g.OHW;
+    kend = kend_;
+    awrap = g.O * g.OHW - g.OHW;
+    const int lane = threadIdx.x & 63, rb = lane >> 3;
+    p = k0 + 4 * ((lane & 7) ^ rb);
+    const uint32_t img = g.dOHW.div((uint32_t)p);
+    rem = p - (int)img * g.OHW;
+    aoff = (int)img * g.O * g.OHW + rem + (o0 + 8 * gwave() + rb) * g.OHW;
+  }
+  __device__ __forceinline__ void issue(int, float* lds, int, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+    const uint32_t voff = p < kend ? (uint32_t)aoff * 4u : OOB;   // kend is a multiple of 4 here: whole groups
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      if (NB % 4 == 0 || wave + 4 * e < NB)
+        buf_load_lds16(rs, lds + (off + (wave + 4 * e) * 8) * BK, voff, (uint32_t)(32 * e * OHW) * 4u);
+    p += BK; rem += BK; aoff += BK;
+    if (rem >= OHW) { rem -= OHW; aoff += awrap; }
+  }
+};
+
+// DIR = false: the same gather through registers (cheaper to issue than
+// transfers into LDS), parked into the same swizzled layout one step later.
+template <int R, bool DIR = true>
+struct ConvWgradTapBDirect {
+  static constexpr bool KC = true, DIRECT = DIR;
+  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int E = R / 8, NLD = E;
+  float v[E];
+  static_assert(R % 8 == 0, "whole row pairs for all four wavefronts");
+  rsrc_t rs;
+  int IH, IW, IHW, OH, OW, kend;
+  int p, oh, ow;            // this lane's output pixel, its row and column inside the image
+  int ih, iw;               // oh*S + kh*D - PADT, ow*S + kw*D - PADL: the input pixel under this group's tap
+  int xoff;                 // its element offset (for the channel of this lane)
+  int qh, rw;               // a K step moves the pixel qh rows and rw columns ahead ...
+  int s_q, s_r, x_step;     // ... i.e. ih by S*qh, iw by S*rw, xoff by S*qh*IW + S*rw
+  int s_OW, s_OH, S, xwrap_w, xwrap_h;   // corrections when the column / the row wraps
+  template <class LA>
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int col0, const LA&, int kend_, int k0) {
+    rs = r;
+    IH = g.IH; IW = g.IW; IHW = g.IHW; OH = g.OH; OW = g.OW; S = g.S;
+    kend = kend_;
+    const int tap = col0 / g.C, c0 = col0 - tap * g.C;
+    const int kh = tap / g.KW, kw = tap - kh * g.KW;
+    qh = BK / g.OW; rw = BK - qh * g.OW;
+    s_q = g.S * qh; s_r = g.S * rw; s_OW = g.S * g.OW; s_OH = g.S * g.OH;
+    x_step = s_q * g.IW + s_r;
+    xwrap_w = g.S * g.IW - s_OW;              // column wrap: one row down, OW columns back
+    xwrap_h = g.C * g.IHW - s_OH * g.IW;      // row wrap: next image, OH rows back
+    p = k0 + wgrad_direct_k();
+    const uint32_t img = g.dOHW.div((uint32_t)p), rem = (uint32_t)p - img * g.OHW;
+    oh = (int)g.dOW.div(rem);
+    ow = (int)rem - oh * g.OW;
+    ih = oh * g.S + kh * g.D - g.PADT;
+    iw = ow * g.S + kw * g.D - g.PADL;
+    xoff = ((int)img * g.C + c0 + 2 * gwave() + (int)((threadIdx.x & 63) >> 5)) * g.IHW + ih * g.IW + iw;
+  }
+  __device__ __forceinline__ void issue(int, float* lds, int, int off) { go<true>(lds, off); }
+  __device__ __forceinline__ void fetch(int) { go<false>(nullptr, 0); }
+  __device__ __forceinline__ void commit(float* lds, int, int off) const {
+    const int wave = gwave(), lane = threadIdx.x & 63;
+#pragma unroll
+    for (int e = 0; e < E; ++e) lds[(off + 8 * e + 2 * wave) * BK + lane] = v[e];
+  }
+  template <bool TO_LDS>
+  __device__ __forceinline__ void go(float* lds, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+    const bool ok = p < kend && (uint32_t)ih < (uint32_t)IH && (uint32_t)iw < (uint32_t)IW;
+    const uint32_t voff = ok ? (uint32_t)xoff * 4u : OOB;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const uint32_t soff = (uint32_t)(8 * e * IHW) * 4u;
+      if (TO_LDS)
+        buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, voff, soff);
+      else
+        v[e] = buf_load_s(rs, voff, soff);
+    }
+    p += BK; oh += qh; ow += rw; ih += s_q; iw += s_r; xoff += x_step;
+    if (ow >= OW) { ow -= OW; ++oh; iw -= s_OW; ih += S; xoff += xwrap_w; }
+    if (oh >= OH) { oh -= OH; ih -= s_OH; xoff += xwrap_h; }
+  }
+};
+
 // ---------------------------------------------------------------------------
 // Output mapping.  plain: off = m*ld + n.  NCHW image tensor with the GEMM
 // column n = (img, pixel): off = (img*Mtot + m)*HW + pixel.
@@ -1006,12 +1154,34 @@ struct layout_of : std::integral_constant<int, T::KC ? LAY_KC : LAY_MC> {};
 template <class T>
 struct layout_of<T, std::void_t<decltype(T::LAYOUT)>> : std::integral_constant<int, T::LAYOUT> {};
 
-// End of a phase.  All of this wavefront's LDS writes (lgkmcnt) and
-// global -> LDS transfers (vmcnt) have landed before it reports to the barrier.
-__device__ __forceinline__ void phase_barrier() {
+// End of a phase.  The barrier is issued by hand so that it waits for exactly
+// what the schedule needs: LDS operations of this wavefront (fragment reads,
+// parked operands) always; its global -> LDS transfers only where stated.
+// Nothing may be scheduled across it: the MFMAs of a phase must not sink into
+// the other group's phase.
+__device__ __forceinline__ void barrier_after_compute() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+__device__ __forceinline__ void barrier_after_issue() {
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
+}
+// All global -> LDS transfers of this wavefront have landed (the compiler
+// tracks register loads by itself, not these).
+template <bool ANY_DIRECT>
+__device__ __forceinline__ void wait_transfers() {
+  if (ANY_DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+template <class LB, class LA>
+__device__ __forceinline__ void issue_b(LB& lb, int k0, float* lds, int ld, int off, LA& la) {
+  if constexpr (needs_a<LB>::value)
+    lb.issue(k0, lds, ld, off, la);
+  else
+    lb.issue(k0, lds, ld, off);
 }
 
 // Body of one group (G = 0 or 1) for one sub-tile: BM = 32*WM rows shared by
@@ -1024,8 +1194,6 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
   using LA = typename P::template LA<HALF>;
   using LB = typename P::template LB<BN>;
   constexpr int LAY_A = layout_of<LA>::value, LAY_B = layout_of<LB>::value;
-  constexpr bool DIRECT = is_direct<LA>::value;
-  static_assert(is_direct<LA>::value == is_direct<LB>::value, "both loaders of a kernel move data the same way");
   constexpr int LDA = LAY_A == LAY_KC ? LDK : (LAY_A == LAY_KC_SWZ ? BK : BM);
   constexpr int LDB = LAY_B == LAY_KC ? LDK : (LAY_B == LAY_KC_SWZ ? BK : BNTOT);
   const int wave = gwave(), lane = threadIdx.x & 63;
@@ -1049,65 +1217,73 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
 
   // Each K step t has two phases separated by barriers.  Group 0 computes in
   // the first and moves data in the second; group 1 the other way round.
-  if constexpr (DIRECT) {
-    // "moving data" in step t = sending K step t+1 from global memory into the
-    // other LDS stage, which was last read for step t-1
-    if (nk > 0) {
-      la.issue(kbeg, ldsA, LDA, G * HALF);
-      if (NT > 0) lb.issue(kbeg, ldsB, LDB, COFF);
+  constexpr int ST = P::STAGES;
+  constexpr bool DA = is_direct<LA>::value, DB = is_direct<LB>::value;
+  static_assert(ST == 3 || (!DA && !DB) || (DA && DB), "a mix of direct and register-staged loaders needs three stages");
+  // request: ask global memory for a K step, into an LDS stage (direct loader) or into registers;
+  // land: park a register-staged K step in its LDS stage
+  auto request = [&](int k0, int stage) {
+    if constexpr (DA) la.issue(k0, ldsA + stage * strideA, LDA, G * HALF); else la.fetch(k0);
+    if constexpr (NT > 0) {
+      if constexpr (DB) issue_b(lb, k0, ldsB + stage * strideB, LDB, COFF, la); else fetch_b(lb, k0, la);
     }
-    phase_barrier();
+  };
+  auto land = [&](int stage) {
+    if constexpr (!DA) la.commit(ldsA + stage * strideA, LDA, G * HALF);
+    if constexpr (NT > 0 && !DB) lb.commit(ldsB + stage * strideB, LDB, COFF);
+  };
+  auto compute = [&](int stage) {
+    if constexpr (NT > 0)
+      mma_stage<NTC, LAY_A, LAY_B, BM, RB>(ldsA + stage * strideA, ldsBr + stage * strideB, acc, arow, brow);
+  };
+  if constexpr (DA && DB && ST == 2) {
+    // "moving data" in step t = sending K step t+1 into the other LDS stage
+    // (last read for step t-1) and waiting for it to land
+    if (nk > 0) request(kbeg, 0);
+    barrier_after_issue();
     for (int t = 0; t < nk; ++t) {
       const int cur = t & 1;
 #pragma unroll
       for (int phase = 0; phase < 2; ++phase) {
         if (phase == G) {
-          if (NT > 0)
-            mma_stage<NTC, LAY_A, LAY_B, BM, RB>(ldsA + cur * strideA, ldsBr + cur * strideB, acc, arow, brow);
-        } else if (t + 1 < nk) {
-          la.issue(kbeg + (t + 1) * BK, ldsA + (cur ^ 1) * strideA, LDA, G * HALF);
-          if (NT > 0) lb.issue(kbeg + (t + 1) * BK, ldsB + (cur ^ 1) * strideB, LDB, COFF);
+          compute(cur);
+          barrier_after_compute();
+        } else {
+          if (t + 1 < nk) request(kbeg + (t + 1) * BK, cur ^ 1);
+          barrier_after_issue();
         }
-        phase_barrier();
       }
     }
   } else {
-    // "moving data" in step t = parking K step t+1 (in registers since step
-    // t-1) in the other LDS stage, then fetching K step t+2 into registers
+    // "moving data" in step t = completing K step t+1 (requested in step t-1:
+    // wait for the transfers, park what sits in registers) in the stage last
+    // read for step t-2 (ST = 3) or t-1 (ST = 2), then requesting K step t+2;
+    // a direct request targets the stage last read for step t-1, which is why
+    // direct loaders need three stages here
     if (nk > 0) {
-      la.fetch(kbeg);
-      if (NT > 0) fetch_b(lb, kbeg, la);
-      la.commit(ldsA, LDA, G * HALF);
-      if (NT > 0) lb.commit(ldsB, LDB, COFF);
+      request(kbeg, 0);
+      wait_transfers<DA || DB>();
+      land(0);
     }
-    if (1 < nk) {
-      la.fetch(kbeg + BK);
-      if (NT > 0) fetch_b(lb, kbeg + BK, la);
-    }
-    __syncthreads();
+    if (nk > 1) request(kbeg + BK, 1);
+    barrier_after_compute();   // LDS writes done; transfers of step 1 stay in flight
+    int cur = 0;
     for (int t = 0; t < nk; ++t) {
-      const int cur = t & 1;
+      const int nxt = cur + 1 == ST ? 0 : cur + 1, nn = nxt + 1 == ST ? 0 : nxt + 1;
 #pragma unroll
       for (int phase = 0; phase < 2; ++phase) {
         if (phase == G) {
-          if (NT > 0)
-            mma_stage<NTC, LAY_A, LAY_B, BM, RB>(ldsA + cur * strideA, ldsBr + cur * strideB, acc, arow, brow);
+          compute(cur);
         } else {
           if (t + 1 < nk) {
-            la.commit(ldsA + (cur ^ 1) * strideA, LDA, G * HALF);
-            if (NT > 0) lb.commit(ldsB + (cur ^ 1) * strideB, LDB, COFF);
+            wait_transfers<DA || DB>();
+            land(nxt);
           }
-          if (t + 2 < nk) {
-            la.fetch(kbeg + (t + 2) * BK);
-            if (NT > 0) fetch_b(lb, kbeg + (t + 2) * BK, la);
-          }
+          if (t + 2 < nk) request(kbeg + (t + 2) * BK, nn);
         }
-        // the phase ends only when all of its MFMAs have been issued: do not let
-        // the scheduler sink them below the barrier into the other group's phase
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
+        barrier_after_compute();
       }
+      cur = nxt;
     }
   }
 
@@ -1216,13 +1392,14 @@ __device__ __forceinline__ void walk_units(const P& p, float* ldsA, float* ldsB,
 // convolution tap): a group's columns never cross a segment, the two groups
 // of a sub-tile may sit in different segments of the same M tile.
 // Units are numbered (mt * segs_per_mt + segment) * seg_units + unit; workgroup
-// b takes units [b*chunk, (b+1)*chunk).
+// chunk_index takes units [chunk_index*chunk, (chunk_index+1)*chunk).
 template <int WM, int NTMAX, class P>
 __device__ __forceinline__ void walk_units_seg(const P& p, float* ldsA, float* ldsB, int strideA, int strideB,
-                                               int seg_units, int segs_per_mt, int total_units, int chunk) {
+                                               int seg_units, int segs_per_mt, int total_units, int chunk,
+                                               int chunk_index) {
   constexpr int WN = 4 / WM;
   const int per_mt = seg_units * segs_per_mt;
-  int pos = (int)blockIdx.x * chunk;
+  int pos = chunk_index * chunk;
   const int end = pos + chunk < total_units ? pos + chunk : total_units;
   while (pos < end) {
     const int mt = pos / per_mt;
