@@ -29,6 +29,13 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 2.4 GHz x 256 flop/clk/CU
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch from hardware counters (FETCH_SIZE + WRITE_SIZE, each scaled by its reading for a plain
+# copy of known size), measured separately under rocprofv3 --pmc; keyed by workload and pass.  A pass that has
+# not been measured reports null.
+MEASURED_TRAFFIC_BYTES = {
+    'cfg3_vgg3x3': {'fwd': 316.1e6, 'dX': 385.1e6, 'dW': 236.6e6 + 33.6e6},   # dW = wgrad kernel + slice reduction
+}
+
 CONV_CONFIGS = {
     # name: (x shape, w shape, stride, dilation, padding, seed)
     'cfg1_stem3x3': ((8, 3, 64, 64), (32, 3, 3, 3), 1, 1, 'same', 0),
@@ -137,10 +144,12 @@ def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
     t_hbm = bytes_pass[dom] / (PEAK_HBM_GBS * 1e6)
     if t_mfma >= t_hbm:
         roof = {'bound': 'mfma', 'kernel': dom, 'achieved': per_pass[dom]['tflops'], 'peak': PEAK_FP32_MFMA_TFLOPS,
-                'unit': 'TFLOP/s', 'frac': per_pass[dom]['frac_mfma'], 'traffic': None}
+                'unit': 'TFLOP/s', 'frac': per_pass[dom]['frac_mfma'],
+                'traffic': MEASURED_TRAFFIC_BYTES.get(name, {}).get(dom)}
     else:
         roof = {'bound': 'hbm', 'kernel': dom, 'achieved': per_pass[dom]['alg_gbs'], 'peak': PEAK_HBM_GBS,
-                'unit': 'GB/s', 'frac': per_pass[dom]['frac_hbm'], 'traffic': None}
+                'unit': 'GB/s', 'frac': per_pass[dom]['frac_hbm'],
+                'traffic': MEASURED_TRAFFIC_BYTES.get(name, {}).get(dom)}
 
     # parity on the very tensors that were timed (fresh outputs, no accumulation history)
     dX.zero()
@@ -306,6 +315,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--all', action='store_true', help='also measure every benchmark configuration')
+    ap.add_argument('--copy-calibration', action='store_true',
+                    help='run only a plain device copy of 256 MiB (three launches of the element-wise kernel) and exit: '
+                         'the reference reading for the FETCH_SIZE / WRITE_SIZE counters')
     ap.add_argument('--config', default='cfg3_vgg3x3', choices=list(CONV_CONFIGS) + ['cfg2_matmul', 'cfg5_encoder'],
                     help='workload of the JSON line (default: the headline configuration)')
     args = ap.parse_args()
@@ -314,6 +326,16 @@ def main():
     from litenn_amd.core.hip import api
     if api.device_count() < 1:
         sys.exit('bench.py needs an MI355X: no HIP device is visible')
+    if args.copy_calibration:
+        n = 1 << 26
+        src, dst = Dev(api, shape=(n,)), Dev(api, shape=(n,))
+        src.zero()
+        for _ in range(3):
+            api.ew_fwd(0, api.EW_ADD_CONST, n, src.ptr, dst.ptr, 0.0, 0)
+        api.synchronize(0)
+        print(json.dumps({'copy_calibration': {'kernel': 'ew_fwd_kernel', 'launches': 3, 'read_bytes': 4 * n,
+                                               'write_bytes': 4 * n}}), flush=True)
+        return
     if args.all:
         os.makedirs(os.path.join(ROOT, 'gpurun_out'), exist_ok=True)
         with open(os.path.join(ROOT, 'gpurun_out', 'bench_all.jsonl'), 'w') as f:
