@@ -246,6 +246,34 @@ def test_conv_channel_multiples_of_32_integer_exact(hip):
     assert cnt > 600
 
 
+def test_conv_wide_images_pixel_walk_integer_exact(hip):
+    """The pixel-major wgrad loaders carry each lane's pixel forward by 32
+    per K step with additions and wrap tests: images wider than, equal to and
+    narrower than a K step, rows that wrap in the middle of a step, several
+    images per K slice, output planes whose size is and is not a multiple of 4."""
+    rs = np.random.RandomState(21)
+    shapes = [(2, 32, 9, 40), (3, 32, 40, 37), (1, 64, 64, 64), (2, 32, 5, 33), (5, 32, 6, 32), (2, 64, 33, 8),
+              (7, 32, 7, 7), (1, 32, 2, 100), (4, 96, 12, 12)]
+    for xs in shapes:
+        for s, d, ks, padding in ((1, 1, 3, 'same'), (2, 1, 3, 1), (1, 2, 2, 'valid'), (1, 1, 1, 'same'), (2, 1, 5, 2)):
+            for oc in (32, 40, 130):
+                try:
+                    ci = info_conv2d(xs[2], xs[3], ks, ks, s, d, padding)
+                except ValueError:
+                    continue
+                if ci.OH <= 0 or ci.OW <= 0:
+                    continue
+                say(f'conv walk x={xs} oc={oc} s={s} d={d} ks={ks} pad={padding}')
+                x = rs.randint(6, size=xs).astype(np.float32)
+                w = rs.randint(6, size=(oc, xs[1], ks, ks)).astype(np.float32)
+                dy = rs.randint(6, size=(xs[0], oc, ci.OH, ci.OW)).astype(np.float32)
+                ry, rdx, rdw = conv2d_all(x, w, dy, s, d, padding)
+                y, dx, dw = _run_conv(hip, x, w, dy, s, d, padding, prefill=None)
+                assert np.array_equal(y, ry), ('fwd', xs, oc, s, d, ks, padding)
+                assert np.array_equal(dx, rdx), ('dX', xs, oc, s, d, ks, padding)
+                assert np.array_equal(dw, rdw), ('dW', xs, oc, s, d, ks, padding)
+
+
 # benchmark geometries at a reduced batch (the oracle materialises im2col in fp64)
 _BENCH = {
     'cfg1': ((8, 3, 64, 64), (32, 3, 3, 3), 1, 1, 'same', 0),
