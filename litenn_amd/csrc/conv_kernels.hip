@@ -34,6 +34,7 @@ struct ConvArgs {
   int beta;
   int n_units, total_units;
   int ksplit;        // wgrad: number of K slices (tap-major: of every chunk but the last)
+  size_t ws_used;    // bytes at the front of the scratch buffer that hold this call's permuted weights
   int n_chunks, ks_last;   // tap-major wgrad: chunks of chunk_units units; K slices of the last, possibly shorter one
   FastDiv dC;        // tap-major wgrad: divide a column index by the channel count
   int chunk_units;   // tap-major wgrad: units per workgroup
@@ -84,16 +85,16 @@ __global__ void build_ktable(KEntry* tab, int K, int Kpad, int mode, ConvGeom g,
   tab[k] = e;
 }
 
-// out[f(i)] (+)= sum over slices of part[slice][i], slices added in a fixed order.
-// A block covers 32 consecutive i (one 128-byte line per slice row) with 8
-// lanes per i striding over the slices.  Elements of units >= last_unit0 (unit
-// = (m >> bm_log) * per_mt + (col >> uw_log)) have only slices_last slices.
-// permute: partial column tap*C + c of row m goes to out[m][c][tap]
-// (tap-major wgrad columns back to OIHW).
+// out[map(m, col)] (+)= sum over slices of part[slice][m][col], slices added in a
+// fixed order.  A block covers 32 consecutive elements (one 128-byte line per
+// slice row) with 8 lanes per element striding over the slices.  Elements of
+// units >= last_unit0 (unit = (m >> bm_log) * per_mt + (col >> uw_log)) have
+// only slices_last slices.
 struct ReduceArgs {
-  int n, slices, slices_last, beta, ncols, KK, permute;
+  int n, slices, slices_last, beta, ncols;
   int bm_log, uw_log, per_mt, last_unit0;
-  FastDiv dN, dC;
+  FastDiv dN;
+  OutMap om;
 };
 __global__ __launch_bounds__(256) void reduce_partials(float* out, const float* part, ReduceArgs a) {
   __shared__ float red[8][33];
@@ -113,11 +114,7 @@ __global__ __launch_bounds__(256) void reduce_partials(float* out, const float* 
   if (ls == 0 && i < a.n) {
 #pragma unroll
     for (int k = 1; k < 8; ++k) s += red[k][li];
-    uint32_t o = (uint32_t)i;
-    if (a.permute) {
-      const uint32_t tap = a.dC.div(col), ch = col - tap * a.dC.d;
-      o = m * (uint32_t)a.ncols + ch * (uint32_t)a.KK + tap;
-    }
+    const uint32_t o = a.om.col(col) + m * (uint32_t)a.om.ld;
     out[o] = a.beta ? out[o] + s : s;
   }
 }
@@ -220,6 +217,28 @@ struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A& la) const { l.init(rx, g, col0, la, kend, kbeg); }
 };
 
+// Where GEMM element (m, column) of a pass lives in its output tensor.
+__host__ __device__ inline OutMap plain_map(int ncols) {
+  OutMap om;
+  om.nchw = 0; om.ld = ncols; om.mtot = 0; om.dHW = FastDiv{0, 0, 1};
+  om.dCW = FastDiv{0, 0, 1}; om.s = 0; om.iw = 0; om.org = 0;
+  return om;
+}
+template <int PASS>
+__host__ __device__ inline OutMap final_map(const ConvArgs& a) {
+  OutMap om = plain_map(a.Ncols);
+  if (PASS == PASS_FWD || PASS == PASS_FWD_TAP) {
+    om.nchw = 1; om.ld = a.g.OHW; om.mtot = a.g.O; om.dHW = a.g.dOHW;
+  } else if (PASS == PASS_DGRAD || PASS == PASS_DGRAD_TAP) {
+    om.nchw = 3; om.ld = a.full_IHW; om.mtot = a.g.C; om.dHW = a.g.dIHW;
+    om.dCW = a.g.dIW; om.s = a.cls_s; om.iw = a.full_IW; om.org = a.cls_org;
+  } else if (PASS == PASS_WGRAD_TAP) {
+    // GEMM column tap*C + c lands in dW[o][c][tap]
+    om.nchw = 2; om.ld = a.Ncols; om.mtot = a.g.KK; om.dHW = a.dC;
+  }
+  return om;
+}
+
 template <int PASS, int WM, int NTMAX, bool FLAG>
 __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
   using Cfg = ConvCfg<PASS, WM, NTMAX, FLAG>;
@@ -234,8 +253,8 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
   p.kend = a.K;
   float* out = a.Out;
   int chunk_i = blockIdx.x;
-  if ((PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP) && a.ksplit > 1) {
-    // K slice of this workgroup: the generic pass has slices in gridDim.y; the tap-major pass has a flat
+  if (a.ksplit > 1) {
+    // K slice of this workgroup: slices are in gridDim.y, except that the tap-major wgrad pass has a flat
     // grid in which the last chunk, if it holds less work, is cut into proportionally fewer slices
     int slice = blockIdx.y, ns = a.ksplit;
     if (PASS == PASS_WGRAD_TAP) {
@@ -257,18 +276,8 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
     out += (size_t)slice * a.M * a.Ncols;
   }
   p.rc = make_rsrc(out, a.bytesOut);
-  if (PASS == PASS_FWD || PASS == PASS_FWD_TAP) {
-    p.om.nchw = 1; p.om.ld = a.g.OHW; p.om.mtot = a.g.O; p.om.dHW = a.g.dOHW;
-  } else if (PASS == PASS_DGRAD || PASS == PASS_DGRAD_TAP) {
-    p.om.nchw = 3; p.om.ld = a.full_IHW; p.om.mtot = a.g.C; p.om.dHW = a.g.dIHW;
-    p.om.dCW = a.g.dIW; p.om.s = a.cls_s; p.om.iw = a.full_IW; p.om.org = a.cls_org;
-  } else if (PASS == PASS_WGRAD_TAP && a.ksplit <= 1) {
-    // GEMM column tap*C + c lands in dW[o][c][tap]; split-K partials stay in
-    // GEMM order (coalesced) and the slice reduction does this permutation
-    p.om.nchw = 2; p.om.ld = a.Ncols; p.om.mtot = a.g.KK; p.om.dHW = a.dC;
-  } else {
-    p.om.nchw = 0; p.om.ld = a.Ncols; p.om.mtot = 0; p.om.dHW = FastDiv{0, 0, 1};
-  }
+  // split-K partials stay in GEMM order (coalesced); the slice reduction applies the final mapping
+  p.om = a.ksplit > 1 ? plain_map(a.Ncols) : final_map<PASS>(a);
   if (PASS == PASS_WGRAD_TAP)
     walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.g.KK, a.total_units,
                               a.chunk_units, chunk_i);
@@ -338,9 +347,12 @@ static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const PixelCla
 // Channel-permuted copy of the weights in the library's scratch buffer (valid
 // until the next call that uses scratch; the stream orders it before its reader).
 static int permuted_weights(DeviceCtx* ctx, const ConvGeom& g, const float* W, int mode, const PixelClass& pc,
-                            const float** out) {
+                            const float** out, size_t* used) {
   const int n = g.O * g.C * (mode == 0 ? g.KK : pc.nkh * pc.nkw);
-  int st = ensure_workspace(ctx, (size_t)(n > 0 ? n : 1) * sizeof(float));
+  *used = ((size_t)(n > 0 ? n : 1) * sizeof(float) + 255) & ~(size_t)255;
+  // leave room behind the weights for the split-K partial sums of the same call (at most one full
+  // 32768-element sub-tile per workgroup slot), so that the buffer is not reallocated under them
+  int st = ensure_workspace(ctx, *used + (size_t)ctx->cus * 32768 * sizeof(float));
   if (st != LNN_OK) return st;
   if (n > 0) {
     hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream,
@@ -405,6 +417,27 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     }
   } else {
     grid = (int)(total < slots ? total : slots);
+    // Few output tiles (small images, deep layers): a workgroup's share would be a sliver of a sub-tile and
+    // most of its time data movement.  Cut the output into full sub-tiles instead and split K over the
+    // workgroups that are left, as wgrad does.
+    const int chunk = 2 * NTMAX;
+    const long long chunks = (total + chunk - 1) / chunk;
+    const int nkt = (a.K + BK - 1) / BK;
+    if (total < slots * (chunk / 2 + 1) && chunks * 2 <= slots && nkt >= 16) {
+      long long s = slots / chunks;
+      if (s > nkt / 8) s = nkt / 8;
+      if (s > 1) {
+        ksplit = (int)s;
+        grid = (int)chunks;
+        grid_y = ksplit;
+        const size_t need = (size_t)ksplit * a.M * a.Ncols * sizeof(float);
+        // the scratch buffer may already hold this call's permuted weights: keep them in front
+        int st = ensure_workspace(ctx, a.ws_used + need);
+        if (st != LNN_OK) return st;
+        a.Out = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + a.ws_used);
+        a.beta = 0;
+      }
+    }
   }
   a.ksplit = ksplit;
   dim3 g(grid, grid_y, 1), b(512, 1, 1);
@@ -418,7 +451,6 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   if (ksplit > 1) {
     ReduceArgs r;
     r.n = a.M * a.Ncols; r.slices = ksplit; r.slices_last = ksplit; r.beta = final_beta; r.ncols = a.Ncols;
-    r.KK = a.g.KK; r.permute = PASS == PASS_WGRAD_TAP ? 1 : 0;
     r.bm_log = WM == 4 ? 7 : (WM == 2 ? 6 : 5); r.uw_log = WN == 4 ? 7 : (WN == 2 ? 6 : 5);
     r.per_mt = 0; r.last_unit0 = 0x7fffffff;
     if (PASS == PASS_WGRAD_TAP) {
@@ -426,9 +458,10 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
       r.per_mt = a.g.KK * a.n_units;
       r.last_unit0 = (a.n_chunks - 1) * a.chunk_units;
     }
-    r.dN = make_fastdiv((uint32_t)a.Ncols); r.dC = make_fastdiv((uint32_t)a.g.C);
+    r.dN = make_fastdiv((uint32_t)a.Ncols);
+    r.om = final_map<PASS>(a);
     hipLaunchKernelGGL(reduce_partials, dim3((r.n + 31) / 32), dim3(256), 0, ctx->stream, final_out,
-                       static_cast<const float*>(ctx->ws), r);
+                       static_cast<const float*>(a.Out), r);
     LNN_HIP(hipGetLastError());
   }
   return LNN_OK;
@@ -445,6 +478,7 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta) {
   ConvArgs a;
+  a.ws_used = 0;
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !W || !Y) return set_error(LNN_ERR_INVALID, "conv2d_fwd: null pointer");
@@ -457,7 +491,7 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   a.M = g.O; a.Ncols = g.N * g.OHW; a.K = g.C * g.KK;
   a.beta = beta ? 1 : 0;
   if (g.C % BK == 0) {
-    st = permuted_weights(ctx, g, W, 0, PixelClass{}, &a.W);
+    st = permuted_weights(ctx, g, W, 0, PixelClass{}, &a.W, &a.ws_used);
     if (st != LNN_OK) return st;
     return launch_by_m<PASS_FWD_TAP>(ctx, a, true);
   }
@@ -486,6 +520,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
       const int nt = pc.nkh * pc.nkw;
       if (nt == 0 && beta) continue;                        // nothing to add; without beta the class is zero-filled
       ConvArgs a;
+      a.ws_used = 0;
       a.g = full;
       ConvGeom& g = a.g;
       g.IH = (full.IH - pc.h0 + S - 1) / S;
@@ -501,7 +536,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
       a.M = g.C; a.Ncols = g.N * g.IHW; a.K = g.O * nt;
       a.beta = beta ? 1 : 0;
       if (g.O % BK == 0) {
-        st = permuted_weights(ctx, full, W, 1, pc, &a.W);
+        st = permuted_weights(ctx, full, W, 1, pc, &a.W, &a.ws_used);
         if (st != LNN_OK) return st;
         a.bytesW = (uint32_t)((uint64_t)g.O * g.C * nt * 4);
         st = get_table(ctx, full, 2, pc, &a.tab);
@@ -519,6 +554,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
 
 int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
   ConvArgs a;
+  a.ws_used = 0;
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");

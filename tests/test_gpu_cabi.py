@@ -274,6 +274,31 @@ def test_conv_wide_images_pixel_walk_integer_exact(hip):
                 assert np.array_equal(dw, rdw), ('dW', xs, oc, s, d, ks, padding)
 
 
+def test_conv_few_tiles_split_k_integer_exact(hip):
+    """Deep layers on small images have a long K and few output tiles: forward
+    and dgrad then split K over the idle compute units and a second kernel
+    sums the slices into the NCHW (or class-strided) output.  Exact on
+    integers, with and without accumulation, stride 1 and 2, channel counts on
+    and off the multiple-of-32 kernels."""
+    rs = np.random.RandomState(31)
+    cases = [((2, 128, 16, 16), (256, 128, 5, 5), 2, 1, 2), ((2, 256, 8, 8), (512, 256, 5, 5), 2, 1, 2),
+             ((1, 256, 6, 6), (96, 256, 3, 3), 1, 1, 'same'), ((3, 130, 5, 7), (70, 130, 3, 3), 1, 1, 'same'),
+             ((1, 512, 4, 4), (40, 512, 1, 1), 1, 1, 'valid'), ((2, 96, 9, 9), (33, 96, 3, 3), 3, 2, 'same')]
+    for i, (xs, ws, s, d, padding) in enumerate(cases):
+        say(f'conv split-K x={xs} w={ws} s={s} d={d} pad={padding}')
+        x = rs.randint(4, size=xs).astype(np.float32)
+        w = rs.randint(4, size=ws).astype(np.float32)
+        ci = info_conv2d(xs[2], xs[3], ws[2], ws[3], s, d, padding)
+        dy = rs.randint(4, size=(xs[0], ws[0], ci.OH, ci.OW)).astype(np.float32)
+        ry, rdx, rdw = conv2d_all(x, w, dy, s, d, padding)
+        for prefill in (None, 5.0):
+            y, dx, dw = _run_conv(hip, x, w, dy, s, d, padding, prefill=prefill)
+            off = 0.0 if prefill is None else prefill
+            assert np.array_equal(y, ry), ('fwd', xs, ws)
+            assert np.array_equal(dx - off, rdx), ('dX', xs, ws)
+            assert np.array_equal(dw - off, rdw), ('dW', xs, ws)
+
+
 # benchmark geometries at a reduced batch (the oracle materialises im2col in fp64)
 _BENCH = {
     'cfg1': ((8, 3, 64, 64), (32, 3, 3, 3), 1, 1, 'same', 0),
