@@ -119,6 +119,32 @@ __global__ __launch_bounds__(256) void reduce_partials(float* out, const float* 
   }
 }
 
+// The same for ncols % 4 == 0 with 128-bit reads: a block covers 128 consecutive
+// elements, 8 lanes per group of 4 striding over the slices.
+__global__ __launch_bounds__(256) void reduce_partials4(float* out, const float* part, ReduceArgs a) {
+  __shared__ float red[8][128];
+  const int q = threadIdx.x & 31, ls = threadIdx.x >> 5;
+  const int i4 = (blockIdx.x * 32 + q) * 4;
+  f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (i4 < a.n) {
+    const uint32_t m = a.dN.div((uint32_t)i4), col = (uint32_t)i4 - m * (uint32_t)a.ncols;
+    const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
+    const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+    for (int k = ls; k < ns; k += 8) s += *reinterpret_cast<const f32x4*>(&part[(size_t)k * a.n + i4]);
+  }
+  *reinterpret_cast<f32x4*>(&red[ls][4 * q]) = s;
+  __syncthreads();
+  const int e = threadIdx.x, i = blockIdx.x * 128 + e;
+  if (e < 128 && i < a.n) {
+    float t = red[0][e];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) t += red[k][e];
+    const uint32_t m = a.dN.div((uint32_t)i), col = (uint32_t)i - m * (uint32_t)a.ncols;
+    const uint32_t o = a.om.col(col) + m * (uint32_t)a.om.ld;
+    out[o] = a.beta ? out[o] + t : t;
+  }
+}
+
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
 enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5 };
 
@@ -460,8 +486,12 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     }
     r.dN = make_fastdiv((uint32_t)a.Ncols);
     r.om = final_map<PASS>(a);
-    hipLaunchKernelGGL(reduce_partials, dim3((r.n + 31) / 32), dim3(256), 0, ctx->stream, final_out,
-                       static_cast<const float*>(a.Out), r);
+    if (a.Ncols % 4 == 0)   // partial buffers start 256-byte aligned
+      hipLaunchKernelGGL(reduce_partials4, dim3((r.n + 127) / 128), dim3(256), 0, ctx->stream, final_out,
+                         static_cast<const float*>(a.Out), r);
+    else
+      hipLaunchKernelGGL(reduce_partials, dim3((r.n + 31) / 32), dim3(256), 0, ctx->stream, final_out,
+                         static_cast<const float*>(a.Out), r);
     LNN_HIP(hipGetLastError());
   }
   return LNN_OK;
