@@ -251,6 +251,83 @@ def bench_matmul(api, steps, warmup, n=4096, cpu=True):
     return res
 
 
+def bench_conv_transpose(api, steps, warmup, cpu=True):
+    """Decoder layer: conv2DTranspose 256 -> 128, 5x5, stride 2, 'same', 16x16 -> 32x32, batch 16.  The three
+    passes run on the convolution kernels with the roles swapped (forward = dgrad, dI = forward, dK = wgrad)
+    on the kernel with its channel axes swapped; the swaps are part of the timed passes."""
+    N, IC, IH, IW, OC, KS, S = 16, 256, 16, 16, 128, 5, 2
+    ci = conv_info((N, IC, IH, IW), (OC, IC, KS, KS), S, 1, 'same')
+    rs = np.random.RandomState(0)
+    x = rs.uniform(-1, 1, (N, IC, IH, IW)).astype(np.float32)
+    k = rs.normal(0, np.sqrt(2.0 / (IC * KS * KS)), (OC, IC, KS, KS)).astype(np.float32)
+    dy = rs.normal(0, 1, (N, OC, ci.OH_T, ci.OW_T)).astype(np.float32)
+    desc = api.conv_desc(N, OC, ci.OH_T, ci.OW_T, IC, KS, KS, IH, IW, ci.PADL, ci.PADT, S, 1)
+    X, K, dY = Dev(api, x), Dev(api, k), Dev(api, dy)
+    Kt, dKt = Dev(api, shape=(IC, OC, KS, KS)), Dev(api, shape=(IC, OC, KS, KS))
+    Y, dI, dK = Dev(api, shape=dy.shape), Dev(api, shape=x.shape), Dev(api, shape=k.shape)
+    flops = 2.0 * N * IC * IH * IW * OC * KS * KS
+
+    def swap(src, dst, shape, beta):
+        api.transpose(0, shape, (1, 0, 2, 3), src, dst, beta)
+
+    def p_fwd():
+        swap(K.ptr, Kt.ptr, k.shape, 0)
+        api.conv2d_dgrad(0, desc, X.ptr, Kt.ptr, Y.ptr, 0)
+
+    def p_di():
+        swap(K.ptr, Kt.ptr, k.shape, 0)
+        api.conv2d_fwd(0, desc, dY.ptr, Kt.ptr, dI.ptr, 1)
+
+    def p_dk():
+        api.conv2d_wgrad(0, desc, dY.ptr, X.ptr, dKt.ptr, 0)
+        swap(dKt.ptr, dK.ptr, (IC, OC, KS, KS), 1)
+
+    passes = {'fwd': p_fwd, 'dI': p_di, 'dK': p_dk}
+
+    def step():
+        for fn in passes.values():
+            fn()
+
+    for _ in range(warmup):
+        step()
+    api.synchronize(0)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    api.synchronize(0)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    per_pass = {}
+    for name, fn in passes.items():
+        ms = time_events(api, fn, max(steps, 5))
+        per_pass[name] = {'ms': ms, 'tflops': flops / ms / 1e9, 'frac_mfma': flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS}
+    dom = max(per_pass, key=lambda n: per_pass[n]['ms'])
+    dI.zero()
+    dK.zero()
+    step()
+    res = {'metric': 'conv2DTranspose fwd+bwd fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
+           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True,
+           'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+           'config': {'workload': f'cfgT_decoder: conv2DTranspose x[{N}, {IC}, {IH}, {IW}] k[{OC}, {IC}, {KS}, {KS}] '
+                                  f"stride {S} 'same', step = fwd + dI(+=) + dK(+=)"},
+           'roofline': {'bound': 'mfma', 'kernel': dom, 'achieved': per_pass[dom]['tflops'],
+                        'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s', 'frac': per_pass[dom]['frac_mfma'],
+                        'traffic': None},
+           'passes': per_pass}
+    if cpu:
+        from oracle import conv2d_transpose_all
+        t0 = time.perf_counter()
+        ry, rdi, rdk = conv2d_transpose_all(x[:2], k, dy[:2], S, 1, 'same')
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': 3 * flops * 2 / N / dt / 1e12, 'unit': 'TFLOP/s', 'cores': 1, 'kind': 'port',
+                               'sample': 'numpy fp64 oracle (unfold + matmul), 2 of the 16 images, one run'}
+        got_y, got_di = Y.get()[:2], dI.get()[:2]
+        res['parity'] = {'checked_against': 'fp64 oracle on images 0-1 (Y, dI)',
+                         'max_rel_err': max(rel_err(got_y, ry), rel_err(got_di, rdi)), 'tolerance': 1e-4}
+    for t in (X, K, dY, Kt, dKt, Y, dI, dK):
+        t.free()
+    return res
+
+
 def bench_encoder(steps, warmup):
     """cfg5: full training step (forward, backward, SGD) of the 4-layer 5x5
     stride-2 encoder through the litenn-compatible Python API."""
@@ -318,7 +395,7 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='run only a plain device copy of 256 MiB (three launches of the element-wise kernel) and exit: '
                          'the reference reading for the FETCH_SIZE / WRITE_SIZE counters')
-    ap.add_argument('--config', default='cfg3_vgg3x3', choices=list(CONV_CONFIGS) + ['cfg2_matmul', 'cfg5_encoder'],
+    ap.add_argument('--config', default='cfg3_vgg3x3', choices=list(CONV_CONFIGS) + ['cfg2_matmul', 'cfg5_encoder', 'cfgT_decoder'],
                     help='workload of the JSON line (default: the headline configuration)')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -350,6 +427,9 @@ def main():
             r = bench_matmul(api, args.steps, args.warmup, cpu=not args.no_cpu)
             f.write(json.dumps(r) + '\n')
             print(f'[bench] cfg2 matmul: {r["value"]:.1f} TFLOP/s', file=sys.stderr, flush=True)
+            r = bench_conv_transpose(api, args.steps, args.warmup, cpu=not args.no_cpu)
+            f.write(json.dumps(r) + '\n')
+            print(f'[bench] cfgT decoder: {r["value"]:.1f} TFLOP/s', file=sys.stderr, flush=True)
             r = bench_encoder(args.steps, args.warmup)
             f.write(json.dumps(r) + '\n')
             print(f'[bench] cfg5 encoder: {r["value"]:.0f} images/s, {r["ms_per_step"]:.3f} ms/step', file=sys.stderr,
@@ -358,6 +438,8 @@ def main():
         res = bench_matmul(api, args.steps, args.warmup, cpu=not args.no_cpu)
     elif args.config == 'cfg5_encoder':
         res = bench_encoder(args.steps, args.warmup)
+    elif args.config == 'cfgT_decoder':
+        res = bench_conv_transpose(api, args.steps, args.warmup, cpu=not args.no_cpu)
     else:
         res = bench_conv(api, args.config, args.steps, args.warmup, cpu=not args.no_cpu)
     if args.all:

@@ -12,6 +12,7 @@ def accumulate_target(grad_t):
 
 
 from .conv2D import conv2D
+from .conv2DTranspose import conv2DTranspose
 from .element_wise_op import (element_wise_op,
                               add_const_op as add_const,
                               div_const_op as div_const,

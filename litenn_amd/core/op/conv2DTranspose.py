@@ -1,0 +1,70 @@
+import litenn_amd as nn
+import litenn_amd.core as nc
+from ..hip import api, launch
+
+
+def conv2DTranspose(input_t, kernel_t, stride=2, dilation=1, padding='same'):
+    """Transposed 2-D convolution, NCHW (same call contract as conv2DTranspose.py:8-36).
+
+     input_t    (batch, in_ch, height, width)
+     kernel_t   (out_ch, in_ch, k_height, k_width)
+     stride(2), dilation(1)   int
+     padding    'valid' | 'same'
+
+    The three passes are the three passes of the convolution that maps the
+    (large) output back to the (small) input, with the roles swapped
+    (conv2DTranspose.py:33-47): forward is that convolution's data gradient,
+    dI its forward, dK its weight gradient.  They run on the same implicit-GEMM
+    kernels; nothing is unfolded.  Those kernels contract over the leading
+    kernel axis, so the kernel is used with its two channel axes swapped.
+    """
+    op = nc.Cacheton.get(_Conv2DTransposeOp, input_t.shape, kernel_t.shape, int(stride), int(dilation), padding)
+    output_t = nn.Tensor(op.output_shape)
+    output_t._set_op_name('conv2DTranspose')
+    output_t._assign_gradfn(input_t, lambda O_t, dO_t: conv2DTranspose_dI_gradfn(op, input_t, kernel_t, dO_t))
+    output_t._assign_gradfn(kernel_t, lambda O_t, dO_t: conv2DTranspose_dK_gradfn(op, input_t, kernel_t, dO_t))
+    kt = op.swapped_kernel(kernel_t)
+    launch(lambda dev, x, w, y: api.conv2d_dgrad(dev, op.desc, x, w, y, 0), input_t, kt, (output_t, 'w'))
+    return output_t
+
+
+def conv2DTranspose_dI_gradfn(op, input_t, kernel_t, dO_t):
+    """input.grad += conv2D(dO, kernel with channel axes swapped)   (conv2DTranspose.py:38-42)."""
+    grad_t, beta = nc.op.accumulate_target(input_t.get_grad())
+    kt = op.swapped_kernel(kernel_t)
+    launch(lambda dev, x, w, y: api.conv2d_fwd(dev, op.desc, x, w, y, beta), dO_t, kt, grad_t)
+
+
+def conv2DTranspose_dK_gradfn(op, input_t, kernel_t, dO_t):
+    """kernel.grad += wgrad(dO, input) with its channel axes swapped back   (conv2DTranspose.py:44-47)."""
+    dkt = nn.Tensor(op.swapped_kernel_shape)
+    launch(lambda dev, x, dy, dw: api.conv2d_wgrad(dev, op.desc, x, dy, dw, 0), dO_t, input_t, (dkt, 'w'))
+    nc.op.transpose(dkt, (1, 0, 2, 3), output_t=kernel_t.get_grad(), is_add_to_output=True)
+
+
+class _Conv2DTransposeOp:
+    """Shape plan of one transposed-convolution geometry, memoised by Cacheton
+    (conv2DTranspose.py:50-70)."""
+
+    def __init__(self, input_shape, kernel_shape, stride, dilation, padding):
+        if padding not in ['valid', 'same']:
+            raise ValueError('Wrong padding value, only valid or same supported for conv2DTranspose.')
+        if input_shape.rank != 4 or kernel_shape.rank != 4:
+            raise ValueError('conv2DTranspose expects 4-D input (N,C,H,W) and kernel (O,C,KH,KW).')
+        N, IC, IH, IW = input_shape
+        KO, KI, KH, KW = kernel_shape
+        if KI != IC:
+            raise ValueError(f'Kernel input channels {KI} does not match input channels {IC}.')
+        if stride < 1 or dilation < 1:
+            raise ValueError('stride and dilation must be >= 1')
+        ci = nc.info.InfoConv2D(IH, IW, KH, KW, stride, dilation, padding)
+        self.info = ci
+        self.output_shape = nc.TensorShape((N, KO, ci.OH_T, ci.OW_T))
+        self.swapped_kernel_shape = nc.TensorShape((KI, KO, KH, KW))
+        # the convolution from the output image (KO channels) down to the input image (IC channels)
+        self.desc = api.conv_desc(N, KO, ci.OH_T, ci.OW_T, IC, KH, KW, IH, IW, ci.PADL, ci.PADT, stride, dilation)
+
+    def swapped_kernel(self, kernel_t):
+        kt = nn.Tensor(self.swapped_kernel_shape)
+        nc.op.transpose(kernel_t, (1, 0, 2, 3), output_t=kt)
+        return kt

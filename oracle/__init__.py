@@ -18,6 +18,11 @@ Pinning status (what checks each function, independent of its own formula):
                      the reference's numpy checker, adjoint identities,
                      1x1 == einsum, full-kernel 'valid' == matmul
                      (tests/test_oracle_conv.py)
+  conv2DTranspose    scatter-form definition loops (exact on integers), the
+   fwd/dI/dK         adjoint identity against the pinned conv2D oracle,
+                     linearity in the kernel, stride-1 == conv2D with the
+                     kernel flipped and its channel axes swapped
+                     (tests/test_oracle_conv_transpose.py)
   matmul fwd/dA/dB   np.matmul fp64 on integer-valued data (exact) and
                      adjoint identities (tests/test_oracle_matmul.py)
   refpath (C, fp32)  must reproduce the fp64 oracle exactly on integer-valued
@@ -30,4 +35,6 @@ from .conv_info import info_conv2d, ConvInfo                      # noqa: F401
 from .unfold import (unfold_index_map, unfold_T_index_map,        # noqa: F401
                      apply_index_map)
 from .conv import conv2d_fwd, conv2d_dx, conv2d_dw, conv2d_all    # noqa: F401
+from .conv_transpose import (conv2d_transpose_fwd, conv2d_transpose_di,   # noqa: F401
+                             conv2d_transpose_dk, conv2d_transpose_all)
 from .matmul import matmul_fwd, matmul_da, matmul_db              # noqa: F401

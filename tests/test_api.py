@@ -9,7 +9,7 @@ import itertools
 import numpy as np
 import pytest
 
-from oracle import conv2d_all, info_conv2d
+from oracle import conv2d_all, conv2d_transpose_all, info_conv2d
 
 
 def test_conv2d_reference_style(nn_backend):
@@ -36,6 +36,60 @@ def test_conv2d_reference_style(nn_backend):
             assert np.array_equal(kernel_t.get_grad().np() - 1.0, dK)
             n_cases += 1
     assert n_cases > 150
+
+
+def test_conv2d_transpose_reference_style(nn_backend):
+    """conv2DTranspose_test (conv2DTranspose.py:74-126): its whole grid, exact
+    on integer-valued data, gradients accumulated onto a pre-filled 1.0; a
+    dilation-2 column is added."""
+    nn = nn_backend
+    rs = np.random.RandomState(1)
+    n_cases = 0
+    for padding, dilation, stride, ks, n, ic, oc, hw in itertools.product(
+            ['same', 'valid'], [1, 2], [3, 2, 1], [1, 3, 5, 7], [4, 1], [1, 4], [1, 4], [16, 8, 4]):
+        if padding == 'valid' and hw < ks:
+            continue
+        if dilation == 2 and (n, hw) != (1, 8):
+            continue
+        input_n = rs.randint(2 ** 4, size=(n, ic, hw, hw)).astype(np.float32)
+        kernel_n = rs.randint(2 ** 4, size=(oc, ic, ks, ks)).astype(np.float32)
+        input_t = nn.Tensor_from_value(input_n)
+        kernel_t = nn.Tensor_from_value(kernel_n)
+        conved_t = nn.conv2DTranspose(input_t, kernel_t, stride=stride, dilation=dilation, padding=padding)
+        grad_n = rs.randint(2 ** 4, size=tuple(conved_t.shape)).astype(np.float32)
+        y, dI, dK = conv2d_transpose_all(input_n, kernel_n, grad_n, stride, dilation, padding)
+        assert y.shape == conved_t.shape
+        assert np.array_equal(conved_t.np(), y), (padding, dilation, stride, ks, n, ic, oc, hw)
+        input_t.get_grad().fill(1.0)
+        kernel_t.get_grad().fill(1.0)
+        nn.backward({conved_t: grad_n}, grad_for_non_trainables=True)
+        assert np.array_equal(input_t.get_grad().np() - 1.0, dI), (padding, dilation, stride, ks, n, ic, oc, hw)
+        assert np.array_equal(kernel_t.get_grad().np() - 1.0, dK), (padding, dilation, stride, ks, n, ic, oc, hw)
+        n_cases += 1
+    assert n_cases > 250
+
+
+def test_conv2d_transpose_module_and_errors(nn_backend):
+    nn = nn_backend
+    rs = np.random.RandomState(2)
+    w = rs.randint(4, size=(8, 4, 3, 3)).astype(np.float32)
+    b = rs.randint(4, size=(8,)).astype(np.float32)
+    module = nn.Conv2DTranspose(4, 8, 3, kernel_initializer=nn.initializer.NumpyArray(w),
+                                bias_initializer=nn.initializer.NumpyArray(b))
+    x_n = rs.randint(4, size=(2, 4, 8, 8)).astype(np.float32)
+    x = nn.Tensor_from_value(x_n)
+    y = module(x)
+    assert tuple(y.shape) == (2, 8, 16, 16)
+    ref, dI, dK = conv2d_transpose_all(x_n, w, np.ones((2, 8, 16, 16), np.float32), 2, 1, 'same')
+    assert np.array_equal(y.np(), ref + b.reshape(1, -1, 1, 1))
+    y.backward(grad_for_non_trainables=True)
+    assert np.array_equal(x.get_grad().np(), dI)
+    assert np.array_equal(module.kernel.get_grad().np(), dK)
+    assert np.array_equal(module.bias.get_grad().np(), np.full((8,), 2 * 16 * 16, np.float32))
+    with pytest.raises(ValueError):
+        nn.conv2DTranspose(x, module.kernel, padding=1)
+    with pytest.raises(ValueError):
+        nn.conv2DTranspose(x, nn.Tensor((8, 5, 3, 3)))
 
 
 def test_matmul_reference_style(nn_backend):
