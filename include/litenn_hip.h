@@ -99,6 +99,15 @@ typedef struct lnn_conv2d_desc {
 /* Y (+)= conv(X, W)                      conv2D.py:39-42 */
 int lnn_conv2d_fwd_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* W,
                        float* Y, int beta);
+/* Y = act(conv(X, W) + bias[o])          the convolution, the bias add that follows it in every layer
+ * (module/Conv2D.py:59-62: x + bias.reshape(1,-1,1,1), dual_wise_op.py:110-130) and the activation users
+ * put after it (element_wise_op.py:208-222: leaky_relu O = I*(I>=0) + alpha*I*(I<0)) in one pass: the
+ * epilogue adds bias[o] (bias may be NULL) and applies act to the fp32 accumulator before the only store,
+ * which gives bit-identical results to the three separate kernels. */
+#define LNN_ACT_NONE 0
+#define LNN_ACT_LEAKY_RELU 1
+int lnn_conv2d_fwd_bias_act_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* W,
+                                const float* bias, int act, float slope, float* Y);
 /* dX (+)= dgrad(dY, W)                   conv2D.py:46-50 (the reference always accumulates) */
 int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* W,
                          float* dX, int beta);

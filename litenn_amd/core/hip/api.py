@@ -63,6 +63,7 @@ SIGNATURES = {
     'lnn_gemm_f32': [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _ptr, _c_int, _c_i64,
                      _ptr, _c_int, _c_i64, _ptr, _c_int, _c_i64, _c_int],
     'lnn_conv2d_fwd_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
+    'lnn_conv2d_fwd_bias_act_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int, ctypes.c_float, _ptr],
     'lnn_conv2d_dgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_wgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_unfold2d_f32': [_c_int] + [_c_int] * 14 + [_ptr, _ptr, _c_int],
@@ -196,6 +197,14 @@ def conv_desc(N, C, IH, IW, O, KH, KW, OH, OW, PADL, PADT, stride, dilation):
 
 def conv2d_fwd(dev, desc, X, W, Y, beta=0):
     check(lib.lnn_conv2d_fwd_f32(dev, ctypes.byref(desc), X, W, Y, int(beta)))
+
+
+ACT_NONE, ACT_LEAKY_RELU = 0, 1
+
+
+def conv2d_fwd_bias_act(dev, desc, X, W, bias, act, slope, Y):
+    """Y = act(conv(X, W) + bias[o]); bias may be None."""
+    check(lib.lnn_conv2d_fwd_bias_act_f32(dev, ctypes.byref(desc), X, W, bias, int(act), float(slope), Y))
 
 
 def conv2d_dgrad(dev, desc, dY, W, dX, beta=1):

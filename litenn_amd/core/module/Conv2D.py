@@ -36,10 +36,11 @@ class Conv2D(nn.Module):
         super().__init__(saveables=['kernel', 'bias'])
 
     def forward(self, x, **kwargs):
-        x = nn.conv2D(x, self.kernel, self.stride, self.dilation, padding=self.padding)
         if self.use_bias:
-            x = x + self.bias.reshape((1, -1, 1, 1))
-        return x
+            # conv2D followed by x + bias.reshape((1,-1,1,1)) (module/Conv2D.py:59-62), the add done in the
+            # convolution's epilogue: same values, same gradients, one pass over the output instead of two
+            return nc.op.conv2D_bias_act(x, self.kernel, self.bias, self.stride, self.dilation, self.padding)
+        return nn.conv2D(x, self.kernel, self.stride, self.dilation, padding=self.padding)
 
     def __str__(self): return f'{self.__class__.__name__} : in_ch:{self.in_ch} out_ch:{self.out_ch} '
     __repr__ = __str__

@@ -11,7 +11,7 @@ def accumulate_target(grad_t):
     return grad_t, 1
 
 
-from .conv2D import conv2D
+from .conv2D import conv2D, conv2D_bias_act
 from .conv2DTranspose import conv2DTranspose
 from .element_wise_op import (element_wise_op,
                               add_const_op as add_const,

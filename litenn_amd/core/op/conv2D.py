@@ -24,6 +24,67 @@ def conv2D(input_t, kernel_t, stride=1, dilation=1, padding='same'):
     return output_t
 
 
+def conv2D_bias_act(input_t, kernel_t, bias_t=None, stride=1, dilation=1, padding='same', leaky_relu_alpha=None):
+    """leaky_relu(conv2D(input, kernel) + bias.reshape(1,-1,1,1), alpha) in one launch.
+
+    The three steps as a layer writes them (module/Conv2D.py:59-62 followed by
+    element_wise_op.py:216-222) cost two extra read+write passes over the
+    output; here the convolution's epilogue adds bias[o] and applies the
+    activation to the fp32 accumulator before its only store, which gives the
+    same bits.  bias_t (out_ch,) and leaky_relu_alpha are optional;
+    alpha must be > 0 (the backward pass reads the sign of the pre-activation
+    off the output).  Gradients: input and kernel as conv2D, bias the sum of
+    the pre-activation gradient over batch and pixels, each accumulated.
+    """
+    op = nc.Cacheton.get(_Conv2DOp, input_t.shape, kernel_t.shape, int(stride), int(dilation), padding)
+    if bias_t is not None and tuple(bias_t.shape) != (kernel_t.shape[0],):
+        raise ValueError(f'bias shape {tuple(bias_t.shape)} does not match {kernel_t.shape[0]} output channels')
+    if leaky_relu_alpha is not None and not leaky_relu_alpha > 0:
+        raise ValueError('leaky_relu_alpha must be > 0 for the fused form')
+    act = api.ACT_NONE if leaky_relu_alpha is None else api.ACT_LEAKY_RELU
+    alpha = 0.0 if leaky_relu_alpha is None else float(leaky_relu_alpha)
+    output_t = nn.Tensor(op.output_shape)
+    output_t._set_op_name('conv2D_bias_act')
+    pre_grad = _PreActivationGrad(act, alpha)
+    output_t._assign_gradfn(input_t, lambda O_t, dO_t: conv2D_dI_gradfn(op, input_t, kernel_t, pre_grad(O_t, dO_t)))
+    output_t._assign_gradfn(kernel_t, lambda O_t, dO_t: conv2D_dK_gradfn(op, input_t, kernel_t, pre_grad(O_t, dO_t)))
+    if bias_t is None:
+        launch(lambda dev, x, w, y: api.conv2d_fwd_bias_act(dev, op.desc, x, w, None, act, alpha, y),
+               input_t, kernel_t, (output_t, 'w'))
+    else:
+        output_t._assign_gradfn(bias_t, lambda O_t, dO_t: _bias_gradfn(bias_t, pre_grad(O_t, dO_t)))
+        launch(lambda dev, x, w, b, y: api.conv2d_fwd_bias_act(dev, op.desc, x, w, b, act, alpha, y),
+               input_t, kernel_t, bias_t, (output_t, 'w'))
+    return output_t
+
+
+class _PreActivationGrad:
+    """dO * f'(pre-activation), computed once per backward pass and shared by
+    the gradient functions of the fused op.  For leaky ReLU with alpha > 0 the
+    output has the sign of the pre-activation, so f' is read off the output."""
+
+    def __init__(self, act, alpha):
+        self.act, self.alpha = act, alpha
+        self.key, self.value = None, None
+
+    def __call__(self, O_t, dO_t):
+        if self.act == api.ACT_NONE:
+            return dO_t
+        if self.key is not dO_t:
+            pre = nn.Tensor(dO_t.shape)
+            n = dO_t.shape.size
+            launch(lambda dev, o, do, di: api.ew_bwd(dev, api.EW_LEAKY_RELU, n, o, do, di, self.alpha),
+                   O_t, dO_t, pre)   # a fresh tensor is zero-filled on first use; the kernel adds into it
+            self.key, self.value = dO_t, pre
+        return self.value
+
+
+def _bias_gradfn(bias_t, dpre_t):
+    """bias.grad[o] += sum over batch and pixels   (dual_wise_op.py:110-130 for the broadcast operand)."""
+    shape = tuple(dpre_t.shape)
+    launch(lambda dev, s, g: api.reduce_sum(dev, shape, (0, 2, 3), 1.0, s, g, 1), dpre_t, bias_t.get_grad())
+
+
 def conv2D_dI_gradfn(op, input_t, kernel_t, dO_t):
     """input.grad += dgrad(dO, kernel)   (conv2D.py:46-50)."""
     grad_t, beta = nc.op.accumulate_target(input_t.get_grad())

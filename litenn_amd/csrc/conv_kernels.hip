@@ -34,6 +34,7 @@ struct ConvArgs {
   int beta;
   int n_units, total_units;
   int ksplit;        // wgrad: number of K slices (tap-major: of every chunk but the last)
+  PostOp post;       // forward only: bias / activation of the stored result
   size_t ws_used;    // bytes at the front of the scratch buffer that hold this call's permuted weights
   int n_chunks, ks_last;   // tap-major wgrad: chunks of chunk_units units; K slices of the last, possibly shorter one
   FastDiv dC;        // tap-major wgrad: divide a column index by the channel count
@@ -95,6 +96,7 @@ struct ReduceArgs {
   int bm_log, uw_log, per_mt, last_unit0;
   FastDiv dN;
   OutMap om;
+  PostOp post;
 };
 __global__ __launch_bounds__(256) void reduce_partials(float* out, const float* part, ReduceArgs a) {
   __shared__ float red[8][33];
@@ -115,6 +117,7 @@ __global__ __launch_bounds__(256) void reduce_partials(float* out, const float* 
 #pragma unroll
     for (int k = 1; k < 8; ++k) s += red[k][li];
     const uint32_t o = a.om.col(col) + m * (uint32_t)a.om.ld;
+    if (a.post.any()) s = a.post.apply(s, a.post.bias != nullptr ? a.post.bias[m] : 0.0f);
     out[o] = a.beta ? out[o] + s : s;
   }
 }
@@ -141,6 +144,7 @@ __global__ __launch_bounds__(256) void reduce_partials4(float* out, const float*
     for (int k = 1; k < 8; ++k) t += red[k][e];
     const uint32_t m = a.dN.div((uint32_t)i), col = (uint32_t)i - m * (uint32_t)a.ncols;
     const uint32_t o = a.om.col(col) + m * (uint32_t)a.om.ld;
+    if (a.post.any()) t = a.post.apply(t, a.post.bias != nullptr ? a.post.bias[m] : 0.0f);
     out[o] = a.beta ? out[o] + t : t;
   }
 }
@@ -191,6 +195,7 @@ struct ConvProblemBase {
   rsrc_t rx, rw, rc;
   int M, Ncols, K, kbeg, kend, beta;
   OutMap om;
+  PostOp post;
 };
 
 template <bool FLAG, int ST>
@@ -304,6 +309,8 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
   p.rc = make_rsrc(out, a.bytesOut);
   // split-K partials stay in GEMM order (coalesced); the slice reduction applies the final mapping
   p.om = a.ksplit > 1 ? plain_map(a.Ncols) : final_map<PASS>(a);
+  p.post = a.post;
+  if (a.ksplit > 1) { p.post.bias = nullptr; p.post.act = 0; }   // applied by the slice reduction
   if (PASS == PASS_WGRAD_TAP)
     walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.g.KK, a.total_units,
                               a.chunk_units, chunk_i);
@@ -486,6 +493,7 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     }
     r.dN = make_fastdiv((uint32_t)a.Ncols);
     r.om = final_map<PASS>(a);
+    r.post = a.post;
     if (a.Ncols % 4 == 0)   // partial buffers start 256-byte aligned
       hipLaunchKernelGGL(reduce_partials4, dim3((r.n + 127) / 128), dim3(256), 0, ctx->stream, final_out,
                          static_cast<const float*>(a.Out), r);
@@ -506,9 +514,12 @@ static int launch_by_m(DeviceCtx* ctx, ConvArgs& a, bool flag) {
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta) {
+int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta,
+                    const float* bias, int act, float slope) {
   ConvArgs a;
   a.ws_used = 0;
+  a.post = PostOp{bias, act, slope};
+  if (beta && a.post.any()) return set_error(LNN_ERR_INVALID, "conv2d_fwd: bias / activation cannot be combined with accumulation");
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !W || !Y) return set_error(LNN_ERR_INVALID, "conv2d_fwd: null pointer");
@@ -551,6 +562,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
       if (nt == 0 && beta) continue;                        // nothing to add; without beta the class is zero-filled
       ConvArgs a;
       a.ws_used = 0;
+      a.post = PostOp{nullptr, 0, 0.0f};
       a.g = full;
       ConvGeom& g = a.g;
       g.IH = (full.IH - pc.h0 + S - 1) / S;
@@ -585,6 +597,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
 int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
   ConvArgs a;
   a.ws_used = 0;
+  a.post = PostOp{nullptr, 0, 0.0f};
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");

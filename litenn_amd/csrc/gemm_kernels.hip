@@ -47,6 +47,7 @@ struct GemmProblem {
   rsrc_t ra, rb, rc;
   int lda, ldb, M, Ncols, K, kbeg, kend, beta;
   OutMap om;
+  PostOp post;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(ra, lda, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rb, ldb, col0, Ncols, K); }
 };
@@ -62,6 +63,7 @@ __global__ __launch_bounds__(512, 2) void gemm_kernel(GemmArgs a) {
   p.rc = make_rsrc(a.C + b * a.sC, a.bytesC);
   p.lda = a.lda; p.ldb = a.ldb; p.M = a.M; p.Ncols = a.N; p.K = a.K;
   p.kbeg = 0; p.kend = a.K; p.beta = a.beta;
+  p.post.bias = nullptr; p.post.act = 0; p.post.slope = 0.0f;
   p.om.nchw = 0; p.om.ld = a.ldc; p.om.mtot = 0; p.om.dHW = FastDiv{0, 0, 1};
   walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
 }

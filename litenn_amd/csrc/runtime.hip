@@ -276,7 +276,14 @@ int lnn_gemm_f32(int dev, int trans_a, int trans_b, int batch, int M, int N, int
 
 int lnn_conv2d_fwd_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta) {
   CTX(dev);
-  return launch_conv_fwd(ctx, d, X, W, Y, beta);
+  return launch_conv_fwd(ctx, d, X, W, Y, beta, nullptr, 0, 0.0f);
+}
+
+int lnn_conv2d_fwd_bias_act_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* W, const float* bias,
+                                int act, float slope, float* Y) {
+  CTX(dev);
+  if (act != LNN_ACT_NONE && act != LNN_ACT_LEAKY_RELU) return set_error(LNN_ERR_INVALID, "conv2d_fwd_bias_act: unknown activation");
+  return launch_conv_fwd(ctx, d, X, W, Y, 0, bias, act, slope);
 }
 
 int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta) {

@@ -1020,6 +1020,20 @@ struct ConvWgradTapBDirect {
   }
 };
 
+// Optional per-row bias and activation applied to a finished element before
+// it is stored ('=' only): y = f(acc + bias[m]), f = identity or leaky ReLU
+// (x >= 0 ? x : slope * x, the same selection the pointwise kernel makes).
+struct PostOp {
+  const float* bias;   // one value per output row m, or null
+  int act;             // 0 none, 1 leaky ReLU
+  float slope;
+  __host__ __device__ bool any() const { return bias != nullptr || act != 0; }
+  __device__ __forceinline__ float apply(float v, float b) const {
+    v += b;
+    return (act == 0 || v >= 0.0f) ? v : slope * v;
+  }
+};
+
 // ---------------------------------------------------------------------------
 // Output mapping.  plain: off = m*ld + n.  NCHW image tensor with the GEMM
 // column n = (img, pixel): off = (img*Mtot + m)*HW + pixel.
@@ -1124,7 +1138,7 @@ struct LdsSize { static constexpr int value = KC ? R * LDK : BK * R; };
 //     template <int R> using LA = ...;   template <int R> using LB = ...;
 //     template <int R> void init_a(LA<R>&, int row0) const;
 //     template <int R, class A> void init_b(LB<R>&, int col0, A& la) const;   (la: this group's A loader)
-//     int kbeg, kend, M, Ncols, beta;  rsrc_t rc;  OutMap om;
+//     int kbeg, kend, M, Ncols, beta;  rsrc_t rc;  OutMap om;  PostOp post;
 //   };
 
 // A B-side loader that shares per-step state with its group's A loader
@@ -1318,6 +1332,19 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
 #pragma unroll
         for (int r = 0; r < 16; ++r) buf_store(p.rc, elem(cb, roff[r]), acc[j][r] + old[j & 1][r]);
         cb = cbn;
+      }
+    } else if (p.post.any()) {
+      float bv[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+        bv[r] = (p.post.bias != nullptr && m < p.M) ? p.post.bias[m] : 0.0f;
+      }
+#pragma unroll
+      for (int j = 0; j < NTC; ++j) {
+        const uint32_t cb = col_off(j);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) buf_store(p.rc, elem(cb, roff[r]), p.post.apply(acc[j][r], bv[r]));
       }
     } else {
 #pragma unroll

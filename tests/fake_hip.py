@@ -11,7 +11,7 @@ from oracle import (conv2d_fwd, conv2d_dx, conv2d_dw, unfold_index_map, unfold_T
 from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
-         'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_dgrad', 'conv2d_wgrad',
+         'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad',
          'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update']
 
 
@@ -95,6 +95,16 @@ class FakeHip:
         r = conv2d_fwd(self.f(X, xs), self.f(W, ws), d.stride, d.dilation, pad)
         assert r.shape == ys, (r.shape, ys)
         self._put(self.f(Y, ys), r, beta)
+
+    def conv2d_fwd_bias_act(self, dev, d, X, W, bias, act, slope, Y):
+        self.launches += 1
+        xs, ws, ys, pad = self._geom(d)
+        r = conv2d_fwd(self.f(X, xs), self.f(W, ws), d.stride, d.dilation, pad).astype(np.float32)
+        if bias is not None:
+            r = r + self.f(bias, (d.O,)).reshape(1, -1, 1, 1)
+        if act == 1:
+            r = np.where(r >= 0, r, np.float32(slope) * r)
+        self._put(self.f(Y, ys), r, 0)
 
     def conv2d_dgrad(self, dev, d, dY, W, dX, beta=1):
         self.launches += 1

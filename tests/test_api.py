@@ -92,6 +92,39 @@ def test_conv2d_transpose_module_and_errors(nn_backend):
         nn.conv2DTranspose(x, nn.Tensor((8, 5, 3, 3)))
 
 
+def test_conv2d_bias_act_equals_separate_ops(nn_backend):
+    """The fused layer step leaky_relu(conv2D(x, k) + bias, alpha) must give the
+    bits and the gradients of the three separate operators, on integer-valued
+    data (alpha = 0.5 keeps every value exactly representable)."""
+    nn = nn_backend
+    import litenn_amd.core as nc
+    rs = np.random.RandomState(4)
+    for (n, ic, oc, hw, ks, stride, padding, alpha) in [(2, 3, 5, 9, 3, 1, 'same', 0.5), (1, 32, 40, 6, 3, 2, 1, 0.5),
+                                                        (3, 4, 2, 8, 1, 1, 'valid', None), (1, 130, 70, 5, 3, 1, 'same', 0.25),
+                                                        (2, 256, 96, 4, 3, 1, 'same', 0.5)]:
+        x_n = rs.randint(-3, 4, size=(n, ic, hw, hw)).astype(np.float32)
+        k_n = rs.randint(-3, 4, size=(oc, ic, ks, ks)).astype(np.float32)
+        b_n = rs.randint(-9, 10, size=(oc,)).astype(np.float32)
+        outs = []
+        for fused in (False, True):
+            x, k, b = nn.Tensor_from_value(x_n), nn.Tensor_from_value(k_n), nn.Tensor_from_value(b_n)
+            if fused:
+                y = nc.op.conv2D_bias_act(x, k, b, stride, 1, padding, leaky_relu_alpha=alpha)
+            else:
+                y = nn.conv2D(x, k, stride=stride, padding=padding) + b.reshape((1, -1, 1, 1))
+                if alpha is not None:
+                    y = nn.leaky_relu(y, alpha)
+            g_n = np.random.RandomState(5).randint(-4, 5, size=tuple(y.shape)).astype(np.float32)
+            nn.backward({y: g_n}, grad_for_non_trainables=True)
+            outs.append((y.np(), x.get_grad().np(), k.get_grad().np(), b.get_grad().np()))
+        for a, f in zip(*outs):
+            assert np.array_equal(a, f), (n, ic, oc, hw, ks, stride, padding, alpha)
+    with pytest.raises(ValueError):
+        nc.op.conv2D_bias_act(nn.Tensor((1, 2, 4, 4)), nn.Tensor((3, 2, 3, 3)), nn.Tensor((4,)))
+    with pytest.raises(ValueError):
+        nc.op.conv2D_bias_act(nn.Tensor((1, 2, 4, 4)), nn.Tensor((3, 2, 3, 3)), leaky_relu_alpha=0.0)
+
+
 def test_matmul_reference_style(nn_backend):
     nn = nn_backend
     rs = np.random.RandomState(1)

@@ -299,6 +299,42 @@ def test_conv_few_tiles_split_k_integer_exact(hip):
             assert np.array_equal(dw - off, rdw), ('dW', xs, ws)
 
 
+def test_conv_fwd_bias_act_matches_separate_kernels(hip):
+    """Fused forward through the C ABI against the three separate launches
+    (convolution, broadcast bias add, leaky ReLU) of the same library, bit for
+    bit on random float data, on the direct, table-driven and split-K paths;
+    bias only, activation only, both."""
+    rs = np.random.RandomState(41)
+    cases = [((2, 128, 12, 12), (128, 128, 3, 3), 1, 1, 'same'), ((2, 3, 17, 9), (5, 3, 3, 3), 2, 1, 1),
+             ((1, 256, 6, 6), (96, 256, 3, 3), 1, 1, 'same'), ((2, 64, 9, 11), (40, 64, 1, 1), 1, 1, 'valid')]
+    for xs, ws, s, d, padding in cases:
+        say(f'conv fused x={xs} w={ws} s={s} pad={padding}')
+        desc, ci = _desc(hip, xs, ws, s, d, padding)
+        x = rs.normal(0, 1, xs).astype(np.float32)
+        w = rs.normal(0, 1, ws).astype(np.float32)
+        b = rs.normal(0, 3, (ws[0],)).astype(np.float32)
+        ys = (xs[0], ws[0], ci.OH, ci.OW)
+        X, W, B = DevArr(hip, x), DevArr(hip, w), DevArr(hip, b)
+        Y0, Y1, Y2 = (DevArr(hip, shape=ys, fill=np.nan) for _ in range(3))
+        hip.conv2d_fwd(0, desc, X.ptr, W.ptr, Y0.ptr, 0)
+        n = int(np.prod(ys))
+        for use_b, act in ((True, hip.ACT_LEAKY_RELU), (True, hip.ACT_NONE), (False, hip.ACT_LEAKY_RELU)):
+            ref = Y0.get()
+            if use_b:
+                ref = ref + b.reshape(1, -1, 1, 1)
+            if act == hip.ACT_LEAKY_RELU:
+                ref = np.where(ref >= 0, ref, np.float32(0.1) * ref)
+            hip.conv2d_fwd_bias_act(0, desc, X.ptr, W.ptr, B.ptr if use_b else None, act, 0.1, Y1.ptr)
+            assert np.array_equal(Y1.get(), ref.astype(np.float32)), (xs, ws, use_b, act)
+        # and against the library's own separate kernels
+        hip.binary_bcast(0, hip.BIN_ADD, ys, ys, (1, ws[0], 1, 1), Y0.ptr, B.ptr, Y2.ptr, 0)
+        hip.ew_fwd(0, hip.EW_LEAKY_RELU, n, Y2.ptr, Y2.ptr, 0.1, 0)
+        hip.conv2d_fwd_bias_act(0, desc, X.ptr, W.ptr, B.ptr, hip.ACT_LEAKY_RELU, 0.1, Y1.ptr)
+        assert np.array_equal(Y1.get(), Y2.get()), (xs, ws)
+    with pytest.raises(hip.HipException):
+        hip.conv2d_fwd_bias_act(0, desc, X.ptr, W.ptr, B.ptr, 7, 0.1, Y1.ptr)
+
+
 # benchmark geometries at a reduced batch (the oracle materialises im2col in fp64)
 _BENCH = {
     'cfg1': ((8, 3, 64, 64), (32, 3, 3, 3), 1, 1, 'same', 0),
