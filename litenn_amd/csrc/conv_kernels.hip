@@ -5,6 +5,8 @@
 //   forward  Y [O  x P ] = W[O x CKK]        . im2col(X)[CKK x P]     P = N*OH*OW
 //   dgrad    dX[C  x Q ] = Wt[C x O*KK]      . im2rowT(dY)[O*KK x Q]  Q = N*IH*IW
 //   wgrad    dW[O  x CKK] = dY[O x P]        . im2row(X)[P x CKK]     (split over P)
+#include <vector>
+
 #include "common.hpp"
 
 #ifndef LNN_STAGES_WGRAD
@@ -33,6 +35,7 @@ struct ConvArgs {
   int M, Ncols, K;   // GEMM extents
   int beta;
   int n_units, total_units;
+  int grid_x;        // workgroups along x that belong to this problem (a batched launch may have more)
   int ksplit;        // wgrad: number of K slices (tap-major: of every chunk but the last)
   PostOp post;       // forward only: bias / activation of the stored result
   size_t ws_used;    // bytes at the front of the scratch buffer that hold this call's permuted weights
@@ -271,9 +274,10 @@ __host__ __device__ inline OutMap final_map(const ConvArgs& a) {
 }
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
-__global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
+__device__ __forceinline__ void conv_body(const ConvArgs& a) {
   using Cfg = ConvCfg<PASS, WM, NTMAX, FLAG>;
   __shared__ __attribute__((aligned(16))) float lds[Cfg::STAGES * (Cfg::SA + Cfg::SB)];
+  if ((int)blockIdx.x >= a.grid_x || (int)blockIdx.y >= (a.ksplit > 1 ? a.ksplit : 1)) return;   // batched launch: not ours
   ConvProblem<PASS, FLAG, Cfg::STAGES> p;
   p.g = a.g;
   p.tab = a.tab;
@@ -315,7 +319,24 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
     walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.g.KK, a.total_units,
                               a.chunk_units, chunk_i);
   else
-    walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
+    walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units,
+                          (int)blockIdx.x, a.grid_x);
+}
+
+template <int PASS, int WM, int NTMAX, bool FLAG>
+__global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
+  conv_body<PASS, WM, NTMAX, FLAG>(a);
+}
+
+// Several independent problems of one pass in one launch (the pixel classes of a strided dgrad):
+// blockIdx.z selects the problem, each uses the leading part of the x / y grid it asked for.
+constexpr int kMaxBatch = 4;
+struct ConvArgsBatch {
+  ConvArgs c[kMaxBatch];
+};
+template <int PASS, int WM, int NTMAX>
+__global__ __launch_bounds__(512, 2) void conv_kernel_batch(ConvArgsBatch b) {
+  conv_body<PASS, WM, NTMAX, true>(b.c[blockIdx.z]);
 }
 
 // ---------------------------------------------------------------------------
@@ -345,6 +366,16 @@ static int fill_geom(const lnn_conv2d_desc* d, ConvGeom& g) {
   return LNN_OK;
 }
 
+// Bound the table cache: before a call that may add up to n tables, drop everything once the work queued so
+// far is done.  Never in the middle of a call: its earlier tables must stay valid until it has launched.
+static int reserve_tables(DeviceCtx* ctx, size_t n) {
+  if (ctx->tables.size() + n <= 256) return LNN_OK;
+  LNN_HIP(hipStreamSynchronize(ctx->stream));
+  for (auto& kv : ctx->tables) (void)hipFree(kv.second);
+  ctx->tables.clear();
+  return LNN_OK;
+}
+
 // mode 0: forward / wgrad table; 1, 2: dgrad tables of pixel class pc (per k / per tap)
 static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const PixelClass& pc, const KEntry** out) {
   const int nt = pc.nkh * pc.nkw;
@@ -357,11 +388,6 @@ static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const PixelCla
   if (it != ctx->tables.end()) {
     *out = it->second;
     return LNN_OK;
-  }
-  if (ctx->tables.size() >= 256) {   // bound the cache: drop everything once work queued so far is done
-    LNN_HIP(hipStreamSynchronize(ctx->stream));
-    for (auto& kv : ctx->tables) (void)hipFree(kv.second);
-    ctx->tables.clear();
   }
   KEntry* tab = nullptr;
   hipError_t e = hipMalloc((void**)&tab, (size_t)Kpad * sizeof(KEntry));
@@ -396,40 +422,98 @@ static int permuted_weights(DeviceCtx* ctx, const ConvGeom& g, const float* W, i
   return LNN_OK;
 }
 
-template <int PASS, int WM, int NTMAX>
-static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
+// Slice reduction of a split-K problem into its final tensor.
+template <int PASS, int WM>
+static int launch_reduce(DeviceCtx* ctx, const ConvArgs& a, float* final_out, int final_beta) {
+  constexpr int WN = 4 / WM;
+  ReduceArgs r;
+  r.n = a.M * a.Ncols; r.slices = a.ksplit; r.slices_last = a.ksplit; r.beta = final_beta; r.ncols = a.Ncols;
+  r.bm_log = WM == 4 ? 7 : (WM == 2 ? 6 : 5); r.uw_log = WN == 4 ? 7 : (WN == 2 ? 6 : 5);
+  r.per_mt = 0; r.last_unit0 = 0x7fffffff;
+  if (PASS == PASS_WGRAD_TAP) {
+    r.slices_last = a.ks_last;
+    r.per_mt = a.g.KK * a.n_units;
+    r.last_unit0 = (a.n_chunks - 1) * a.chunk_units;
+  }
+  r.dN = make_fastdiv((uint32_t)a.Ncols);
+  r.om = final_map<PASS>(a);
+  r.post = a.post;
+  if (a.Ncols % 4 == 0)   // partial buffers start 256-byte aligned
+    hipLaunchKernelGGL(reduce_partials4, dim3((r.n + 127) / 128), dim3(256), 0, ctx->stream, final_out,
+                       static_cast<const float*>(a.Out), r);
+  else
+    hipLaunchKernelGGL(reduce_partials, dim3((r.n + 31) / 32), dim3(256), 0, ctx->stream, final_out,
+                       static_cast<const float*>(a.Out), r);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+// Forward / dgrad: units, grid and K split of one problem that may use `slots` workgroups.
+// Returns the bytes of partial sums it needs (0 without a K split).
+template <int WM, int NTMAX>
+static size_t plan_tiles(ConvArgs& a, long long slots) {
   constexpr int WN = 4 / WM, BM = 32 * WM;
   const int m_tiles = (a.M + BM - 1) / BM;
   a.n_units = (a.Ncols + 32 * WN - 1) / (32 * WN);
-  long long total = (long long)m_tiles * a.n_units;
+  const long long total = (long long)m_tiles * a.n_units;
+  a.total_units = total > 0x7fffffffll ? -1 : (int)total;
   a.chunk_units = 0;
-  if (PASS == PASS_WGRAD_TAP) {
-    // columns are tap-major: KK segments of C / (32*WN) units per M tile; a workgroup
-    // takes one sub-tile's worth of whole segments (or of one segment's halves)
-    a.n_units = a.g.C / (32 * WN);
-    const int per_group = a.n_units < NTMAX ? a.n_units : NTMAX;
-    a.chunk_units = 2 * per_group;
-    total = (long long)m_tiles * a.g.KK * a.n_units;
-    a.dC = make_fastdiv((uint32_t)a.g.C);
-  }
-  if (total > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
-  a.total_units = (int)total;
-  const long long slots = ctx->cus;   // one 512-thread workgroup per compute unit
-  int grid, ksplit = 1, grid_y = 1;
-  float* final_out = a.Out;
-  const int final_beta = a.beta;
   a.n_chunks = 1;
   a.ks_last = 1;
+  a.ksplit = 1;
+  a.grid_x = (int)(total < slots ? total : slots);
+  // Few output tiles (small images, deep layers): a workgroup's share would be a sliver of a sub-tile and
+  // most of its time data movement.  Cut the output into full sub-tiles instead and split K over the
+  // workgroups that are left, as wgrad does.
+  const int chunk = 2 * NTMAX;
+  const long long chunks = (total + chunk - 1) / chunk;
+  const int nkt = (a.K + BK - 1) / BK;
+  if (total < slots * (chunk / 2 + 1) && chunks * 2 <= slots && nkt >= 16) {
+    long long s = slots / chunks;
+    if (s > nkt / 8) s = nkt / 8;
+    if (s > 1) {
+      a.ksplit = (int)s;
+      a.grid_x = (int)chunks;
+      return (size_t)a.ksplit * a.M * a.Ncols * sizeof(float);
+    }
+  }
+  return 0;
+}
+
+template <int PASS, int WM, int NTMAX>
+static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
+  constexpr int WN = 4 / WM, BM = 32 * WM;
+  const long long slots = ctx->cus;   // one 512-thread workgroup per compute unit
+  float* final_out = a.Out;
+  const int final_beta = a.beta;
+  int grid_y = 1;
   if (PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP) {
+    const int m_tiles = (a.M + BM - 1) / BM;
+    a.n_units = (a.Ncols + 32 * WN - 1) / (32 * WN);
+    long long total = (long long)m_tiles * a.n_units;
+    a.chunk_units = 0;
+    if (PASS == PASS_WGRAD_TAP) {
+      // columns are tap-major: KK segments of C / (32*WN) units per M tile; a workgroup
+      // takes one sub-tile's worth of whole segments (or of one segment's halves)
+      a.n_units = a.g.C / (32 * WN);
+      const int per_group = a.n_units < NTMAX ? a.n_units : NTMAX;
+      a.chunk_units = 2 * per_group;
+      total = (long long)m_tiles * a.g.KK * a.n_units;
+      a.dC = make_fastdiv((uint32_t)a.g.C);
+    }
+    if (total > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
+    a.total_units = (int)total;
+    a.n_chunks = 1;
+    a.ks_last = 1;
     // one full-width sub-tile per workgroup, then as many K slices as fill the chip
     const int chunk = PASS == PASS_WGRAD_TAP ? a.chunk_units : 2 * NTMAX;
-    grid = (int)((total + chunk - 1) / chunk);
+    int grid = (int)((total + chunk - 1) / chunk);
     const int nkt = (a.K + BK - 1) / BK;
     long long s = PASS == PASS_WGRAD_TAP ? slots * chunk / total : slots / grid;
     if (s > nkt / 4) s = nkt / 4;
     if (s > 1024) s = 1024;
     if (s < 1) s = 1;
-    ksplit = (int)s;
+    int ksplit = (int)s;
     grid_y = ksplit;
     if (PASS == PASS_WGRAD_TAP) {
       // the last chunk holds rem <= chunk units: give it that share of the slices
@@ -441,6 +525,8 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
       if (ksplit > 1) grid = (grid - 1) * ksplit + a.ks_last;
       grid_y = 1;
     }
+    a.ksplit = ksplit;
+    a.grid_x = grid;
     if (ksplit > 1) {
       const size_t need = (size_t)ksplit * a.M * a.Ncols * sizeof(float);
       int st = ensure_workspace(ctx, need);
@@ -449,31 +535,18 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
       a.beta = 0;
     }
   } else {
-    grid = (int)(total < slots ? total : slots);
-    // Few output tiles (small images, deep layers): a workgroup's share would be a sliver of a sub-tile and
-    // most of its time data movement.  Cut the output into full sub-tiles instead and split K over the
-    // workgroups that are left, as wgrad does.
-    const int chunk = 2 * NTMAX;
-    const long long chunks = (total + chunk - 1) / chunk;
-    const int nkt = (a.K + BK - 1) / BK;
-    if (total < slots * (chunk / 2 + 1) && chunks * 2 <= slots && nkt >= 16) {
-      long long s = slots / chunks;
-      if (s > nkt / 8) s = nkt / 8;
-      if (s > 1) {
-        ksplit = (int)s;
-        grid = (int)chunks;
-        grid_y = ksplit;
-        const size_t need = (size_t)ksplit * a.M * a.Ncols * sizeof(float);
-        // the scratch buffer may already hold this call's permuted weights: keep them in front
-        int st = ensure_workspace(ctx, a.ws_used + need);
-        if (st != LNN_OK) return st;
-        a.Out = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + a.ws_used);
-        a.beta = 0;
-      }
+    const size_t need = plan_tiles<WM, NTMAX>(a, slots);
+    if (a.total_units < 0) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
+    if (need) {
+      // the scratch buffer may already hold this call's permuted weights: keep them in front
+      int st = ensure_workspace(ctx, a.ws_used + need);
+      if (st != LNN_OK) return st;
+      a.Out = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + a.ws_used);
+      a.beta = 0;
+      grid_y = a.ksplit;
     }
   }
-  a.ksplit = ksplit;
-  dim3 g(grid, grid_y, 1), b(512, 1, 1);
+  dim3 g(a.grid_x, grid_y, 1), b(512, 1, 1);
   constexpr bool kUsesFlag = PASS == PASS_FWD || PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP;   // the other passes have one variant
   if (flag || !kUsesFlag) {
     hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, true>), g, b, 0, ctx->stream, a);
@@ -481,28 +554,63 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, false>), g, b, 0, ctx->stream, a);
   }
   LNN_HIP(hipGetLastError());
-  if (ksplit > 1) {
-    ReduceArgs r;
-    r.n = a.M * a.Ncols; r.slices = ksplit; r.slices_last = ksplit; r.beta = final_beta; r.ncols = a.Ncols;
-    r.bm_log = WM == 4 ? 7 : (WM == 2 ? 6 : 5); r.uw_log = WN == 4 ? 7 : (WN == 2 ? 6 : 5);
-    r.per_mt = 0; r.last_unit0 = 0x7fffffff;
-    if (PASS == PASS_WGRAD_TAP) {
-      r.slices_last = a.ks_last;
-      r.per_mt = a.g.KK * a.n_units;
-      r.last_unit0 = (a.n_chunks - 1) * a.chunk_units;
+  if (a.ksplit > 1) return launch_reduce<PASS, WM>(ctx, a, final_out, final_beta);
+  return LNN_OK;
+}
+
+// The pixel classes of one strided dgrad (all the same M, hence the same tile shape): planned for an equal
+// share of the chip each, launched kMaxBatch at a time, partial sums behind `ws_off` in the scratch buffer
+// (which the caller has sized), then reduced one by one.
+template <int PASS, int WM, int NTMAX>
+static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_off) {
+  const int n = (int)cls.size();
+  const int per_batch = n < kMaxBatch ? n : kMaxBatch;
+  const long long slots = ctx->cus / per_batch > 0 ? ctx->cus / per_batch : 1;   // equal shares of the chip
+  std::vector<float*> final_out(n);
+  std::vector<int> final_beta(n);
+  for (int i = 0; i < n; ++i) {
+    ConvArgs& a = cls[i];
+    const size_t need = plan_tiles<WM, NTMAX>(a, slots);
+    if (a.total_units < 0) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
+    final_out[i] = a.Out;
+    final_beta[i] = a.beta;
+    if (need) {
+      a.Out = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + ws_off);
+      a.beta = 0;
+      ws_off += (need + 255) & ~(size_t)255;
     }
-    r.dN = make_fastdiv((uint32_t)a.Ncols);
-    r.om = final_map<PASS>(a);
-    r.post = a.post;
-    if (a.Ncols % 4 == 0)   // partial buffers start 256-byte aligned
-      hipLaunchKernelGGL(reduce_partials4, dim3((r.n + 127) / 128), dim3(256), 0, ctx->stream, final_out,
-                         static_cast<const float*>(a.Out), r);
-    else
-      hipLaunchKernelGGL(reduce_partials, dim3((r.n + 31) / 32), dim3(256), 0, ctx->stream, final_out,
-                         static_cast<const float*>(a.Out), r);
+  }
+  if (ws_off > ctx->ws_bytes) return set_error(LNN_ERR_HIP, "conv2d_dgrad: scratch buffer smaller than planned");
+  for (int i0 = 0; i0 < n; i0 += kMaxBatch) {
+    const int nb = n - i0 < kMaxBatch ? n - i0 : kMaxBatch;
+    ConvArgsBatch b;
+    int gx = 1, gy = 1;
+    for (int i = 0; i < nb; ++i) {
+      b.c[i] = cls[i0 + i];
+      if (b.c[i].grid_x > gx) gx = b.c[i].grid_x;
+      if (b.c[i].ksplit > gy) gy = b.c[i].ksplit;
+    }
+    for (int i = nb; i < kMaxBatch; ++i) {
+      b.c[i] = cls[i0];
+      b.c[i].grid_x = 0;
+    }
+    hipLaunchKernelGGL((conv_kernel_batch<PASS, WM, NTMAX>), dim3(gx, gy, nb), dim3(512, 1, 1), 0, ctx->stream, b);
     LNN_HIP(hipGetLastError());
   }
+  for (int i = 0; i < n; ++i)
+    if (cls[i].ksplit > 1) {
+      int st = launch_reduce<PASS, WM>(ctx, cls[i], final_out[i], final_beta[i]);
+      if (st != LNN_OK) return st;
+    }
   return LNN_OK;
+}
+
+template <int PASS>
+static int launch_classes_by_m(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_off) {
+  const int M = cls[0].M;
+  if (M > 64) return launch_classes<PASS, 4, 4>(ctx, cls, ws_off);
+  if (M > 32) return launch_classes<PASS, 2, 2>(ctx, cls, ws_off);
+  return launch_classes<PASS, 1, 1>(ctx, cls, ws_off);
 }
 
 template <int PASS>
@@ -523,6 +631,8 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !W || !Y) return set_error(LNN_ERR_INVALID, "conv2d_fwd: null pointer");
+  st = reserve_tables(ctx, 1);
+  if (st != LNN_OK) return st;
   a.tab = nullptr;
   const ConvGeom& g = a.g;
   a.X = X; a.W = W; a.Out = Y;
@@ -547,7 +657,14 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   if (st != LNN_OK) return st;
   if (!dY || !W || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
   const int S = full.S;
+  if (S > 15) return set_error(LNN_ERR_UNSUPPORTED, "conv2d_dgrad: stride > 15");
+  st = reserve_tables(ctx, (size_t)S * S);
+  if (st != LNN_OK) return st;
+  const bool tap = full.O % BK == 0;
   // one stride-1 problem per class of input pixels (see ConvDgradB)
+  std::vector<ConvArgs> cls;
+  std::vector<PixelClass> pcs;
+  size_t w_bytes = 0;   // permuted weights of all classes, back to back
   for (int rh = 0; rh < S; ++rh)
     for (int rw = 0; rw < S; ++rw) {
       PixelClass pc;
@@ -573,25 +690,60 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
       a.tab = nullptr;
       a.X = dY; a.W = W; a.Out = dX;
       a.bytesX = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
-      a.bytesW = (uint32_t)((uint64_t)g.O * g.C * g.KK * 4);
+      a.bytesW = (uint32_t)((uint64_t)g.O * g.C * (tap ? nt : g.KK) * 4);
       a.bytesOut = (uint32_t)((uint64_t)g.N * g.C * full.IHW * 4);
       a.M = g.C; a.Ncols = g.N * g.IHW; a.K = g.O * nt;
       a.beta = beta ? 1 : 0;
-      if (g.O % BK == 0) {
-        st = permuted_weights(ctx, full, W, 1, pc, &a.W, &a.ws_used);
-        if (st != LNN_OK) return st;
-        a.bytesW = (uint32_t)((uint64_t)g.O * g.C * nt * 4);
-        st = get_table(ctx, full, 2, pc, &a.tab);
+      a.dC = make_fastdiv(1);
+      st = get_table(ctx, full, tap ? 2 : 1, pc, &a.tab);
+      if (st != LNN_OK) return st;
+      if (tap) {
+        a.ws_used = w_bytes;   // here: offset of this class's permuted weights in the scratch buffer
+        w_bytes += ((size_t)(a.bytesW ? a.bytesW : 4) + 255) & ~(size_t)255;
+      }
+      cls.push_back(a);
+      pcs.push_back(pc);
+    }
+  if (cls.empty()) return LNN_OK;
+  // scratch: permuted weights of every class, then room for the split-K partial sums of one batch of
+  // classes (at most one full 32768-element sub-tile per workgroup slot)
+  const int nc = (int)cls.size();
+  const size_t part_bytes = (size_t)ctx->cus * 32768 * sizeof(float) + 256 * (size_t)nc;
+  // A class that fills the chip on its own (several units of output per workgroup) gains nothing from
+  // sharing it; neither do more classes than one launch holds (stride > 2).
+  const int unit_cols = cls[0].M > 64 ? 32 : (cls[0].M > 32 ? 64 : 128);
+  const long long units0 = (long long)((cls[0].M + 127) / 128) * ((cls[0].Ncols + unit_cols - 1) / unit_cols);
+  if (nc > kMaxBatch || units0 >= 4ll * ctx->cus) {
+    // one after the other, each with the whole chip
+    for (int i = 0; i < nc; ++i) {
+      ConvArgs& a = cls[i];
+      if (tap) {
+        st = permuted_weights(ctx, full, W, 1, pcs[i], &a.W, &a.ws_used);
         if (st != LNN_OK) return st;
         st = launch_by_m<PASS_DGRAD_TAP>(ctx, a, true);
       } else {
-        st = get_table(ctx, full, 1, pc, &a.tab);
-        if (st != LNN_OK) return st;
+        a.ws_used = 0;
         st = launch_by_m<PASS_DGRAD>(ctx, a, true);
       }
       if (st != LNN_OK) return st;
     }
-  return LNN_OK;
+    return LNN_OK;
+  }
+  st = ensure_workspace(ctx, w_bytes + part_bytes);
+  if (st != LNN_OK) return st;
+  if (tap)
+    for (int i = 0; i < nc; ++i) {
+      ConvArgs& a = cls[i];
+      float* wp = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + a.ws_used);
+      const int n = full.O * full.C * pcs[i].nkh * pcs[i].nkw;
+      if (n > 0) {
+        hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, wp, W, full.O, full.C,
+                           full.KK, 1, full, pcs[i]);
+        LNN_HIP(hipGetLastError());
+      }
+      a.W = wp;
+    }
+  return tap ? launch_classes_by_m<PASS_DGRAD_TAP>(ctx, cls, w_bytes) : launch_classes_by_m<PASS_DGRAD>(ctx, cls, w_bytes);
 }
 
 int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
@@ -601,6 +753,8 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");
+  st = reserve_tables(ctx, 1);
+  if (st != LNN_OK) return st;
   st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);
   if (st != LNN_OK) return st;
   const ConvGeom& g = a.g;

@@ -65,7 +65,7 @@ __global__ __launch_bounds__(512, 2) void gemm_kernel(GemmArgs a) {
   p.kbeg = 0; p.kend = a.K; p.beta = a.beta;
   p.post.bias = nullptr; p.post.act = 0; p.post.slope = 0.0f;
   p.om.nchw = 0; p.om.ld = a.ldc; p.om.mtot = 0; p.om.dHW = FastDiv{0, 0, 1};
-  walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units);
+  walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units, (int)blockIdx.x, (int)gridDim.x);
 }
 
 template <int WM, int NTMAX, bool TA, bool TB>

@@ -1400,10 +1400,10 @@ __device__ __forceinline__ int pick_units(int cnt) {
 // The walk of one workgroup over its share of the (M tile, unit) space.
 template <int WM, int NTMAX, class P>
 __device__ __forceinline__ void walk_units(const P& p, float* ldsA, float* ldsB, int strideA, int strideB,
-                                           int n_units, int total_units) {
+                                           int n_units, int total_units, int wg, int n_wg) {
   constexpr int WN = 4 / WM;
-  long long u0 = (long long)total_units * blockIdx.x / gridDim.x;
-  const long long u1 = (long long)total_units * (blockIdx.x + 1) / gridDim.x;
+  long long u0 = (long long)total_units * wg / n_wg;
+  const long long u1 = (long long)total_units * (wg + 1) / n_wg;
   while (u0 < u1) {
     const int mt = (int)(u0 / n_units), un = (int)(u0 - (long long)mt * n_units);
     long long cnt = u1 - u0;
