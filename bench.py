@@ -328,6 +328,71 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
     return res
 
 
+def bench_depthwise(api, steps, warmup, cpu=True):
+    """Depthwise 3x3 'same' on x[32, 256, 56, 56]: no contraction over channels, so the roofline that binds is
+    HBM: forward reads X and writes Y (K is 9 KB), dX reads dY and reads + writes dX, dK reads X and dY."""
+    N, C, H, KS = 32, 256, 56, 3
+    ci = conv_info((N, C, H, H), (C, C, KS, KS), 1, 1, 'same')
+    rs = np.random.RandomState(0)
+    x = rs.uniform(-1, 1, (N, C, H, H)).astype(np.float32)
+    k = rs.normal(0, 0.5, (C, KS, KS)).astype(np.float32)
+    dy = rs.normal(0, 1, (N, C, ci.OH, ci.OW)).astype(np.float32)
+    desc = api.conv_desc(N, C, H, H, C, KS, KS, ci.OH, ci.OW, ci.PADL, ci.PADT, 1, 1)
+    X, K, dY = Dev(api, x), Dev(api, k), Dev(api, dy)
+    Y, dX, dK = Dev(api, shape=dy.shape), Dev(api, shape=x.shape), Dev(api, shape=k.shape)
+    nx, ny, nk = x.size, dy.size, k.size
+    bytes_pass = {'fwd': 4.0 * (nx + ny + nk), 'dX': 4.0 * (ny + 2 * nx + nk), 'dK': 4.0 * (nx + ny + 2 * nk)}
+    passes = {
+        'fwd': lambda: api.depthwise_conv2d_fwd(0, desc, X.ptr, K.ptr, Y.ptr, 0),
+        'dX': lambda: api.depthwise_conv2d_dgrad(0, desc, dY.ptr, K.ptr, dX.ptr, 1),
+        'dK': lambda: api.depthwise_conv2d_wgrad(0, desc, X.ptr, dY.ptr, dK.ptr, 1),
+    }
+
+    def step():
+        for fn in passes.values():
+            fn()
+
+    for _ in range(warmup):
+        step()
+    api.synchronize(0)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    api.synchronize(0)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    per_pass = {}
+    for name, fn in passes.items():
+        ms = time_events(api, fn, max(steps, 5))
+        per_pass[name] = {'ms': ms, 'alg_gbs': bytes_pass[name] / ms / 1e6,
+                          'frac_hbm': bytes_pass[name] / ms / 1e6 / PEAK_HBM_GBS, 'frac_mfma': 0.0}
+    dom = max(per_pass, key=lambda n: per_pass[n]['ms'])
+    dX.zero()
+    dK.zero()
+    step()
+    total_bytes = sum(bytes_pass.values())
+    res = {'metric': 'depthwise_conv2D fwd+bwd algorithmic GB/s', 'value': total_bytes / wall_ms / 1e6, 'unit': 'GB/s',
+           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True,
+           'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+           'config': {'workload': f"cfgD_depthwise: x[{N}, {C}, {H}, {H}] k[{C}, {KS}, {KS}] stride 1 'same', "
+                                  'step = fwd + dX(+=) + dK(+=)'},
+           'images_per_s': N / wall_ms * 1e3,
+           'roofline': {'bound': 'hbm', 'kernel': dom, 'achieved': per_pass[dom]['alg_gbs'], 'peak': PEAK_HBM_GBS,
+                        'unit': 'GB/s', 'frac': per_pass[dom]['frac_hbm'], 'traffic': None},
+           'passes': per_pass}
+    if cpu:
+        from oracle import depthwise_all
+        t0 = time.perf_counter()
+        ry, rdx, rdk = depthwise_all(x[:4], k, dy[:4], 1, 1, 'same')
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': total_bytes * 4 / N / dt / 1e9, 'unit': 'GB/s', 'cores': 1, 'kind': 'port',
+                               'sample': 'numpy fp64 oracle, 4 of the 32 images, one run'}
+        res['parity'] = {'checked_against': 'fp64 oracle on images 0-3 (Y, dX)',
+                         'max_rel_err': max(rel_err(Y.get()[:4], ry), rel_err(dX.get()[:4], rdx)), 'tolerance': 1e-4}
+    for t in (X, K, dY, Y, dX, dK):
+        t.free()
+    return res
+
+
 def bench_encoder(steps, warmup):
     """cfg5: full training step (forward, backward, SGD) of the 4-layer 5x5
     stride-2 encoder through the litenn-compatible Python API."""
@@ -395,7 +460,7 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='run only a plain device copy of 256 MiB (three launches of the element-wise kernel) and exit: '
                          'the reference reading for the FETCH_SIZE / WRITE_SIZE counters')
-    ap.add_argument('--config', default='cfg3_vgg3x3', choices=list(CONV_CONFIGS) + ['cfg2_matmul', 'cfg5_encoder', 'cfgT_decoder'],
+    ap.add_argument('--config', default='cfg3_vgg3x3', choices=list(CONV_CONFIGS) + ['cfg2_matmul', 'cfg5_encoder', 'cfgT_decoder', 'cfgD_depthwise'],
                     help='workload of the JSON line (default: the headline configuration)')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -430,6 +495,9 @@ def main():
             r = bench_conv_transpose(api, args.steps, args.warmup, cpu=not args.no_cpu)
             f.write(json.dumps(r) + '\n')
             print(f'[bench] cfgT decoder: {r["value"]:.1f} TFLOP/s', file=sys.stderr, flush=True)
+            r = bench_depthwise(api, args.steps, args.warmup, cpu=not args.no_cpu)
+            f.write(json.dumps(r) + '\n')
+            print(f'[bench] cfgD depthwise: {r["value"]:.0f} GB/s', file=sys.stderr, flush=True)
             r = bench_encoder(args.steps, args.warmup)
             f.write(json.dumps(r) + '\n')
             print(f'[bench] cfg5 encoder: {r["value"]:.0f} images/s, {r["ms_per_step"]:.3f} ms/step', file=sys.stderr,
@@ -440,6 +508,8 @@ def main():
         res = bench_encoder(args.steps, args.warmup)
     elif args.config == 'cfgT_decoder':
         res = bench_conv_transpose(api, args.steps, args.warmup, cpu=not args.no_cpu)
+    elif args.config == 'cfgD_depthwise':
+        res = bench_depthwise(api, args.steps, args.warmup, cpu=not args.no_cpu)
     else:
         res = bench_conv(api, args.config, args.steps, args.warmup, cpu=not args.no_cpu)
     if args.all:

@@ -115,6 +115,17 @@ int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, con
 int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
                          float* dW, int beta);
 
+/* ---- depthwise convolution (one KH x KW filter per channel; K is [C,KH,KW], desc.O must equal desc.C).
+ * Y (+)= depthwise(X, K)                 depthwise_conv2D.py:74-96  (O_depthwise_krn)
+ * dX (+)= its data gradient              depthwise_conv2D.py:98-124 (dI_depthwise_krn; the reference always accumulates)
+ * dK (+)= sum over n,oh,ow of im2col(X) * dY   depthwise_conv2D.py:44-49 (unfold, broadcast multiply, reduce_sum) */
+int lnn_depthwise_conv2d_fwd_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* K,
+                                 float* Y, int beta);
+int lnn_depthwise_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* K,
+                                   float* dX, int beta);
+int lnn_depthwise_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
+                                   float* dK, int beta);
+
 /* ---- nc.op.unfold2D (unfold2D.py:6-48): materialised im2col / im2row /
  * transposed im2row.  Shares its index arithmetic with the gather loaders of
  * the convolution kernels and exists so that arithmetic can be checked bit for

@@ -27,6 +27,7 @@ from litenn_amd.core.backward import backward
 
 from litenn_amd.core.op.conv2D import conv2D
 from litenn_amd.core.op.conv2DTranspose import conv2DTranspose
+from litenn_amd.core.op.depthwise_conv2D import depthwise_conv2D
 from litenn_amd.core.op.dual_wise_op import add, sub, mul
 from litenn_amd.core.op.element_wise_op import (add_const, sub_const, mul_const, div_const,
                                                 leaky_relu, relu, square)
@@ -41,6 +42,8 @@ from litenn_amd.core import devices
 from litenn_amd.core.module.Module import Module
 from litenn_amd.core.module.Conv2D import Conv2D
 from litenn_amd.core.module.Conv2DTranspose import Conv2DTranspose
+from litenn_amd.core.module.DepthwiseConv2D import DepthwiseConv2D
+from litenn_amd.core.module.SeparableConv2D import SeparableConv2D
 from litenn_amd.core.module.Dense import Dense
 
 import litenn_amd.core.optimizer as optimizer

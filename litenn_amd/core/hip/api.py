@@ -64,6 +64,9 @@ SIGNATURES = {
                      _ptr, _c_int, _c_i64, _ptr, _c_int, _c_i64, _c_int],
     'lnn_conv2d_fwd_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_fwd_bias_act_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int, ctypes.c_float, _ptr],
+    'lnn_depthwise_conv2d_fwd_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
+    'lnn_depthwise_conv2d_dgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
+    'lnn_depthwise_conv2d_wgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_dgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_wgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_unfold2d_f32': [_c_int] + [_c_int] * 14 + [_ptr, _ptr, _c_int],
@@ -213,6 +216,18 @@ def conv2d_dgrad(dev, desc, dY, W, dX, beta=1):
 
 def conv2d_wgrad(dev, desc, X, dY, dW, beta=1):
     check(lib.lnn_conv2d_wgrad_f32(dev, ctypes.byref(desc), X, dY, dW, int(beta)))
+
+
+def depthwise_conv2d_fwd(dev, desc, X, K, Y, beta=0):
+    check(lib.lnn_depthwise_conv2d_fwd_f32(dev, ctypes.byref(desc), X, K, Y, int(beta)))
+
+
+def depthwise_conv2d_dgrad(dev, desc, dY, K, dX, beta=1):
+    check(lib.lnn_depthwise_conv2d_dgrad_f32(dev, ctypes.byref(desc), dY, K, dX, int(beta)))
+
+
+def depthwise_conv2d_wgrad(dev, desc, X, dY, dK, beta=1):
+    check(lib.lnn_depthwise_conv2d_wgrad_f32(dev, ctypes.byref(desc), X, dY, dK, int(beta)))
 
 
 def unfold2d(dev, N, C, H, W, OH, OW, KH, KW, PADL, PADT, dilation, stride, order, is_transpose, src, dst, beta=0):

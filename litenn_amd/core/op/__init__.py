@@ -13,6 +13,7 @@ def accumulate_target(grad_t):
 
 from .conv2D import conv2D, conv2D_bias_act
 from .conv2DTranspose import conv2DTranspose
+from .depthwise_conv2D import depthwise_conv2D
 from .element_wise_op import (element_wise_op,
                               add_const_op as add_const,
                               div_const_op as div_const,

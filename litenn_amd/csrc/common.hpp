@@ -43,6 +43,9 @@ int launch_gemm(DeviceCtx* ctx, int ta, int tb, int batch, int M, int N, int K, 
                 long long sA, const float* B, int ldb, long long sB, float* C, int ldc, long long sC, int beta);
 int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta,
                     const float* bias, int act, float slope);
+int launch_dw_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* K, float* Y, int beta);
+int launch_dw_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* K, float* dX, int beta);
+int launch_dw_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dK, int beta);
 int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta);
 int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta);
 

@@ -286,6 +286,23 @@ int lnn_conv2d_fwd_bias_act_f32(int dev, const lnn_conv2d_desc* d, const float* 
   return launch_conv_fwd(ctx, d, X, W, Y, 0, bias, act, slope);
 }
 
+int lnn_depthwise_conv2d_fwd_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* K, float* Y, int beta) {
+  CTX(dev);
+  return launch_dw_fwd(ctx, d, X, K, Y, beta);
+}
+
+int lnn_depthwise_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* K, float* dX,
+                                   int beta) {
+  CTX(dev);
+  return launch_dw_dgrad(ctx, d, dY, K, dX, beta);
+}
+
+int lnn_depthwise_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dK,
+                                   int beta) {
+  CTX(dev);
+  return launch_dw_wgrad(ctx, d, X, dY, dK, beta);
+}
+
 int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta) {
   CTX(dev);
   return launch_conv_dgrad(ctx, d, dY, W, dX, beta);

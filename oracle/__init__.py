@@ -23,6 +23,10 @@ Pinning status (what checks each function, independent of its own formula):
                      linearity in the kernel, stride-1 == conv2D with the
                      kernel flipped and its channel axes swapped
                      (tests/test_oracle_conv_transpose.py)
+  depthwise          equals the pinned conv2D oracle applied to a kernel that is
+   fwd/dI/dK         zero off the channel diagonal (forward, dI, and the
+                     diagonal of dK), exact on integers
+                     (tests/test_oracle_depthwise.py)
   matmul fwd/dA/dB   np.matmul fp64 on integer-valued data (exact) and
                      adjoint identities (tests/test_oracle_matmul.py)
   refpath (C, fp32)  must reproduce the fp64 oracle exactly on integer-valued
@@ -37,4 +41,5 @@ from .unfold import (unfold_index_map, unfold_T_index_map,        # noqa: F401
 from .conv import conv2d_fwd, conv2d_dx, conv2d_dw, conv2d_all    # noqa: F401
 from .conv_transpose import (conv2d_transpose_fwd, conv2d_transpose_di,   # noqa: F401
                              conv2d_transpose_dk, conv2d_transpose_all)
+from .depthwise import depthwise_fwd, depthwise_di, depthwise_dk, depthwise_all   # noqa: F401
 from .matmul import matmul_fwd, matmul_da, matmul_db              # noqa: F401

@@ -7,11 +7,12 @@ package has no such path: without liblitenn_hip.so and a GPU it raises.
 """
 import numpy as np
 
-from oracle import (conv2d_fwd, conv2d_dx, conv2d_dw, unfold_index_map, unfold_T_index_map, apply_index_map)
+from oracle import (conv2d_fwd, conv2d_dx, conv2d_dw, unfold_index_map, unfold_T_index_map, apply_index_map,
+                    depthwise_fwd, depthwise_di, depthwise_dk)
 from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
-         'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad',
+         'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
          'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update']
 
 
@@ -115,6 +116,22 @@ class FakeHip:
         self.launches += 1
         xs, ws, ys, pad = self._geom(d)
         self._put(self.f(dW, ws), conv2d_dw(self.f(X, xs), self.f(dY, ys), ws, d.stride, d.dilation, pad), beta)
+
+    def depthwise_conv2d_fwd(self, dev, d, X, K, Y, beta=0):
+        self.launches += 1
+        xs, ws, ys, pad = self._geom(d)
+        self._put(self.f(Y, ys), depthwise_fwd(self.f(X, xs), self.f(K, (d.C, d.KH, d.KW)), d.stride, d.dilation, pad), beta)
+
+    def depthwise_conv2d_dgrad(self, dev, d, dY, K, dX, beta=1):
+        self.launches += 1
+        xs, ws, ys, pad = self._geom(d)
+        self._put(self.f(dX, xs), depthwise_di(self.f(dY, ys), self.f(K, (d.C, d.KH, d.KW)), xs, d.stride, d.dilation, pad), beta)
+
+    def depthwise_conv2d_wgrad(self, dev, d, X, dY, dK, beta=1):
+        self.launches += 1
+        xs, ws, ys, pad = self._geom(d)
+        ks = (d.C, d.KH, d.KW)
+        self._put(self.f(dK, ks), depthwise_dk(self.f(X, xs), self.f(dY, ys), ks, d.stride, d.dilation, pad), beta)
 
     def unfold2d(self, dev, N, C, H, W, OH, OW, KH, KW, PADL, PADT, dil, stride, order, is_transpose, src, dst, beta=0):
         self.launches += 1

@@ -9,7 +9,7 @@ import itertools
 import numpy as np
 import pytest
 
-from oracle import conv2d_all, conv2d_transpose_all, info_conv2d
+from oracle import conv2d_all, conv2d_transpose_all, depthwise_all, info_conv2d
 
 
 def test_conv2d_reference_style(nn_backend):
@@ -123,6 +123,71 @@ def test_conv2d_bias_act_equals_separate_ops(nn_backend):
         nc.op.conv2D_bias_act(nn.Tensor((1, 2, 4, 4)), nn.Tensor((3, 2, 3, 3)), nn.Tensor((4,)))
     with pytest.raises(ValueError):
         nc.op.conv2D_bias_act(nn.Tensor((1, 2, 4, 4)), nn.Tensor((3, 2, 3, 3)), leaky_relu_alpha=0.0)
+
+
+def test_depthwise_conv2d_reference_style(nn_backend):
+    """depthwise_conv2D_test (depthwise_conv2D.py:128-…): its grid of paddings,
+    dilations, strides, kernel sizes and shapes, exact on integer-valued data,
+    gradients accumulated onto a pre-filled 1.0."""
+    nn = nn_backend
+    rs = np.random.RandomState(6)
+    n_cases = 0
+    for padding, dilation, stride, ks in itertools.product(['same', 'valid', 0, 1, 2], [1, 2], [1, 2, 3], [1, 3, 5, 7]):
+        for n, ic, hw in [(1, 1, 8), (4, 2, 16), (1, 4, 32)]:
+            if padding == 'valid' and hw < (ks - 1) * dilation + 1:
+                continue
+            x_n = rs.randint(2 ** 4, size=(n, ic, hw, hw)).astype(np.float32)
+            k_n = rs.randint(2 ** 4, size=(ic, ks, ks)).astype(np.float32)
+            x, k = nn.Tensor_from_value(x_n), nn.Tensor_from_value(k_n)
+            try:
+                ci = info_conv2d(hw, hw, ks, ks, stride, dilation, padding)
+            except ValueError:
+                continue
+            if ci.OH <= 0 or ci.OW <= 0:
+                continue
+            y = nn.depthwise_conv2D(x, k, stride=stride, dilation=dilation, padding=padding)
+            g_n = rs.randint(2 ** 4, size=tuple(y.shape)).astype(np.float32)
+            ry, rdi, rdk = depthwise_all(x_n, k_n, g_n, stride, dilation, padding)
+            assert np.array_equal(y.np(), ry), (padding, dilation, stride, ks, n, ic, hw)
+            x.get_grad().fill(1.0)
+            k.get_grad().fill(1.0)
+            nn.backward({y: g_n}, grad_for_non_trainables=True)
+            assert np.array_equal(x.get_grad().np() - 1.0, rdi), (padding, dilation, stride, ks, n, ic, hw)
+            assert np.array_equal(k.get_grad().np() - 1.0, rdk), (padding, dilation, stride, ks, n, ic, hw)
+            n_cases += 1
+    assert n_cases > 250
+
+
+def test_depthwise_and_separable_modules(nn_backend):
+    nn = nn_backend
+    rs = np.random.RandomState(8)
+    dk = rs.randint(-2, 3, size=(4, 3, 3)).astype(np.float32)
+    pk = rs.randint(-2, 3, size=(6, 4, 1, 1)).astype(np.float32)
+    b = rs.randint(-2, 3, size=(6,)).astype(np.float32)
+    x_n = rs.randint(-2, 3, size=(2, 4, 8, 8)).astype(np.float32)
+    sep = nn.SeparableConv2D(4, 6, 3, depthwise_initializer=nn.initializer.NumpyArray(dk),
+                             pointwise_initializer=nn.initializer.NumpyArray(pk),
+                             bias_initializer=nn.initializer.NumpyArray(b))
+    x = nn.Tensor_from_value(x_n)
+    y = sep(x)
+    mid, _, _ = depthwise_all(x_n, dk, np.zeros((2, 4, 8, 8)), 1, 1, 'same')
+    ref, _, _ = conv2d_all(mid, pk, np.zeros((2, 6, 8, 8)), 1, 1, 'valid')
+    assert np.array_equal(y.np(), ref + b.reshape(1, -1, 1, 1))
+    y.backward(grad_for_non_trainables=True)
+    ones = np.ones((2, 6, 8, 8))
+    _, dmid, dpk = conv2d_all(mid, pk, ones, 1, 1, 'valid')
+    _, dx, ddk = depthwise_all(x_n, dk, dmid, 1, 1, 'same')
+    assert np.array_equal(x.get_grad().np(), dx)
+    assert np.array_equal(sep.depthwise_kernel.get_grad().np(), ddk)
+    assert np.array_equal(sep.pointwise_kernel.get_grad().np(), dpk)
+    assert np.array_equal(sep.bias.get_grad().np(), np.full((6,), 2 * 64, np.float32))
+    dwm = nn.DepthwiseConv2D(4, 3, use_bias=False, depthwise_initializer=nn.initializer.NumpyArray(dk))
+    y2 = dwm(nn.Tensor_from_value(x_n))
+    assert np.array_equal(y2.np(), mid)
+    with pytest.raises(ValueError):
+        nn.depthwise_conv2D(x, nn.Tensor((4, 1, 3, 3)))
+    with pytest.raises(ValueError):
+        nn.depthwise_conv2D(x, nn.Tensor((5, 3, 3)))
 
 
 def test_matmul_reference_style(nn_backend):

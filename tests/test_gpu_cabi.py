@@ -11,6 +11,7 @@ import itertools
 import numpy as np
 import pytest
 
+from oracle import depthwise_all
 from oracle import (info_conv2d, conv2d_all, conv2d_fwd, conv2d_dx, conv2d_dw, unfold_index_map,
                     unfold_T_index_map, matmul_fwd)
 from tests.gpu_util import DevArr, rel_err, say
@@ -333,6 +334,62 @@ def test_conv_fwd_bias_act_matches_separate_kernels(hip):
         assert np.array_equal(Y1.get(), Y2.get()), (xs, ws)
     with pytest.raises(hip.HipException):
         hip.conv2d_fwd_bias_act(0, desc, X.ptr, W.ptr, B.ptr, 7, 0.1, Y1.ptr)
+
+
+def test_depthwise_integer_exact_and_float(hip):
+    """Depthwise forward / dgrad / wgrad through the C ABI: integer-exact over
+    strides, dilations, kernel sizes and paddings with '=' and '+=', then a
+    larger float case within tolerance (the kernel gradient sums tens of
+    thousands of products per tap)."""
+    rs = np.random.RandomState(51)
+    cnt = 0
+    for s, d, ks, padding, xs in itertools.product((1, 2, 3), (1, 2), (1, 2, 3, 5), ('same', 'valid', 1, (2, 0, 1, 3)),
+                                                   ((2, 3, 11, 9), (1, 70, 6, 7))):
+        try:
+            ci = info_conv2d(xs[2], xs[3], ks, ks, s, d, padding)
+        except ValueError:
+            continue
+        if ci.OH <= 0 or ci.OW <= 0:
+            continue
+        if cnt % 40 == 0:
+            say(f'depthwise case {cnt}: x={xs} ks={ks} s={s} d={d} pad={padding}')
+        x = rs.randint(-4, 5, size=xs).astype(np.float32)
+        k = rs.randint(-4, 5, size=(xs[1], ks, ks)).astype(np.float32)
+        dy = rs.randint(-4, 5, size=(xs[0], xs[1], ci.OH, ci.OW)).astype(np.float32)
+        ry, rdx, rdk = depthwise_all(x, k, dy, s, d, padding)
+        desc = hip.conv_desc(xs[0], xs[1], xs[2], xs[3], xs[1], ks, ks, ci.OH, ci.OW, ci.PADL, ci.PADT, s, d)
+        pre = None if cnt % 2 else 2.0
+        X, K, dY = DevArr(hip, x), DevArr(hip, k), DevArr(hip, dy)
+        Y = DevArr(hip, shape=dy.shape, fill=np.nan)
+        dX = DevArr(hip, shape=xs, fill=np.nan if pre is None else pre)
+        dK = DevArr(hip, shape=k.shape, fill=np.nan if pre is None else pre)
+        beta = 0 if pre is None else 1
+        hip.depthwise_conv2d_fwd(0, desc, X.ptr, K.ptr, Y.ptr, 0)
+        hip.depthwise_conv2d_dgrad(0, desc, dY.ptr, K.ptr, dX.ptr, beta)
+        hip.depthwise_conv2d_wgrad(0, desc, X.ptr, dY.ptr, dK.ptr, beta)
+        off = 0.0 if pre is None else pre
+        assert np.array_equal(Y.get(), ry), ('fwd', xs, ks, s, d, padding)
+        assert np.array_equal(dX.get() - off, rdx), ('dX', xs, ks, s, d, padding)
+        assert np.array_equal(dK.get() - off, rdk), ('dK', xs, ks, s, d, padding)
+        cnt += 1
+    assert cnt > 150
+    xs, ks = (4, 96, 56, 56), 3
+    say(f'depthwise float x={xs}')
+    ci = info_conv2d(56, 56, ks, ks, 1, 1, 'same')
+    x = rs.normal(0, 1, xs).astype(np.float32)
+    k = rs.normal(0, 1, (96, ks, ks)).astype(np.float32)
+    dy = rs.normal(0, 1, xs).astype(np.float32)
+    ry, rdx, rdk = depthwise_all(x, k, dy, 1, 1, 'same')
+    desc = hip.conv_desc(4, 96, 56, 56, 96, ks, ks, 56, 56, ci.PADL, ci.PADT, 1, 1)
+    X, K, dY = DevArr(hip, x), DevArr(hip, k), DevArr(hip, dy)
+    Y, dX, dK = DevArr(hip, shape=xs, fill=np.nan), DevArr(hip, shape=xs, fill=np.nan), DevArr(hip, shape=k.shape, fill=np.nan)
+    hip.depthwise_conv2d_fwd(0, desc, X.ptr, K.ptr, Y.ptr, 0)
+    hip.depthwise_conv2d_dgrad(0, desc, dY.ptr, K.ptr, dX.ptr, 0)
+    hip.depthwise_conv2d_wgrad(0, desc, X.ptr, dY.ptr, dK.ptr, 0)
+    assert rel_err(Y.get(), ry) <= TOL and rel_err(dX.get(), rdx) <= TOL and rel_err(dK.get(), rdk) <= TOL
+    bad = hip.conv_desc(4, 96, 56, 56, 64, ks, ks, 56, 56, 1, 1, 1, 1)
+    with pytest.raises(hip.HipException):
+        hip.depthwise_conv2d_fwd(0, bad, X.ptr, K.ptr, Y.ptr, 0)
 
 
 # benchmark geometries at a reduced batch (the oracle materialises im2col in fp64)
