@@ -13,99 +13,217 @@
 #include "common.hpp"
 #include "tile_engine.hpp"
 
+// the tap loops carry an unroll request that only the compile-time filter sizes can honour
+#pragma clang diagnostic ignored "-Wpass-failed"
+
 namespace lnn {
 
 struct DwGeom {
   int N, C, IH, IW, KH, KW, OH, OW, PADL, PADT, S, D;
-  FastDiv dOW, dOH, dIW, dIH, dC;
+  FastDiv dOW, dIW, dS;
 };
 
-__global__ __launch_bounds__(256) void dw_fwd_kernel(DwGeom g, const float* __restrict__ X, const float* __restrict__ K,
-                                                     float* __restrict__ Y, uint32_t n, int beta) {
-  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += gridDim.x * 256u) {
-    const uint32_t q = g.dOW.div(i), ow = i - q * g.OW;
-    const uint32_t nc = g.dOH.div(q), oh = q - nc * g.OH;           // nc = n*C + c
-    const uint32_t c = nc - g.dC.div(nc) * g.C;
-    const float* xp = X + (size_t)nc * g.IH * g.IW;
-    const float* kp = K + (size_t)c * g.KH * g.KW;
-    const int ih0 = (int)oh * g.S - g.PADT, iw0 = (int)ow * g.S - g.PADL;
-    float v = 0.0f;
-    for (int kh = 0; kh < g.KH; ++kh) {
-      const int ih = ih0 + kh * g.D;
-      if ((uint32_t)ih < (uint32_t)g.IH)
-        for (int kw = 0; kw < g.KW; ++kw) {
-          const int iw = iw0 + kw * g.D;
-          if ((uint32_t)iw < (uint32_t)g.IW) v += xp[ih * g.IW + iw] * kp[kh * g.KW + kw];
-        }
-    }
-    Y[i] = beta ? Y[i] + v : v;
+// All three kernels work on one band of rows of one (image, channel) plane per block: the rows of the
+// source plane(s) that the band touches are copied to LDS once with coalesced reads, then every thread
+// produces elements from LDS.  Each input element leaves HBM once.
+// LDSF floats of source rows per block: 4096 (16 KB, eight blocks per compute unit hide the copy latency)
+// when a useful band fits, else 32768 (128 KB, one block) for very wide rows.
+constexpr int kDwSmall = 4096, kDwLarge = 32768;
+
+__device__ __forceinline__ void dw_copy_rows(float* lds, const float* __restrict__ plane, int row_lo, int row_hi, int W) {
+  const int n = (row_hi - row_lo + 1) * W;
+  const float* src = plane + (size_t)row_lo * W;
+  if (((reinterpret_cast<uintptr_t>(src) | (uintptr_t)(n * 4)) & 15) == 0) {   // block-uniform
+    for (int i = threadIdx.x; i < n / 4; i += 256)
+      reinterpret_cast<f32x4*>(lds)[i] = reinterpret_cast<const f32x4*>(src)[i];
+  } else {
+    for (int i = threadIdx.x; i < n; i += 256) lds[i] = src[i];
   }
 }
 
-__global__ __launch_bounds__(256) void dw_dgrad_kernel(DwGeom g, const float* __restrict__ dY,
-                                                       const float* __restrict__ K, float* __restrict__ dX, uint32_t n,
-                                                       int beta, FastDiv dS) {
-  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += gridDim.x * 256u) {
-    const uint32_t q = g.dIW.div(i), iw = i - q * g.IW;
-    const uint32_t nc = g.dIH.div(q), ih = q - nc * g.IH;
-    const uint32_t c = nc - g.dC.div(nc) * g.C;
-    const float* yp = dY + (size_t)nc * g.OH * g.OW;
-    const float* kp = K + (size_t)c * g.KH * g.KW;
+// KS > 0: square KS x KS filter known at compile time (tap loops unrolled, filter in registers);
+// KS == 0: any KH x KW, filter read from LDS.
+template <int KS>
+struct DwFilter {
+  float k[KS > 0 ? KS * KS : 1];
+  const float* lk;
+  int KH, KW;
+  __device__ __forceinline__ void load(const float* __restrict__ kp, float* ldsk, int kh, int kw) {
+    KH = KS > 0 ? KS : kh;
+    KW = KS > 0 ? KS : kw;
+    if (KS > 0) {
+#pragma unroll
+      for (int i = 0; i < KS * KS; ++i) k[i] = kp[i];
+    } else {
+      for (int i = threadIdx.x; i < kh * kw; i += 256) ldsk[i] = kp[i];
+      lk = ldsk;
+    }
+  }
+  __device__ __forceinline__ float at(int kh, int kw) const { return KS > 0 ? k[kh * KS + kw] : lk[kh * KW + kw]; }
+};
+constexpr int kDwMaxTaps = 1024;   // runtime-sized filters of up to 32 x 32 taps
+
+// forward: Y rows [r0, r1) of the plane from X rows [lo, hi]
+template <int KS, int LDSF>
+__global__ __launch_bounds__(256) void dw_fwd_kernel(DwGeom g, const float* __restrict__ X, const float* __restrict__ K,
+                                                     float* __restrict__ Y, int bands, int TH, int beta) {
+  __shared__ __attribute__((aligned(16))) float lds[LDSF];
+  __shared__ float ldsk[KS > 0 ? 1 : kDwMaxTaps];
+  const int plane = blockIdx.x / bands, band = blockIdx.x - plane * bands;
+  const int c = plane % g.C;
+  const int r0 = band * TH, r1 = r0 + TH < g.OH ? r0 + TH : g.OH;
+  int lo = r0 * g.S - g.PADT, hi = (r1 - 1) * g.S - g.PADT + (g.KH - 1) * g.D;
+  lo = lo < 0 ? 0 : lo;
+  hi = hi >= g.IH ? g.IH - 1 : hi;
+  if (hi >= lo) dw_copy_rows(lds, X + (size_t)plane * g.IH * g.IW, lo, hi, g.IW);
+  DwFilter<KS> f;
+  f.load(K + (size_t)c * g.KH * g.KW, ldsk, g.KH, g.KW);
+  __syncthreads();
+  float* yp = Y + (size_t)plane * g.OH * g.OW;
+  const int n = (r1 - r0) * g.OW;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const int r = (int)g.dOW.div((uint32_t)i), ow = i - r * g.OW, oh = r0 + r;
+    const int ih0 = oh * g.S - g.PADT, iw0 = ow * g.S - g.PADL;
     float v = 0.0f;
-    for (int kh = 0; kh < g.KH; ++kh) {
-      const int nh = (int)ih + g.PADT - kh * g.D;
-      if (nh < 0) break;                       // later taps only move further up
-      const uint32_t oh = dS.div((uint32_t)nh);
-      if (oh * (uint32_t)g.S != (uint32_t)nh || oh >= (uint32_t)g.OH) continue;
-      for (int kw = 0; kw < g.KW; ++kw) {
-        const int nw = (int)iw + g.PADL - kw * g.D;
-        if (nw < 0) break;
-        const uint32_t ow = dS.div((uint32_t)nw);
-        if (ow * (uint32_t)g.S == (uint32_t)nw && ow < (uint32_t)g.OW) v += yp[oh * g.OW + ow] * kp[kh * g.KW + kw];
+#pragma unroll
+    for (int kh = 0; kh < f.KH; ++kh) {
+      const int ih = ih0 + kh * g.D;
+      if ((uint32_t)ih < (uint32_t)g.IH) {
+        const float* row = lds + (ih - lo) * g.IW;
+#pragma unroll
+        for (int kw = 0; kw < f.KW; ++kw) {
+          const int iw = iw0 + kw * g.D;
+          if ((uint32_t)iw < (uint32_t)g.IW) v += row[iw] * f.at(kh, kw);
+        }
       }
     }
-    dX[i] = beta ? dX[i] + v : v;
+    const int o = oh * g.OW + ow;
+    yp[o] = beta ? yp[o] + v : v;
   }
 }
 
-// grid (C, splits): block (c, s) sums its share of the N*OH*OW pixels of channel c for every tap and
-// writes part[(c*splits + s)*KK + tap]; the shares are contiguous pixel ranges, the order of addition is fixed.
+// data gradient: dX rows [r0, r1) of the plane from dY rows [lo, hi]
+template <int KS, int LDSF>
+__global__ __launch_bounds__(256) void dw_dgrad_kernel(DwGeom g, const float* __restrict__ dY,
+                                                       const float* __restrict__ K, float* __restrict__ dX, int bands,
+                                                       int TH, int beta) {
+  __shared__ __attribute__((aligned(16))) float lds[LDSF];
+  const int plane = blockIdx.x / bands, band = blockIdx.x - plane * bands;
+  const int c = plane % g.C;
+  const int r0 = band * TH, r1 = r0 + TH < g.IH ? r0 + TH : g.IH;
+  // output rows oh = (ih + PT - kh*D) / S for ih in [r0, r1)
+  int lo = r0 + g.PADT - (g.KH - 1) * g.D, hi = (r1 - 1 + g.PADT) / g.S;
+  lo = lo <= 0 ? 0 : (lo + g.S - 1) / g.S;
+  hi = hi >= g.OH ? g.OH - 1 : hi;
+  if (hi >= lo) dw_copy_rows(lds, dY + (size_t)plane * g.OH * g.OW, lo, hi, g.OW);
+  __shared__ float ldsk[KS > 0 ? 1 : kDwMaxTaps];
+  DwFilter<KS> f;
+  f.load(K + (size_t)c * g.KH * g.KW, ldsk, g.KH, g.KW);
+  __syncthreads();
+  float* xp = dX + (size_t)plane * g.IH * g.IW;
+  const int n = (r1 - r0) * g.IW;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const int r = (int)g.dIW.div((uint32_t)i), iw = i - r * g.IW, ih = r0 + r;
+    float v = 0.0f;
+#pragma unroll
+    for (int kh = 0; kh < f.KH; ++kh) {
+      const int nh = ih + g.PADT - kh * g.D;
+      const int oh = (int)g.dS.div((uint32_t)nh & 0x7fffffffu);
+      if (nh >= 0 && oh * g.S == nh && oh < g.OH) {
+        const float* row = lds + (oh - lo) * g.OW;
+#pragma unroll
+        for (int kw = 0; kw < f.KW; ++kw) {
+          const int nw = iw + g.PADL - kw * g.D;
+          const int ow = (int)g.dS.div((uint32_t)nw & 0x7fffffffu);
+          if (nw >= 0 && ow * g.S == nw && ow < g.OW) v += row[ow] * f.at(kh, kw);
+        }
+      }
+    }
+    const int o = ih * g.IW + iw;
+    xp[o] = beta ? xp[o] + v : v;
+  }
+}
+
+// kernel gradient: block (plane, band) holds dY rows [r0, r1) and the X rows under them and writes, per tap,
+// the sum of X * dY over the band to part[(plane*bands + band)*KK + tap]
+template <int KS, int LDSF>
 __global__ __launch_bounds__(256) void dw_wgrad_kernel(DwGeom g, const float* __restrict__ X,
                                                        const float* __restrict__ dY, float* __restrict__ part,
-                                                       int splits) {
+                                                       int bands, int TH) {
+  __shared__ __attribute__((aligned(16))) float ldsx[LDSF];
+  __shared__ __attribute__((aligned(16))) float ldsy[LDSF / 2];
   __shared__ float red[4];
-  const int c = blockIdx.x, s = blockIdx.y;
-  const uint32_t OHW = (uint32_t)g.OH * g.OW, P = (uint32_t)g.N * OHW;
-  const uint32_t p0 = (uint32_t)((uint64_t)P * s / splits), p1 = (uint32_t)((uint64_t)P * (s + 1) / splits);
-  const FastDiv dOHW = g.dIH;   // the host passes the divider by OH*OW in this slot for this kernel
-  for (int kh = 0; kh < g.KH; ++kh)
-    for (int kw = 0; kw < g.KW; ++kw) {
-      float v = 0.0f;
-      for (uint32_t p = p0 + threadIdx.x; p < p1; p += 256u) {
-        const uint32_t img = dOHW.div(p), rem = p - img * OHW;
-        const uint32_t oh = g.dOW.div(rem), ow = rem - oh * g.OW;
-        const int ih = (int)oh * g.S - g.PADT + kh * g.D, iw = (int)ow * g.S - g.PADL + kw * g.D;
-        if ((uint32_t)ih < (uint32_t)g.IH && (uint32_t)iw < (uint32_t)g.IW)
-          v += X[((size_t)img * g.C + c) * g.IH * g.IW + ih * g.IW + iw] * dY[((size_t)img * g.C + c) * OHW + rem];
+  const int plane = blockIdx.x / bands, band = blockIdx.x - plane * bands;
+  const int r0 = band * TH, r1 = r0 + TH < g.OH ? r0 + TH : g.OH;
+  int lo = r0 * g.S - g.PADT, hi = (r1 - 1) * g.S - g.PADT + (g.KH - 1) * g.D;
+  lo = lo < 0 ? 0 : lo;
+  hi = hi >= g.IH ? g.IH - 1 : hi;
+  if (hi >= lo) dw_copy_rows(ldsx, X + (size_t)plane * g.IH * g.IW, lo, hi, g.IW);
+  dw_copy_rows(ldsy, dY + (size_t)plane * g.OH * g.OW, r0, r1 - 1, g.OW);
+  __syncthreads();
+  const int n = (r1 - r0) * g.OW, KK = g.KH * g.KW;
+  float* out = part + ((size_t)plane * bands + band) * KK;
+  if (KS > 0) {
+    // every thread keeps one running sum per tap over its pixels, then the taps are reduced over the block
+    constexpr int T = KS > 0 ? KS * KS : 1;
+    float acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) {
+      const int r = (int)g.dOW.div((uint32_t)i), ow = i - r * g.OW;
+      const int ih0 = (r0 + r) * g.S - g.PADT, iw0 = ow * g.S - g.PADL;
+      const float dyv = ldsy[i];
+#pragma unroll
+      for (int kh = 0; kh < KS; ++kh) {
+        const int ih = ih0 + kh * g.D;
+        const float* row = ldsx + (ih - lo) * g.IW;
+#pragma unroll
+        for (int kw = 0; kw < KS; ++kw) {
+          const int iw = iw0 + kw * g.D;
+          const bool ok = (uint32_t)ih < (uint32_t)g.IH && (uint32_t)iw < (uint32_t)g.IW;
+          acc[kh * KS + kw] += ok ? row[iw] * dyv : 0.0f;
+        }
       }
-      // wavefront butterfly, then the four wavefront sums in a fixed order
+    }
+    __shared__ float red2[4][T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      float v = acc[t];
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-      if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-      __syncthreads();
-      if (threadIdx.x == 0)
-        part[((size_t)c * splits + s) * (g.KH * g.KW) + kh * g.KW + kw] = (red[0] + red[1]) + (red[2] + red[3]);
-      __syncthreads();
+      if ((threadIdx.x & 63) == 0) red2[threadIdx.x >> 6][t] = v;
     }
+    __syncthreads();
+    if (threadIdx.x < T) out[threadIdx.x] = (red2[0][threadIdx.x] + red2[1][threadIdx.x]) + (red2[2][threadIdx.x] + red2[3][threadIdx.x]);
+  } else {
+    for (int kh = 0; kh < g.KH; ++kh)
+      for (int kw = 0; kw < g.KW; ++kw) {
+        float v = 0.0f;
+        for (int i = threadIdx.x; i < n; i += 256) {
+          const int r = (int)g.dOW.div((uint32_t)i), ow = i - r * g.OW;
+          const int ih = (r0 + r) * g.S - g.PADT + kh * g.D, iw = ow * g.S - g.PADL + kw * g.D;
+          if ((uint32_t)ih < (uint32_t)g.IH && (uint32_t)iw < (uint32_t)g.IW) v += ldsx[(ih - lo) * g.IW + iw] * ldsy[i];
+        }
+        // wavefront butterfly, then the four wavefront sums in a fixed order
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+        __syncthreads();
+        if (threadIdx.x == 0) out[kh * g.KW + kw] = (red[0] + red[1]) + (red[2] + red[3]);
+        __syncthreads();
+      }
+  }
 }
 
-__global__ void dw_wgrad_finish_kernel(float* __restrict__ dK, const float* __restrict__ part, int n, int KK, int splits,
-                                       int beta) {
+// dK[c][tap] (+)= sum over images and bands, in a fixed order
+__global__ void dw_wgrad_finish_kernel(float* __restrict__ dK, const float* __restrict__ part, int C, int KK, int N,
+                                       int bands, int beta) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;   // i = c*KK + tap
-  if (i >= n) return;
+  if (i >= C * KK) return;
   const int c = i / KK, tap = i - c * KK;
   float v = 0.0f;
-  for (int s = 0; s < splits; ++s) v += part[((size_t)c * splits + s) * KK + tap];
+  for (int n = 0; n < N; ++n)
+    for (int b = 0; b < bands; ++b) v += part[(((size_t)n * C + c) * bands + b) * KK + tap];
   dK[i] = beta ? dK[i] + v : v;
 }
 
@@ -121,15 +239,17 @@ static int dw_geom(const lnn_conv2d_desc* d, DwGeom& g, const char* who) {
     return set_error(LNN_ERR_UNSUPPORTED, std::string(who) + ": a tensor of 2 GiB or more");
   g.N = d->N; g.C = d->C; g.IH = d->IH; g.IW = d->IW; g.KH = d->KH; g.KW = d->KW; g.OH = d->OH; g.OW = d->OW;
   g.PADL = d->PADL; g.PADT = d->PADT; g.S = d->stride; g.D = d->dilation;
-  g.dOW = make_fastdiv(g.OW); g.dOH = make_fastdiv(g.OH); g.dIW = make_fastdiv(g.IW); g.dIH = make_fastdiv(g.IH);
-  g.dC = make_fastdiv(g.C);
+  g.dOW = make_fastdiv(g.OW); g.dIW = make_fastdiv(g.IW); g.dS = make_fastdiv(g.S);
+  if ((uint64_t)d->N * d->C > 0x7fffffffull / 64) return set_error(LNN_ERR_UNSUPPORTED, std::string(who) + ": too many planes");
   return LNN_OK;
 }
 
-static dim3 dw_grid(uint32_t n, int cus) {
-  uint64_t blocks = ((uint64_t)n + 255) / 256;
-  const uint64_t cap = (uint64_t)cus * 32;
-  return dim3((unsigned)(blocks > cap ? cap : (blocks < 1 ? 1 : blocks)));
+// Rows of the produced plane per block such that the source rows they touch fit in `floats` of LDS:
+// src_rows(TH) = (TH - 1) * num / den + extra + 1 rows of `width` floats.  0 if even one row does not fit.
+static int dw_band_rows(int out_rows, int width, long long num, long long den, long long extra, int floats) {
+  int th = out_rows;
+  while (th >= 1 && (((long long)(th - 1) * num) / den + extra + 1) * width > floats) th = th > 8 ? th * 3 / 4 : th - 1;
+  return th;
 }
 
 int launch_dw_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* K, float* Y, int beta) {
@@ -137,8 +257,24 @@ int launch_dw_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, cons
   int st = dw_geom(d, g, "depthwise_conv2d_fwd");
   if (st != LNN_OK) return st;
   if (!X || !K || !Y) return set_error(LNN_ERR_INVALID, "depthwise_conv2d_fwd: null pointer");
-  const uint32_t n = (uint32_t)((uint64_t)g.N * g.C * g.OH * g.OW);
-  hipLaunchKernelGGL(dw_fwd_kernel, dw_grid(n, ctx->cus), dim3(256), 0, ctx->stream, g, X, K, Y, n, beta ? 1 : 0);
+  int TH = dw_band_rows(g.OH, g.IW, g.S, 1, (long long)(g.KH - 1) * g.D, kDwSmall);
+  const bool small = TH >= 8 || TH >= g.OH;
+  if (!small) TH = dw_band_rows(g.OH, g.IW, g.S, 1, (long long)(g.KH - 1) * g.D, kDwLarge);
+  if (TH < 1) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d_fwd: image rows wider than the LDS band");
+  const int bands = (g.OH + TH - 1) / TH;
+  if (g.KH * g.KW > kDwMaxTaps) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d: more than 1024 taps");
+  const dim3 grid((unsigned)(g.N * g.C * bands)), block(256);
+  const int b = beta ? 1 : 0;
+#define LNN_DW_LAUNCH(KS)                                                                                  \
+  do {                                                                                                     \
+    if (small) hipLaunchKernelGGL((dw_fwd_kernel<KS, kDwSmall>), grid, block, 0, ctx->stream, g, X, K, Y, bands, TH, b); \
+    else hipLaunchKernelGGL((dw_fwd_kernel<KS, kDwLarge>), grid, block, 0, ctx->stream, g, X, K, Y, bands, TH, b);       \
+  } while (0)
+  if (g.KH == g.KW && g.KH == 3) LNN_DW_LAUNCH(3);
+  else if (g.KH == g.KW && g.KH == 5) LNN_DW_LAUNCH(5);
+  else if (g.KH == g.KW && g.KH == 1) LNN_DW_LAUNCH(1);
+  else LNN_DW_LAUNCH(0);
+#undef LNN_DW_LAUNCH
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }
@@ -148,9 +284,25 @@ int launch_dw_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, c
   int st = dw_geom(d, g, "depthwise_conv2d_dgrad");
   if (st != LNN_OK) return st;
   if (!dY || !K || !dX) return set_error(LNN_ERR_INVALID, "depthwise_conv2d_dgrad: null pointer");
-  const uint32_t n = (uint32_t)((uint64_t)g.N * g.C * g.IH * g.IW);
-  hipLaunchKernelGGL(dw_dgrad_kernel, dw_grid(n, ctx->cus), dim3(256), 0, ctx->stream, g, dY, K, dX, n, beta ? 1 : 0,
-                     make_fastdiv(g.S));
+  // TH rows of dX touch at most (TH - 1 + (KH-1)*D) / S + 2 rows of dY
+  int TH = dw_band_rows(g.IH, g.OW, 1, g.S, (long long)((g.KH - 1) * g.D) / g.S + 2, kDwSmall);
+  const bool small = TH >= 8 || TH >= g.IH;
+  if (!small) TH = dw_band_rows(g.IH, g.OW, 1, g.S, (long long)((g.KH - 1) * g.D) / g.S + 2, kDwLarge);
+  if (TH < 1) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d_dgrad: image rows wider than the LDS band");
+  const int bands = (g.IH + TH - 1) / TH;
+  if (g.KH * g.KW > kDwMaxTaps) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d: more than 1024 taps");
+  const dim3 grid((unsigned)(g.N * g.C * bands)), block(256);
+  const int b = beta ? 1 : 0;
+#define LNN_DW_LAUNCH(KS)                                                                                    \
+  do {                                                                                                       \
+    if (small) hipLaunchKernelGGL((dw_dgrad_kernel<KS, kDwSmall>), grid, block, 0, ctx->stream, g, dY, K, dX, bands, TH, b); \
+    else hipLaunchKernelGGL((dw_dgrad_kernel<KS, kDwLarge>), grid, block, 0, ctx->stream, g, dY, K, dX, bands, TH, b);       \
+  } while (0)
+  if (g.KH == g.KW && g.KH == 3) LNN_DW_LAUNCH(3);
+  else if (g.KH == g.KW && g.KH == 5) LNN_DW_LAUNCH(5);
+  else if (g.KH == g.KW && g.KH == 1) LNN_DW_LAUNCH(1);
+  else LNN_DW_LAUNCH(0);
+#undef LNN_DW_LAUNCH
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }
@@ -161,22 +313,36 @@ int launch_dw_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   if (st != LNN_OK) return st;
   if (!X || !dY || !dK) return set_error(LNN_ERR_INVALID, "depthwise_conv2d_wgrad: null pointer");
   const int KK = g.KH * g.KW;
-  const uint64_t P = (uint64_t)g.N * g.OH * g.OW;
-  // enough blocks to fill the chip a few times over, each with at least a few thousand pixels
-  long long splits = ((long long)ctx->cus * 8 + g.C - 1) / g.C;
-  if (splits > (long long)((P + 2047) / 2048)) splits = (long long)((P + 2047) / 2048);
-  if (splits < 1) splits = 1;
-  if (splits > 65535) splits = 65535;
-  if (g.C > 0x7fffffff / KK) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d_wgrad: kernel tensor too large");
-  st = ensure_workspace(ctx, (size_t)g.C * splits * KK * sizeof(float));
+  auto rows = [&](int floats) {
+    int th = dw_band_rows(g.OH, g.IW, g.S, 1, (long long)(g.KH - 1) * g.D, floats);
+    while (th >= 1 && (long long)th * g.OW > floats / 2) --th;
+    return th;
+  };
+  int TH = rows(kDwSmall);
+  const bool small = TH >= 8 || TH >= g.OH;
+  if (!small) TH = rows(kDwLarge * 2 / 3);   // X rows and half as many floats of dY rows share the 160 KB
+  if (TH < 1) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d_wgrad: image rows wider than the LDS band");
+  const int bands = (g.OH + TH - 1) / TH;
+  const size_t need = (size_t)g.N * g.C * bands * KK * sizeof(float);
+  if (need > kMaxTensorBytes) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d_wgrad: partial sums of 2 GiB or more");
+  st = ensure_workspace(ctx, need);
   if (st != LNN_OK) return st;
-  g.dIH = make_fastdiv((uint32_t)(g.OH * g.OW));   // see dw_wgrad_kernel
-  hipLaunchKernelGGL(dw_wgrad_kernel, dim3(g.C, (unsigned)splits), dim3(256), 0, ctx->stream, g, X, dY,
-                     static_cast<float*>(ctx->ws), (int)splits);
+  const dim3 grid((unsigned)(g.N * g.C * bands)), block(256);
+  float* part = static_cast<float*>(ctx->ws);
+#define LNN_DW_LAUNCH(KS)                                                                                      \
+  do {                                                                                                         \
+    if (small) hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwSmall>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
+    else hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwLarge * 2 / 3>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
+  } while (0)
+  if (g.KH == g.KW && g.KH == 3) LNN_DW_LAUNCH(3);
+  else if (g.KH == g.KW && g.KH == 5) LNN_DW_LAUNCH(5);
+  else if (g.KH == g.KW && g.KH == 1) LNN_DW_LAUNCH(1);
+  else LNN_DW_LAUNCH(0);
+#undef LNN_DW_LAUNCH
   LNN_HIP(hipGetLastError());
   const int n = g.C * KK;
   hipLaunchKernelGGL(dw_wgrad_finish_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, dK,
-                     static_cast<const float*>(ctx->ws), n, KK, (int)splits, beta ? 1 : 0);
+                     static_cast<const float*>(ctx->ws), g.C, KK, g.N, bands, beta ? 1 : 0);
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }

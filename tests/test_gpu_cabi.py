@@ -343,8 +343,12 @@ def test_depthwise_integer_exact_and_float(hip):
     thousands of products per tap)."""
     rs = np.random.RandomState(51)
     cnt = 0
-    for s, d, ks, padding, xs in itertools.product((1, 2, 3), (1, 2), (1, 2, 3, 5), ('same', 'valid', 1, (2, 0, 1, 3)),
-                                                   ((2, 3, 11, 9), (1, 70, 6, 7))):
+    grid = list(itertools.product((1, 2, 3), (1, 2), (1, 2, 3, 5), ('same', 'valid', 1, (2, 0, 1, 3)),
+                                  ((2, 3, 11, 9), (1, 70, 6, 7))))
+    # rows too wide for the small LDS band (the one-block-per-CU variant), and a 7x7 filter
+    grid += [(1, 1, 3, 'same', (1, 2, 12, 1500)), (2, 1, 5, 'same', (1, 2, 9, 2100)), (1, 2, 7, 'same', (2, 3, 20, 20)),
+             (2, 1, 7, 3, (1, 2, 30, 700))]
+    for s, d, ks, padding, xs in grid:
         try:
             ci = info_conv2d(xs[2], xs[3], ks, ks, s, d, padding)
         except ValueError:
