@@ -170,6 +170,10 @@ int lnn_reduce_sum_bwd_f32(int dev, int rank, const int32_t* shape, uint32_t red
 /* SGD.py:42-74: acc = momentum*acc - lr*g;  v += nesterov ? momentum*acc - lr*g : acc */
 int lnn_sgd_update_f32(int dev, uint64_t n, float* v, const float* g, float* acc, float momentum,
                        float lr, int nesterov);
+/* Adam step as the reference writes it (optimizer/Adam.py:43-72, three kernels there, no bias correction):
+ *   m = beta1*m + (1-beta1)*g;  v = beta2*v + (1-beta2)*g*g;  t += -lr*m / (sqrt(v) + 1e-7) */
+int lnn_adam_update_f32(int dev, uint64_t n, float* t, const float* g, float* m, float* v,
+                        float beta1, float beta2, float lr);
 
 #ifdef __cplusplus
 }

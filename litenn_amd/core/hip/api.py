@@ -77,6 +77,7 @@ SIGNATURES = {
     'lnn_reduce_sum_f32': [_c_int, _c_int, _i32arr, _c_u32, _c_f32, _ptr, _ptr, _c_int],
     'lnn_reduce_sum_bwd_f32': [_c_int, _c_int, _i32arr, _c_u32, _c_f32, _ptr, _ptr],
     'lnn_sgd_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int],
+    'lnn_adam_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32],
 }
 
 
@@ -269,3 +270,7 @@ def reduce_sum_bwd(dev, shape, axes, scale, dout, din):
 
 def sgd_update(dev, n, v, g, acc, momentum, lr, nesterov):
     check(lib.lnn_sgd_update_f32(dev, n, v, g, acc, float(momentum), float(lr), int(bool(nesterov))))
+
+
+def adam_update(dev, n, t, g, m, v, beta1, beta2, lr):
+    check(lib.lnn_adam_update_f32(dev, int(n), t, g, m, v, float(beta1), float(beta2), float(lr)))

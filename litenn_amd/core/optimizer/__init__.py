@@ -1,8 +1,9 @@
-"""Optimizers (nn.optimizer.*).  Only SGD is on this package's path."""
+"""Optimizers (nn.optimizer.*): SGD and Adam."""
 import litenn_amd as nn
 
 from .Optimizer import Optimizer
 from .SGD import SGD
+from .Adam import Adam
 
 
 class freeze:

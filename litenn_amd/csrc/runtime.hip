@@ -16,6 +16,7 @@ int launch_transpose(DeviceCtx*, int, const int32_t*, const int32_t*, const floa
 int launch_unfold2d(DeviceCtx*, int, int, int, int, int, int, int, int, int, int, int, int, int, int, const float*,
                     float*, int);
 int launch_sgd(DeviceCtx*, uint64_t, float*, const float*, float*, float, float, int);
+int launch_adam(DeviceCtx*, uint64_t, float*, const float*, float*, float*, float, float, float);
 
 static thread_local std::string g_error;
 constexpr int kMaxDevices = 64;
@@ -374,6 +375,12 @@ int lnn_sgd_update_f32(int dev, uint64_t n, float* v, const float* g, float* acc
   if (n && (!v || !g || !acc)) return set_error(LNN_ERR_INVALID, "sgd_update: null pointer");
   CTX(dev);
   return launch_sgd(ctx, n, v, g, acc, momentum, lr, nesterov);
+}
+
+int lnn_adam_update_f32(int dev, uint64_t n, float* t, const float* g, float* m, float* v, float beta1, float beta2,
+                        float lr) {
+  CTX(dev);
+  return launch_adam(ctx, n, t, g, m, v, beta1, beta2, lr);
 }
 
 }  // extern "C"

@@ -208,6 +208,19 @@ __global__ void sgd_kernel(uint64_t n, float* v, const float* g, float* acc, flo
   }
 }
 
+// m = b1*m + (1-b1)*g;  v2 = b2*v2 + (1-b2)*g*g;  t -= lr*m / (sqrt(v2) + 1e-7)   (no bias correction)
+__global__ void adam_kernel(uint64_t n, float* t, const float* g, float* m, float* v2, float beta1, float beta2,
+                            float lr) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const float gi = g[i];
+    const float mi = beta1 * m[i] + (1.0f - beta1) * gi;
+    const float vi = beta2 * v2[i] + (1.0f - beta2) * gi * gi;
+    m[i] = mi;
+    v2[i] = vi;
+    t[i] += -lr * mi / (sqrtf(vi) + 1e-7f);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host launchers (called from the C ABI)
 // ---------------------------------------------------------------------------
@@ -385,6 +398,15 @@ int launch_sgd(DeviceCtx* ctx, uint64_t n, float* v, const float* g, float* acc,
   if (n == 0) return LNN_OK;
   hipLaunchKernelGGL(sgd_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, n, v, g, acc, momentum, lr,
                      nesterov ? 1 : 0);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+int launch_adam(DeviceCtx* ctx, uint64_t n, float* t, const float* g, float* m, float* v2, float beta1, float beta2,
+                float lr) {
+  if (n == 0) return LNN_OK;
+  if (!t || !g || !m || !v2) return set_error(LNN_ERR_INVALID, "adam_update: null pointer");
+  hipLaunchKernelGGL(adam_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, n, t, g, m, v2, beta1, beta2, lr);
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }

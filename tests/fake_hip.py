@@ -13,7 +13,7 @@ from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
          'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
-         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update']
+         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update']
 
 
 class FakeHip:
@@ -184,6 +184,14 @@ class FakeHip:
         a = (np.float32(momentum) * A - np.float32(lr) * G).astype(np.float32)
         A[:] = a
         V[:] = V + ((np.float32(momentum) * a - np.float32(lr) * G) if nesterov else a)
+
+    def adam_update(self, dev, n, t, g, m, v, beta1, beta2, lr):
+        self.launches += 1
+        T, G, M, V = self.f(t)[:n], self.f(g)[:n], self.f(m)[:n], self.f(v)[:n]
+        b1, b2 = np.float32(beta1), np.float32(beta2)
+        M[:] = b1 * M + (np.float32(1) - b1) * G
+        V[:] = b2 * V + (np.float32(1) - b2) * G * G
+        T[:] = T - np.float32(lr) * M / (np.sqrt(V) + np.float32(1e-7))
 
 
 def install(monkeypatch, capacity=None):

@@ -401,6 +401,26 @@ def test_sgd_closed_form(nn_backend):
         nn.optimizer.SGD([nn.Tensor((4,))], lr_dropout=0.7)
 
 
+def test_adam_closed_form(nn_backend):
+    """Adam.py:43-72 in float64: m and v without bias correction, t += -lr*m/(sqrt(v)+1e-7)."""
+    nn = nn_backend
+    for b1, b2, decay in [(0.9, 0.999, 0.0), (0.5, 0.9, 0.1)]:
+        w0 = np.linspace(-1, 1, 37).astype(np.float32)
+        w_t = nn.Tensor_from_value(w0)
+        opt = nn.optimizer.Adam([w_t], beta_1=b1, beta_2=b2, lr=0.01, lr_decay=decay)
+        w, m, v = w0.astype(np.float64), np.zeros(37), np.zeros(37)
+        for it in range(4):
+            g = np.linspace(1 + it, 2, 37).astype(np.float32) * (-1) ** it
+            w_t.get_grad().set(g)
+            opt.step()
+            lr = 0.01 / (1.0 + decay * it)
+            m = b1 * m + (1 - b1) * g
+            v = b2 * v + (1 - b2) * g.astype(np.float64) ** 2
+            w = w - lr * m / (np.sqrt(v) + 1e-7)
+        np.testing.assert_allclose(w_t.np(), w, rtol=2e-5, atol=1e-6)
+        w_t._set_trainable(False)
+
+
 def test_pointwise_broadcast_and_reduce(nn_backend):
     nn = nn_backend
     rs = np.random.RandomState(5)
