@@ -641,9 +641,11 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   a.bytesOut = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
   a.M = g.O; a.Ncols = g.N * g.OHW; a.K = g.C * g.KK;
   a.beta = beta ? 1 : 0;
-  if (g.C % BK == 0) {
-    st = permuted_weights(ctx, g, W, 0, PixelClass{}, &a.W, &a.ws_used);
-    if (st != LNN_OK) return st;
+  if (g.C % BK == 0 && (g.KK > 1 || aligned16(W))) {
+    if (g.KK > 1) {   // a 1x1 kernel already is [O][tap][C]
+      st = permuted_weights(ctx, g, W, 0, PixelClass{}, &a.W, &a.ws_used);
+      if (st != LNN_OK) return st;
+    }
     return launch_by_m<PASS_FWD_TAP>(ctx, a, true);
   }
   st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);
@@ -664,7 +666,8 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   // one stride-1 problem per class of input pixels (see ConvDgradB)
   std::vector<ConvArgs> cls;
   std::vector<PixelClass> pcs;
-  size_t w_bytes = 0;   // permuted weights of all classes, back to back
+  std::vector<size_t> w_off;   // where each class's permuted weights start in the scratch buffer
+  size_t w_bytes = 0;          // permuted weights of all classes, back to back
   for (int rh = 0; rh < S; ++rh)
     for (int rw = 0; rw < S; ++rw) {
       PixelClass pc;
@@ -698,7 +701,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
       st = get_table(ctx, full, tap ? 2 : 1, pc, &a.tab);
       if (st != LNN_OK) return st;
       if (tap) {
-        a.ws_used = w_bytes;   // here: offset of this class's permuted weights in the scratch buffer
+        w_off.push_back(w_bytes);
         w_bytes += ((size_t)(a.bytesW ? a.bytesW : 4) + 255) & ~(size_t)255;
       }
       cls.push_back(a);
@@ -734,7 +737,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   if (tap)
     for (int i = 0; i < nc; ++i) {
       ConvArgs& a = cls[i];
-      float* wp = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + a.ws_used);
+      float* wp = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + w_off[i]);
       const int n = full.O * full.C * pcs[i].nkh * pcs[i].nkw;
       if (n > 0) {
         hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, wp, W, full.O, full.C,
