@@ -13,7 +13,7 @@ CPU restatement of the reference algorithm timed on the host cores.
 
 --all additionally measures every benchmark configuration (conv geometries,
 the 4096^3 matmul with both gradients, the 4-layer encoder training step) and
-writes one JSON object per line to gpurun_out/bench_all.jsonl.
+writes one JSON object per line to bench_all.jsonl in --out-dir (default: the current directory).
 """
 import argparse
 import json
@@ -457,6 +457,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--all', action='store_true', help='also measure every benchmark configuration')
+    ap.add_argument('--out-dir', default='.', help='where --all writes bench_all.jsonl')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='run only a plain device copy of 256 MiB (three launches of the element-wise kernel) and exit: '
                          'the reference reading for the FETCH_SIZE / WRITE_SIZE counters')
@@ -479,8 +480,8 @@ def main():
                                                'write_bytes': 4 * n}}), flush=True)
         return
     if args.all:
-        os.makedirs(os.path.join(ROOT, 'gpurun_out'), exist_ok=True)
-        with open(os.path.join(ROOT, 'gpurun_out', 'bench_all.jsonl'), 'w') as f:
+        os.makedirs(args.out_dir, exist_ok=True)
+        with open(os.path.join(args.out_dir, 'bench_all.jsonl'), 'w') as f:
             for name in CONV_CONFIGS:
                 if name == 'cfg3_vgg3x3':
                     continue
@@ -513,7 +514,7 @@ def main():
     else:
         res = bench_conv(api, args.config, args.steps, args.warmup, cpu=not args.no_cpu)
     if args.all:
-        with open(os.path.join(ROOT, 'gpurun_out', 'bench_all.jsonl'), 'a') as f:
+        with open(os.path.join(args.out_dir, 'bench_all.jsonl'), 'a') as f:
             f.write(json.dumps(res) + '\n')
     print(json.dumps(res), flush=True)
 
