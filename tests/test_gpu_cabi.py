@@ -473,3 +473,64 @@ def test_transpose_exact(hip):
             out = DevArr(hip, shape=tuple(shape[a] for a in axes), fill=1.0)
             hip.transpose(0, shape, axes, V.ptr, out.ptr, 1)
             assert np.array_equal(out.get() - 1.0, v.transpose(axes))
+
+
+# ------------------------------------------------------------------ full-size properties
+def _dot(a, b):
+    return float(np.dot(a.astype(np.float64).ravel(), b.astype(np.float64).ravel()))
+
+
+@pytest.mark.parametrize('xs,ws,s,d,padding', [((32, 128, 56, 56), (128, 128, 3, 3), 1, 1, 'same'),
+                                               ((64, 256, 28, 28), (512, 256, 1, 1), 1, 1, 'valid'),
+                                               ((16, 128, 32, 32), (256, 128, 5, 5), 2, 1, 2)])
+def test_conv_full_size_adjoint_and_linearity(hip, xs, ws, s, d, padding):
+    """At the benchmark sizes the oracle is too slow to run, but the three
+    passes are tied together by identities that hold for any size:
+      <conv(X, W), dY> = <X, dgrad(dY, W)> = <W, wgrad(X, dY)>        (adjoints)
+      conv(X, W1 + W2) = conv(X, W1) + conv(X, W2)                    (linearity)
+    and a dropped tap, a transposed operand or a wrong pad would break them.
+    Sums are taken in fp64 on the host; tolerance 1e-5 of the magnitude sum."""
+    rs = np.random.RandomState(77)
+    desc, ci = _desc(hip, xs, ws, s, d, padding)
+    x = rs.uniform(-1, 1, xs).astype(np.float32)
+    w = rs.normal(0, 0.05, ws).astype(np.float32)
+    w2 = rs.normal(0, 0.05, ws).astype(np.float32)
+    dy = rs.normal(0, 1, (xs[0], ws[0], ci.OH, ci.OW)).astype(np.float32)
+    say(f'full-size identities x={xs} w={ws}')
+    X, W, W2, dY = DevArr(hip, x), DevArr(hip, w), DevArr(hip, w2), DevArr(hip, dy)
+    Y, Y2, Y12 = (DevArr(hip, shape=dy.shape, fill=np.nan) for _ in range(3))
+    dX, dW = DevArr(hip, shape=xs, fill=np.nan), DevArr(hip, shape=ws, fill=np.nan)
+    hip.conv2d_fwd(0, desc, X.ptr, W.ptr, Y.ptr, 0)
+    hip.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, 0)
+    hip.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW.ptr, 0)
+    y, dx, dw = Y.get(), dX.get(), dW.get()
+    a, b, c = _dot(y, dy), _dot(x, dx), _dot(w, dw)
+    scale = float(np.dot(np.abs(y).astype(np.float64).ravel(), np.abs(dy).astype(np.float64).ravel()))
+    assert abs(a - b) <= 1e-5 * scale and abs(a - c) <= 1e-5 * scale, (a, b, c, scale)
+    W12 = DevArr(hip, w + w2)
+    hip.conv2d_fwd(0, desc, X.ptr, W2.ptr, Y2.ptr, 0)
+    hip.conv2d_fwd(0, desc, X.ptr, W12.ptr, Y12.ptr, 0)
+    assert rel_err(Y12.get(), y.astype(np.float64) + Y2.get()) <= 1e-5
+    # accumulation: a second '+=' pass doubles a gradient exactly
+    hip.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW.ptr, 1)
+    assert np.array_equal(dW.get(), dw + dw)
+
+
+def test_gemm_full_size_adjoints(hip):
+    """<A.B, dC> = <A, dC.B^T> = <B, A^T.dC> at 4096^3."""
+    rs = np.random.RandomState(78)
+    n = 4096
+    a, b, dc = (rs.normal(0, 1, (n, n)).astype(np.float32) for _ in range(3))
+    A, B, D = DevArr(hip, a), DevArr(hip, b), DevArr(hip, dc)
+    C, dA, dB = (DevArr(hip, shape=(n, n), fill=np.nan) for _ in range(3))
+    say('gemm 4096^3 adjoint identities')
+    hip.gemm(0, 0, 0, 1, n, n, n, A.ptr, n, 0, B.ptr, n, 0, C.ptr, n, 0, 0)
+    hip.gemm(0, 0, 1, 1, n, n, n, D.ptr, n, 0, B.ptr, n, 0, dA.ptr, n, 0, 0)
+    hip.gemm(0, 1, 0, 1, n, n, n, A.ptr, n, 0, D.ptr, n, 0, dB.ptr, n, 0, 0)
+    c = C.get()
+    x, y, z = _dot(c, dc), _dot(a, dA.get()), _dot(b, dB.get())
+    scale = float(np.dot(np.abs(c).astype(np.float64).ravel(), np.abs(dc).astype(np.float64).ravel()))
+    assert abs(x - y) <= 1e-5 * scale and abs(x - z) <= 1e-5 * scale, (x, y, z, scale)
+    rows = np.arange(0, n, 511)
+    assert rel_err(c[rows], a[rows].astype(np.float64) @ b.astype(np.float64)) <= TOL
+
