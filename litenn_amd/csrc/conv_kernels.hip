@@ -516,9 +516,12 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     int ksplit = (int)s;
     grid_y = ksplit;
     if (PASS == PASS_WGRAD_TAP) {
-      // the last chunk holds rem <= chunk units: give it that share of the slices
+      // the last chunk holds rem <= chunk units: give it the matching share of the slices.  A K step of u
+      // units costs about (o + u) with a fixed part o worth an eighth of a full chunk (measured: a half
+      // chunk's step takes 0.56 of a full one), so that is the ratio of the slice counts.
       const int rem = (int)(total - (long long)(grid - 1) * chunk);
-      auto last = [&](int sf) { const int l = (sf * rem + chunk - 1) / chunk; return l < 1 ? 1 : l; };
+      const int o = chunk >= 8 ? chunk / 8 : 1;
+      auto last = [&](int sf) { const int l = (sf * (o + rem) + o + chunk - 1) / (o + chunk); return l < 1 ? 1 : (l > sf ? sf : l); };
       while (ksplit > 1 && (long long)(grid - 1) * ksplit + last(ksplit) > slots) --ksplit;
       a.n_chunks = grid;
       a.ks_last = last(ksplit);
