@@ -33,7 +33,7 @@ PEAK_HBM_GBS = 8000.0
 # copy of known size), measured separately under rocprofv3 --pmc; keyed by workload and pass.  A pass that has
 # not been measured reports null.
 MEASURED_TRAFFIC_BYTES = {
-    'cfg3_vgg3x3': {'fwd': 316.1e6, 'dX': 385.1e6, 'dW': 236.6e6 + 33.6e6},   # dW = wgrad kernel + slice reduction
+    'cfg3_vgg3x3': {'fwd': 340.0e6, 'dX': 360.9e6, 'dW': 236.4e6 + 40.5e6},   # dW = wgrad kernel + slice reduction
 }
 
 CONV_CONFIGS = {
