@@ -1077,8 +1077,10 @@ __device__ __forceinline__ void load_frags(const float* __restrict__ As, const f
   } else {   // two [BK][RA/2] slabs
     constexpr int H = RA / 2;
     const int r = arow + i;
+    // one address per lane, the four k as immediate offsets (they pair into two-dword reads)
+    const float* ap = As + ((r / H) * (BK * H) + r % H + h * (4 * H)) + kk * (8 * H);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) a[t] = As[(r / H) * (BK * H) + (kb + t) * H + r % H];
+    for (int t = 0; t < 4; ++t) a[t] = ap[t * H];
   }
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
