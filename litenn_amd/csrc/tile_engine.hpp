@@ -1072,8 +1072,9 @@ __device__ __forceinline__ void load_frags(const float* __restrict__ As, const f
     const f32x4 t = *reinterpret_cast<const f32x4*>(LAY_A == LAY_KC ? &As[(arow + i) * LDK + kb] : &As[(arow + i) * BK + sw]);
     a[0] = t[0]; a[1] = t[1]; a[2] = t[2]; a[3] = t[3];
   } else if (LAY_A == LAY_MC) {
+    const float* ap = As + (arow + i + h * (4 * RA));   // one address per lane, k as immediate offsets
 #pragma unroll
-    for (int t = 0; t < 4; ++t) a[t] = As[(kb + t) * RA + arow + i];
+    for (int t = 0; t < 4; ++t) a[t] = ap[(kk * 8 + t) * RA];
   } else {   // two [BK][RA/2] slabs
     constexpr int H = RA / 2;
     const int r = arow + i;
@@ -1089,8 +1090,11 @@ __device__ __forceinline__ void load_frags(const float* __restrict__ As, const f
       const f32x4 t = *reinterpret_cast<const f32x4*>(LAY_B == LAY_KC ? &Bs[r * LDK + kb] : &Bs[r * BK + sw]);
       b[j][0] = t[0]; b[j][1] = t[1]; b[j][2] = t[2]; b[j][3] = t[3];
     } else {   // shared tile or the group's own slab: the caller passes the matching base, pitch and brow
+      // one address per lane and accumulator tile; kk and t are immediate offsets, so with RB a multiple
+      // of 64 the four reads pair into two-dword reads without any address arithmetic in the K loop
+      const float* bp = Bs + (brow + 32 * j + i + h * (4 * RB));
 #pragma unroll
-      for (int t = 0; t < 4; ++t) b[j][t] = Bs[(kb + t) * RB + brow + 32 * j + i];
+      for (int t = 0; t < 4; ++t) b[j][t] = bp[(kk * 8 + t) * RB];
     }
   }
 }
