@@ -29,17 +29,25 @@ struct DwGeom {
 // LDSF floats of source rows per block: 4096 (16 KB, eight blocks per compute unit hide the copy latency)
 // when a useful band fits, else 32768 (128 KB, one block) for very wide rows.
 constexpr int kDwSmall = 4096, kDwLarge = 32768;
+// kernel gradient with very wide rows: X rows and dY rows share the LDS (120 KB), both multiples of 256 floats
+constexpr int kDwWgradX = 20480, kDwWgradY = 10240;
 
+// Rows row_lo..row_hi of a plane are one contiguous run of floats.  They go to LDS with global->LDS transfers,
+// which occupy no registers and are all in flight at once: one memory latency per block.  A transfer that
+// starts inside the run and ends past it deposits zeros, so the LDS array must hold the run rounded up to
+// 256 floats.  dw_copy_wait() before the block barrier.
 __device__ __forceinline__ void dw_copy_rows(float* lds, const float* __restrict__ plane, int row_lo, int row_hi, int W) {
   const int n = (row_hi - row_lo + 1) * W;
   const float* src = plane + (size_t)row_lo * W;
+  const rsrc_t rs = make_rsrc(src, (uint32_t)n * 4u);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (((reinterpret_cast<uintptr_t>(src) | (uintptr_t)(n * 4)) & 15) == 0) {   // block-uniform
-    for (int i = threadIdx.x; i < n / 4; i += 256)
-      reinterpret_cast<f32x4*>(lds)[i] = reinterpret_cast<const f32x4*>(src)[i];
+    for (int c = wave * 256; c < n; c += 1024) buf_load_lds16(rs, lds + c, (uint32_t)(c + lane * 4) * 4u, 0);
   } else {
-    for (int i = threadIdx.x; i < n; i += 256) lds[i] = src[i];
+    for (int c = wave * 64; c < n; c += 256) buf_load_lds4(rs, lds + c, (uint32_t)(c + lane) * 4u, 0);
   }
 }
+__device__ __forceinline__ void dw_copy_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // KS > 0: square KS x KS filter known at compile time (tap loops unrolled, filter in registers);
 // KS == 0: any KH x KW, filter read from LDS.
@@ -78,19 +86,58 @@ __global__ __launch_bounds__(256) void dw_fwd_kernel(DwGeom g, const float* __re
   if (hi >= lo) dw_copy_rows(lds, X + (size_t)plane * g.IH * g.IW, lo, hi, g.IW);
   DwFilter<KS> f;
   f.load(K + (size_t)c * g.KH * g.KW, ldsk, g.KH, g.KW);
+  dw_copy_wait();
   __syncthreads();
   float* yp = Y + (size_t)plane * g.OH * g.OW;
+  if (KS > 0) {
+    // A thread keeps one output column and walks down the band's rows: the column tests and offsets of the
+    // KS taps are computed once, a row costs KS row tests and KS*KS guarded multiply-adds.
+    const int ncol = g.OW < 256 ? g.OW : 256, ngrp = 256 / ncol;
+    const int tc = threadIdx.x % ncol, tg = threadIdx.x / ncol;
+    for (int ow = tc; ow < g.OW; ow += ncol) {
+      if (tg >= ngrp) break;
+      // a tap outside the image reads element 0 of the band instead and is dropped afterwards: every LDS
+      // read of a row is unconditional, so all of them are in flight together
+      int iw[KS > 0 ? KS : 1];
+      bool okw[KS > 0 ? KS : 1];
+#pragma unroll
+      for (int kw = 0; kw < KS; ++kw) {
+        const int w = ow * g.S - g.PADL + kw * g.D;
+        okw[kw] = (uint32_t)w < (uint32_t)g.IW;
+        iw[kw] = okw[kw] ? w : 0;
+      }
+      for (int oh = r0 + tg; oh < r1; oh += ngrp) {
+        const int ih0 = oh * g.S - g.PADT;
+        float x[KS > 0 ? KS * KS : 1];
+        bool okh[KS > 0 ? KS : 1];
+#pragma unroll
+        for (int kh = 0; kh < KS; ++kh) {
+          const int ih = ih0 + kh * g.D;
+          okh[kh] = (uint32_t)ih < (uint32_t)g.IH;
+          const float* row = lds + (okh[kh] ? (ih - lo) * g.IW : 0);
+#pragma unroll
+          for (int kw = 0; kw < KS; ++kw) x[kh * KS + kw] = row[iw[kw]];
+        }
+        float v = 0.0f;
+#pragma unroll
+        for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+          for (int kw = 0; kw < KS; ++kw) v += (okh[kh] && okw[kw]) ? x[kh * KS + kw] * f.at(kh, kw) : 0.0f;
+        const int o = oh * g.OW + ow;
+        yp[o] = beta ? yp[o] + v : v;
+      }
+    }
+    return;
+  }
   const int n = (r1 - r0) * g.OW;
   for (int i = threadIdx.x; i < n; i += 256) {
     const int r = (int)g.dOW.div((uint32_t)i), ow = i - r * g.OW, oh = r0 + r;
     const int ih0 = oh * g.S - g.PADT, iw0 = ow * g.S - g.PADL;
     float v = 0.0f;
-#pragma unroll
     for (int kh = 0; kh < f.KH; ++kh) {
       const int ih = ih0 + kh * g.D;
       if ((uint32_t)ih < (uint32_t)g.IH) {
         const float* row = lds + (ih - lo) * g.IW;
-#pragma unroll
         for (int kw = 0; kw < f.KW; ++kw) {
           const int iw = iw0 + kw * g.D;
           if ((uint32_t)iw < (uint32_t)g.IW) v += row[iw] * f.at(kh, kw);
@@ -101,8 +148,6 @@ __global__ __launch_bounds__(256) void dw_fwd_kernel(DwGeom g, const float* __re
     yp[o] = beta ? yp[o] + v : v;
   }
 }
-
-// data gradient: dX rows [r0, r1) of the plane from dY rows [lo, hi]
 template <int KS, int LDSF>
 __global__ __launch_bounds__(256) void dw_dgrad_kernel(DwGeom g, const float* __restrict__ dY,
                                                        const float* __restrict__ K, float* __restrict__ dX, int bands,
@@ -119,19 +164,56 @@ __global__ __launch_bounds__(256) void dw_dgrad_kernel(DwGeom g, const float* __
   __shared__ float ldsk[KS > 0 ? 1 : kDwMaxTaps];
   DwFilter<KS> f;
   f.load(K + (size_t)c * g.KH * g.KW, ldsk, g.KH, g.KW);
+  dw_copy_wait();
   __syncthreads();
   float* xp = dX + (size_t)plane * g.IH * g.IW;
+  if (KS > 0) {
+    // column walk as in the forward kernel: the output column of each tap and whether it exists are fixed per thread
+    const int ncol = g.IW < 256 ? g.IW : 256, ngrp = 256 / ncol;
+    const int tc = threadIdx.x % ncol, tg = threadIdx.x / ncol;
+    for (int iw = tc; iw < g.IW; iw += ncol) {
+      if (tg >= ngrp) break;
+      int ow[KS > 0 ? KS : 1];
+      bool okw[KS > 0 ? KS : 1];
+#pragma unroll
+      for (int kw = 0; kw < KS; ++kw) {
+        const int nw = iw + g.PADL - kw * g.D;
+        const int q = (int)g.dS.div((uint32_t)nw & 0x7fffffffu);
+        okw[kw] = nw >= 0 && q * g.S == nw && q < g.OW;
+        ow[kw] = okw[kw] ? q : 0;
+      }
+      for (int ih = r0 + tg; ih < r1; ih += ngrp) {
+        float y[KS > 0 ? KS * KS : 1];
+        bool okh[KS > 0 ? KS : 1];
+#pragma unroll
+        for (int kh = 0; kh < KS; ++kh) {
+          const int nh = ih + g.PADT - kh * g.D;
+          const int oh = (int)g.dS.div((uint32_t)nh & 0x7fffffffu);
+          okh[kh] = nh >= 0 && oh * g.S == nh && oh < g.OH;
+          const float* row = lds + (okh[kh] ? (oh - lo) * g.OW : 0);
+#pragma unroll
+          for (int kw = 0; kw < KS; ++kw) y[kh * KS + kw] = row[ow[kw]];
+        }
+        float v = 0.0f;
+#pragma unroll
+        for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+          for (int kw = 0; kw < KS; ++kw) v += (okh[kh] && okw[kw]) ? y[kh * KS + kw] * f.at(kh, kw) : 0.0f;
+        const int o = ih * g.IW + iw;
+        xp[o] = beta ? xp[o] + v : v;
+      }
+    }
+    return;
+  }
   const int n = (r1 - r0) * g.IW;
   for (int i = threadIdx.x; i < n; i += 256) {
     const int r = (int)g.dIW.div((uint32_t)i), iw = i - r * g.IW, ih = r0 + r;
     float v = 0.0f;
-#pragma unroll
     for (int kh = 0; kh < f.KH; ++kh) {
       const int nh = ih + g.PADT - kh * g.D;
       const int oh = (int)g.dS.div((uint32_t)nh & 0x7fffffffu);
       if (nh >= 0 && oh * g.S == nh && oh < g.OH) {
         const float* row = lds + (oh - lo) * g.OW;
-#pragma unroll
         for (int kw = 0; kw < f.KW; ++kw) {
           const int nw = iw + g.PADL - kw * g.D;
           const int ow = (int)g.dS.div((uint32_t)nw & 0x7fffffffu);
@@ -146,12 +228,12 @@ __global__ __launch_bounds__(256) void dw_dgrad_kernel(DwGeom g, const float* __
 
 // kernel gradient: block (plane, band) holds dY rows [r0, r1) and the X rows under them and writes, per tap,
 // the sum of X * dY over the band to part[(plane*bands + band)*KK + tap]
-template <int KS, int LDSF>
+template <int KS, int LDSF, int LDSY>
 __global__ __launch_bounds__(256) void dw_wgrad_kernel(DwGeom g, const float* __restrict__ X,
                                                        const float* __restrict__ dY, float* __restrict__ part,
                                                        int bands, int TH) {
   __shared__ __attribute__((aligned(16))) float ldsx[LDSF];
-  __shared__ __attribute__((aligned(16))) float ldsy[LDSF / 2];
+  __shared__ __attribute__((aligned(16))) float ldsy[LDSY];
   __shared__ float red[4];
   const int plane = blockIdx.x / bands, band = blockIdx.x - plane * bands;
   const int r0 = band * TH, r1 = r0 + TH < g.OH ? r0 + TH : g.OH;
@@ -160,6 +242,7 @@ __global__ __launch_bounds__(256) void dw_wgrad_kernel(DwGeom g, const float* __
   hi = hi >= g.IH ? g.IH - 1 : hi;
   if (hi >= lo) dw_copy_rows(ldsx, X + (size_t)plane * g.IH * g.IW, lo, hi, g.IW);
   dw_copy_rows(ldsy, dY + (size_t)plane * g.OH * g.OW, r0, r1 - 1, g.OW);
+  dw_copy_wait();
   __syncthreads();
   const int n = (r1 - r0) * g.OW, KK = g.KH * g.KW;
   float* out = part + ((size_t)plane * bands + band) * KK;
@@ -169,29 +252,50 @@ __global__ __launch_bounds__(256) void dw_wgrad_kernel(DwGeom g, const float* __
     float acc[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) {
-      const int r = (int)g.dOW.div((uint32_t)i), ow = i - r * g.OW;
-      const int ih0 = (r0 + r) * g.S - g.PADT, iw0 = ow * g.S - g.PADL;
-      const float dyv = ldsy[i];
+    const int ncol = g.OW < 256 ? g.OW : 256, ngrp = 256 / ncol;
+    const int tc = threadIdx.x % ncol, tg = threadIdx.x / ncol;
+    for (int ow = tc; ow < g.OW; ow += ncol) {
+      if (tg >= ngrp) break;
+      int iw[T];
+      bool okw[T];
 #pragma unroll
-      for (int kh = 0; kh < KS; ++kh) {
-        const int ih = ih0 + kh * g.D;
-        const float* row = ldsx + (ih - lo) * g.IW;
+      for (int kw = 0; kw < KS; ++kw) {
+        const int w = ow * g.S - g.PADL + kw * g.D;
+        okw[kw] = (uint32_t)w < (uint32_t)g.IW;
+        iw[kw] = okw[kw] ? w : 0;
+      }
+      for (int r = tg; r < r1 - r0; r += ngrp) {
+        const int ih0 = (r0 + r) * g.S - g.PADT;
+        const float dyv = ldsy[r * g.OW + ow];
+        float x[T];
+        bool okh[T];
 #pragma unroll
-        for (int kw = 0; kw < KS; ++kw) {
-          const int iw = iw0 + kw * g.D;
-          const bool ok = (uint32_t)ih < (uint32_t)g.IH && (uint32_t)iw < (uint32_t)g.IW;
-          acc[kh * KS + kw] += ok ? row[iw] * dyv : 0.0f;
+        for (int kh = 0; kh < KS; ++kh) {
+          const int ih = ih0 + kh * g.D;
+          okh[kh] = (uint32_t)ih < (uint32_t)g.IH;
+          const float* row = ldsx + (okh[kh] ? (ih - lo) * g.IW : 0);
+#pragma unroll
+          for (int kw = 0; kw < KS; ++kw) x[kh * KS + kw] = row[iw[kw]];
         }
+#pragma unroll
+        for (int kh = 0; kh < KS; ++kh)
+#pragma unroll
+          for (int kw = 0; kw < KS; ++kw) acc[kh * KS + kw] += (okh[kh] && okw[kw]) ? x[kh * KS + kw] * dyv : 0.0f;
       }
     }
+    // wavefront butterflies of all taps side by side (their exchanges overlap), then the four wavefront sums
     __shared__ float red2[4][T];
 #pragma unroll
-    for (int t = 0; t < T; ++t) {
-      float v = acc[t];
+    for (int o = 32; o > 0; o >>= 1) {
+      float got[T];
 #pragma unroll
-      for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-      if ((threadIdx.x & 63) == 0) red2[threadIdx.x >> 6][t] = v;
+      for (int t = 0; t < T; ++t) got[t] = __shfl_xor(acc[t], o, 64);
+#pragma unroll
+      for (int t = 0; t < T; ++t) acc[t] += got[t];
+    }
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+      for (int t = 0; t < T; ++t) red2[threadIdx.x >> 6][t] = acc[t];
     }
     __syncthreads();
     if (threadIdx.x < T) out[threadIdx.x] = (red2[0][threadIdx.x] + red2[1][threadIdx.x]) + (red2[2][threadIdx.x] + red2[3][threadIdx.x]);
@@ -215,16 +319,31 @@ __global__ __launch_bounds__(256) void dw_wgrad_kernel(DwGeom g, const float* __
   }
 }
 
-// dK[c][tap] (+)= sum over images and bands, in a fixed order
-__global__ void dw_wgrad_finish_kernel(float* __restrict__ dK, const float* __restrict__ part, int C, int KK, int N,
-                                       int bands, int beta) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;   // i = c*KK + tap
-  if (i >= C * KK) return;
-  const int c = i / KK, tap = i - c * KK;
-  float v = 0.0f;
-  for (int n = 0; n < N; ++n)
-    for (int b = 0; b < bands; ++b) v += part[(((size_t)n * C + c) * bands + b) * KK + tap];
-  dK[i] = beta ? dK[i] + v : v;
+// dK[c][tap] (+)= sum over images and bands, in a fixed order.  One block per channel: thread (j, tap) adds every
+// J-th (image, band) entry of its tap, then the J running sums of a tap are added in ascending j.
+__global__ __launch_bounds__(256) void dw_wgrad_finish_kernel(float* __restrict__ dK, const float* __restrict__ part,
+                                                              int C, int KK, int N, int bands, int beta) {
+  __shared__ float red[256];
+  const int c = blockIdx.x, E = N * bands;
+  for (int t0 = 0; t0 < KK; t0 += 256) {
+    const int tl = KK - t0 < 256 ? KK - t0 : 256, J = 256 / tl;
+    const int j = threadIdx.x / tl, tap = t0 + threadIdx.x - j * tl;
+    float v = 0.0f;
+    if (j < J)
+      for (int e = j; e < E; e += J) {
+        const int n = e / bands, b = e - n * bands;
+        v += part[(((size_t)n * C + c) * bands + b) * KK + tap];
+      }
+    red[threadIdx.x] = v;
+    __syncthreads();
+    if (threadIdx.x < tl) {
+      float s = 0.0f;
+      for (int q = 0; q < J; ++q) s += red[q * tl + threadIdx.x];
+      float* o = dK + (size_t)c * KK + tap;
+      *o = beta ? *o + s : s;
+    }
+    __syncthreads();
+  }
 }
 
 static int dw_geom(const lnn_conv2d_desc* d, DwGeom& g, const char* who) {
@@ -313,14 +432,14 @@ int launch_dw_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   if (st != LNN_OK) return st;
   if (!X || !dY || !dK) return set_error(LNN_ERR_INVALID, "depthwise_conv2d_wgrad: null pointer");
   const int KK = g.KH * g.KW;
-  auto rows = [&](int floats) {
-    int th = dw_band_rows(g.OH, g.IW, g.S, 1, (long long)(g.KH - 1) * g.D, floats);
-    while (th >= 1 && (long long)th * g.OW > floats / 2) --th;
+  auto rows = [&](int xfloats, int yfloats) {
+    int th = dw_band_rows(g.OH, g.IW, g.S, 1, (long long)(g.KH - 1) * g.D, xfloats);
+    while (th >= 1 && (long long)th * g.OW > yfloats) --th;
     return th;
   };
-  int TH = rows(kDwSmall);
+  int TH = rows(kDwSmall, kDwSmall);
   const bool small = TH >= 8 || TH >= g.OH;
-  if (!small) TH = rows(kDwLarge * 2 / 3);   // X rows and half as many floats of dY rows share the 160 KB
+  if (!small) TH = rows(kDwWgradX, kDwWgradY);
   if (TH < 1) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d_wgrad: image rows wider than the LDS band");
   const int bands = (g.OH + TH - 1) / TH;
   const size_t need = (size_t)g.N * g.C * bands * KK * sizeof(float);
@@ -331,8 +450,8 @@ int launch_dw_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   float* part = static_cast<float*>(ctx->ws);
 #define LNN_DW_LAUNCH(KS)                                                                                      \
   do {                                                                                                         \
-    if (small) hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwSmall>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
-    else hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwLarge * 2 / 3>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
+    if (small) hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwSmall, kDwSmall>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
+    else hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwWgradX, kDwWgradY>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
   } while (0)
   if (g.KH == g.KW && g.KH == 3) LNN_DW_LAUNCH(3);
   else if (g.KH == g.KW && g.KH == 5) LNN_DW_LAUNCH(5);
@@ -340,8 +459,7 @@ int launch_dw_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   else LNN_DW_LAUNCH(0);
 #undef LNN_DW_LAUNCH
   LNN_HIP(hipGetLastError());
-  const int n = g.C * KK;
-  hipLaunchKernelGGL(dw_wgrad_finish_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, dK,
+  hipLaunchKernelGGL(dw_wgrad_finish_kernel, dim3((unsigned)g.C), dim3(256), 0, ctx->stream, dK,
                      static_cast<const float*>(ctx->ws), g.C, KK, g.N, bands, beta ? 1 : 0);
   LNN_HIP(hipGetLastError());
   return LNN_OK;
