@@ -175,6 +175,15 @@ int lnn_sgd_update_f32(int dev, uint64_t n, float* v, const float* g, float* acc
 int lnn_adam_update_f32(int dev, uint64_t n, float* t, const float* g, float* m, float* v,
                         float beta1, float beta2, float lr);
 
+/* On-device random initialisers: element i is drawn from a counter hash of (uint32)(i + seed), so a tensor
+ * is filled in place without host staging (initializer/RandomUniform.py:13-27, RandomNormal.py:10-30; the PCG
+ * hashes of CLKernelHelper.py:210-228).  The reference draws seed = np.random.randint(2^31) on the host.
+ *   uniform: out[i] = u*(high-low) + low,           u = (float)hash(i+seed) * 2^-32   (can equal high)
+ *   normal : out[i] = mean + stddev * sqrt(-2 ln u0) * cos(2 pi u1),  (u0,u1) = 2-D hash of (i+seed, 1) * 2^-32
+ * He / Glorot initialisers are these two with derived bounds (initializer/He.py:18-33, Glorot.py:20-35). */
+int lnn_random_uniform_f32(int dev, float* out, uint64_t n, uint32_t seed, double low, double high);
+int lnn_random_normal_f32(int dev, float* out, uint64_t n, uint32_t seed, double mean, double stddev);
+
 #ifdef __cplusplus
 }
 #endif

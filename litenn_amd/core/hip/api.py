@@ -39,6 +39,7 @@ class ConvDesc(ctypes.Structure):
 
 
 _c_int, _c_u32, _c_u64, _c_i64, _c_f32 = ctypes.c_int, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int64, ctypes.c_float
+_c_f64 = ctypes.c_double
 _ptr = ctypes.c_void_p
 _i32arr = ctypes.POINTER(ctypes.c_int32)
 
@@ -78,6 +79,8 @@ SIGNATURES = {
     'lnn_reduce_sum_bwd_f32': [_c_int, _c_int, _i32arr, _c_u32, _c_f32, _ptr, _ptr],
     'lnn_sgd_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int],
     'lnn_adam_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32],
+    'lnn_random_uniform_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
+    'lnn_random_normal_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
 }
 
 
@@ -274,3 +277,11 @@ def sgd_update(dev, n, v, g, acc, momentum, lr, nesterov):
 
 def adam_update(dev, n, t, g, m, v, beta1, beta2, lr):
     check(lib.lnn_adam_update_f32(dev, int(n), t, g, m, v, float(beta1), float(beta2), float(lr)))
+
+
+def random_uniform(dev, out, n, seed, low, high):
+    check(lib.lnn_random_uniform_f32(dev, out, int(n), int(seed), float(low), float(high)))
+
+
+def random_normal(dev, out, n, seed, mean, stddev):
+    check(lib.lnn_random_normal_f32(dev, out, int(n), int(seed), float(mean), float(stddev)))

@@ -2,15 +2,16 @@
 
 Scalar and NumpyArray are the ones the conv2D / matmul path needs
 (initializer/Scalar.py:5-20, NumpyArray.py:5-21).  The random initialisers
-draw on the HOST with numpy and upload the result; the reference instead runs
-a hash-based generator on the device (initializer/RandomNormal.py:6-30), whose
-stream is not reproduced here.
+fill the buffer on the device from a counter hash, as the reference's do
+(initializer/RandomUniform.py:13-27, RandomNormal.py:10-30): the host only
+draws the 31-bit seed from numpy's global generator, so np.random.seed(k)
+fixes the initial weights here exactly as it does there.
 """
-import math
-
 import numpy as np
 
 import litenn_amd.core as nc
+from litenn_amd.core.hip import api
+from litenn_amd.core.hip.ShallowMode import ShallowMode
 
 
 class Initializer:
@@ -59,68 +60,113 @@ def NumpyArray(np_array):
     return _NumpyArrayInit(np_array)
 
 
-class _HostRandom(Initializer):
-    def _draw(self, shape):
-        raise NotImplementedError()
-
-    def initialize_CLBuffer(self, buffer, tensor_shape):
-        buffer.set(np.ascontiguousarray(self._draw(tuple(tensor_shape)), dtype=np.float32))
+def _draw_seed():
+    """The reference's seed draw (RandomUniform.py:26, RandomNormal.py:29)."""
+    return int(np.random.randint(2147483648))
 
 
-class RandomUniform(_HostRandom):
-    def __init__(self, low=-1.0, high=1.0):
+class _RandomUniform(Initializer):
+    def __init__(self, low=0.0, high=1.0):
         self.low, self.high = low, high
 
-    def _draw(self, shape): return np.random.uniform(self.low, self.high, shape)
+    def initialize_CLBuffer(self, buffer, tensor_shape):
+        seed = _draw_seed()
+        if ShallowMode.active():
+            return
+        api.random_uniform(buffer.device.index, buffer.get_ptr(skip_init=True), buffer.size // 4, seed,
+                           self.low, self.high)
+
     def __str__(self): return f'RandomUniform low={self.low}, high={self.high}'
 
 
-class RandomNormal(_HostRandom):
+def RandomUniform(low=0.0, high=1.0):
+    """U[low, high] from the device hash (RandomUniform.py:32-43)."""
+    return nc.Cacheton.get(_RandomUniform, low, high)
+
+
+class _RandomNormal(Initializer):
     def __init__(self, mean=0.0, stddev=1.0):
         self.mean, self.stddev = mean, stddev
 
-    def _draw(self, shape): return np.random.normal(self.mean, self.stddev, shape)
+    def initialize_CLBuffer(self, buffer, tensor_shape):
+        seed = _draw_seed()
+        if ShallowMode.active():
+            return
+        api.random_normal(buffer.device.index, buffer.get_ptr(skip_init=True), buffer.size // 4, seed,
+                          self.mean, self.stddev)
+
     def __str__(self): return f'RandomNormal mean={self.mean}, stddev={self.stddev}'
 
 
-class _FanInit(_HostRandom):
-    def __init__(self, gain=1.0, fan_in=None, fan_out=None):
-        self.gain, self.fan_in, self.fan_out = gain, fan_in, fan_out
+def RandomNormal(mean=0.0, stddev=1.0):
+    """N(mean, stddev) by Box-Muller on the device hash (RandomNormal.py:35-46)."""
+    return nc.Cacheton.get(_RandomNormal, mean, stddev)
+
+
+class _FanInit(Initializer):
+    """He / Glorot: a RandomUniform(-a, a) with a = sqrt(3)*std or a RandomNormal(0, std), chosen on first use
+    once the layer has supplied the fans (He.py:18-33, Glorot.py:20-35).
+
+    Every call of HeNormal() etc. returns a fresh object, so each layer that fills in fan_in / fan_out gets its
+    own bound; the reference hands out one cached object per argument tuple, which keeps the fans (and the
+    bound) of the first layer that used it."""
+
+    def __init__(self, type, gain, fan_in=None, fan_out=None):
+        self.type, self.gain, self.fan_in, self.fan_out = type, gain, fan_in, fan_out
+        self.initer = None
 
     def has_fan_in(self): return True
 
+    def _std(self):
+        raise NotImplementedError()
 
-class HeNormal(_FanInit):
-    """N(0, gain*sqrt(2/fan_in))  (He.py:18-33,51-64)."""
-    def __init__(self, gain=1.0, fan_in=None):
-        super().__init__(gain, fan_in)
-
-    def _draw(self, shape):
-        return np.random.normal(0.0, self.gain * math.sqrt(2.0 / self.fan_in), shape)
-
-
-class HeUniform(_FanInit):
-    """U(-l, l), l = gain*sqrt(6/fan_in); default gain 2  (He.py:18-49)."""
-    def __init__(self, gain=2.0, fan_in=None):
-        super().__init__(gain, fan_in)
-
-    def _draw(self, shape):
-        lim = self.gain * math.sqrt(6.0 / self.fan_in)
-        return np.random.uniform(-lim, lim, shape)
+    def initialize_CLBuffer(self, buffer, tensor_shape):
+        if self.initer is None:
+            std = self._std()
+            if self.type == 'uniform':
+                a = np.sqrt(3.0) * std
+                self.initer = RandomUniform(-a, a)
+            else:
+                self.initer = RandomNormal(0.0, std)
+        self.initer.initialize_CLBuffer(buffer, tensor_shape)
 
 
-class GlorotNormal(_FanInit):
-    """N(0, gain*sqrt(2/(fan_in+fan_out)))  (Glorot.py:20-35,61-78)."""
+class _InitHe(_FanInit):
+    def _std(self):
+        if self.fan_in is None:
+            raise ValueError(f'fan_in should be set for {str(self)}')
+        return self.gain * np.sqrt(2.0 / self.fan_in)
+
+    def __str__(self): return f'InitHe type={self.type}, gain={self.gain}, fan_in={self.fan_in}'
+
+
+class _InitGlorot(_FanInit):
     def has_fan_out(self): return True
 
-    def _draw(self, shape):
-        return np.random.normal(0.0, self.gain * math.sqrt(2.0 / (self.fan_in + self.fan_out)), shape)
+    def _std(self):
+        if self.fan_in is None or self.fan_out is None:
+            raise ValueError(f'fan_in/fan_out should be set for {str(self)}')
+        return self.gain * np.sqrt(2.0 / (self.fan_in + self.fan_out))
+
+    def __str__(self):
+        return f'InitGlorot type={self.type}, gain={self.gain}, fan_in={self.fan_in}, fan_out={self.fan_out}'
 
 
-class GlorotUniform(_FanInit):
-    """U(-l, l), l = gain*sqrt(6/(fan_in+fan_out))  (Glorot.py:20-35,37-59)."""
-    def has_fan_out(self): return True
+def HeUniform(gain=2.0, fan_in=None):
+    """U(-a, a), a = sqrt(3)*gain*sqrt(2/fan_in); default gain 2 (He.py:36-49)."""
+    return _InitHe('uniform', gain, fan_in)
 
-    def _draw(self, shape):
-        lim = self.gain * math.sqrt(6.0 / (self.fan_in + self.fan_out))
-        return np.random.uniform(-lim, lim, shape)
+
+def HeNormal(gain=1.0, fan_in=None):
+    """N(0, gain*sqrt(2/fan_in)) (He.py:51-64)."""
+    return _InitHe('normal', gain, fan_in)
+
+
+def GlorotUniform(gain=1.0, fan_in=None, fan_out=None):
+    """U(-a, a), a = sqrt(3)*gain*sqrt(2/(fan_in+fan_out)) (Glorot.py:37-59)."""
+    return _InitGlorot('uniform', gain, fan_in, fan_out)
+
+
+def GlorotNormal(gain=1.0, fan_in=None, fan_out=None):
+    """N(0, gain*sqrt(2/(fan_in+fan_out))) (Glorot.py:61-78)."""
+    return _InitGlorot('normal', gain, fan_in, fan_out)

@@ -17,6 +17,8 @@ int launch_unfold2d(DeviceCtx*, int, int, int, int, int, int, int, int, int, int
                     float*, int);
 int launch_sgd(DeviceCtx*, uint64_t, float*, const float*, float*, float, float, int);
 int launch_adam(DeviceCtx*, uint64_t, float*, const float*, float*, float*, float, float, float);
+int launch_random_uniform(DeviceCtx*, float*, uint64_t, uint32_t, double, double);
+int launch_random_normal(DeviceCtx*, float*, uint64_t, uint32_t, double, double);
 
 static thread_local std::string g_error;
 constexpr int kMaxDevices = 64;
@@ -381,6 +383,16 @@ int lnn_adam_update_f32(int dev, uint64_t n, float* t, const float* g, float* m,
                         float lr) {
   CTX(dev);
   return launch_adam(ctx, n, t, g, m, v, beta1, beta2, lr);
+}
+
+int lnn_random_uniform_f32(int dev, float* out, uint64_t n, uint32_t seed, double low, double high) {
+  CTX(dev);
+  return launch_random_uniform(ctx, out, n, seed, low, high);
+}
+
+int lnn_random_normal_f32(int dev, float* out, uint64_t n, uint32_t seed, double mean, double stddev) {
+  CTX(dev);
+  return launch_random_normal(ctx, out, n, seed, mean, stddev);
 }
 
 }  // extern "C"

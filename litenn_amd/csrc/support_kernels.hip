@@ -402,6 +402,66 @@ int launch_sgd(DeviceCtx* ctx, uint64_t n, float* v, const float* g, float* acc,
   return LNN_OK;
 }
 
+// ---- on-device random initialisers ------------------------------------------------------------------------
+// The reference fills a fresh parameter tensor on the device from a counter hash: element i draws from
+// hash(i + seed), seed a host-side 31-bit integer (initializer/RandomUniform.py:13-27, RandomNormal.py:10-30).
+// The two PCG hashes follow the reference's device helper text (CLKernelHelper.py:210-228); unsigned 32-bit
+// arithmetic throughout, so the integer stream is reproducible bit for bit.
+__device__ __forceinline__ uint32_t hash_u32(uint32_t v) {
+  const uint32_t state = v * 747796405u + 2891336453u;
+  const uint32_t word = ((state >> ((state >> 28u) + 4u)) ^ state) * 277803737u;
+  return (word >> 22u) ^ word;
+}
+__device__ __forceinline__ void hash_u32x2(uint32_t& x, uint32_t& y) {
+  x = x * 1664525u + 1013904223u;
+  y = y * 1664525u + 1013904223u;
+  x += y * 1664525u;
+  y += x * 1664525u;
+  x ^= x >> 16u;
+  y ^= y >> 16u;
+  x += y * 1664525u;
+  y += x * 1664525u;
+  x ^= x >> 16u;
+  y ^= y >> 16u;
+}
+// (float)h * 2^-32: the reference multiplies by 1.0 / (float)0xffffffffU, and (float)0xffffffffU rounds to 2^32
+constexpr float kUnitScale = 1.0f / 4294967296.0f;
+
+// out[i] = u * (high - low) + low in double, as the reference's double literals make it (RandomUniform.py:17-21)
+__global__ void random_uniform_kernel(float* __restrict__ out, uint64_t n, uint32_t seed, double span, double low) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
+    const float u = (float)hash_u32((uint32_t)(i + seed)) * kUnitScale;
+    out[i] = (float)((double)u * span + low);
+  }
+}
+// Box-Muller on the two halves of the 2-D hash of (i + seed, 1) (RandomNormal.py:14-24); sqrt, log and cos in
+// single precision, mean + normal * stddev in double
+__global__ void random_normal_kernel(float* __restrict__ out, uint64_t n, uint32_t seed, double mean, double stddev) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
+    uint32_t x = (uint32_t)(i + seed), y = 1u;
+    hash_u32x2(x, y);
+    const float fx = (float)x * kUnitScale, fy = (float)y * kUnitScale;
+    const float normal = sqrtf(-2.0f * logf(fx)) * cosf((2.0f * 3.14159274101257f) * fy);
+    out[i] = (float)(mean + (double)normal * stddev);
+  }
+}
+
+int launch_random_uniform(DeviceCtx* ctx, float* out, uint64_t n, uint32_t seed, double low, double high) {
+  if (n == 0) return LNN_OK;
+  if (!out) return set_error(LNN_ERR_INVALID, "random_uniform: null pointer");
+  hipLaunchKernelGGL(random_uniform_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, out, n, seed, high - low, low);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+int launch_random_normal(DeviceCtx* ctx, float* out, uint64_t n, uint32_t seed, double mean, double stddev) {
+  if (n == 0) return LNN_OK;
+  if (!out) return set_error(LNN_ERR_INVALID, "random_normal: null pointer");
+  hipLaunchKernelGGL(random_normal_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, out, n, seed, mean, stddev);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
 int launch_adam(DeviceCtx* ctx, uint64_t n, float* t, const float* g, float* m, float* v2, float beta1, float beta2,
                 float lr) {
   if (n == 0) return LNN_OK;

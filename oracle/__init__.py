@@ -33,7 +33,14 @@ Pinning status (what checks each function, independent of its own formula):
                      data and within 1e-5 on random data
                      (tests/test_oracle_refpath.py)
 
-No function here is "parity unpinned".
+  hash_rng           integer hashes: permutation property by independent inversion,
+                     no collisions over 2**22 counters, avalanche; float stages:
+                     moments and Kolmogorov-Smirnov against scipy.stats
+                     (tests/test_oracle_hash_rng.py).  PARITY UNPINNED against the
+                     reference's device output: the reference holds no vector of
+                     these kernels and its OpenCL text cannot run here.
+
+No other function here is "parity unpinned".
 """
 from .conv_info import info_conv2d, ConvInfo                      # noqa: F401
 from .unfold import (unfold_index_map, unfold_T_index_map,        # noqa: F401

@@ -13,7 +13,7 @@ from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
          'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
-         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update']
+         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal']
 
 
 class FakeHip:
@@ -192,6 +192,16 @@ class FakeHip:
         M[:] = b1 * M + (np.float32(1) - b1) * G
         V[:] = b2 * V + (np.float32(1) - b2) * G * G
         T[:] = T - np.float32(lr) * M / (np.sqrt(V) + np.float32(1e-7))
+
+    def random_uniform(self, dev, out, n, seed, low, high):
+        from oracle import hash_rng
+        self.launches += 1
+        self.f(out)[:n] = hash_rng.random_uniform(n, seed, low, high)
+
+    def random_normal(self, dev, out, n, seed, mean, stddev):
+        from oracle import hash_rng
+        self.launches += 1
+        self.f(out)[:n] = hash_rng.random_normal(n, seed, mean, stddev)
 
 
 def install(monkeypatch, capacity=None):

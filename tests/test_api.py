@@ -9,7 +9,7 @@ import itertools
 import numpy as np
 import pytest
 
-from oracle import conv2d_all, conv2d_transpose_all, depthwise_all, info_conv2d
+from oracle import conv2d_all, conv2d_transpose_all, depthwise_all, hash_rng, info_conv2d
 
 
 def test_conv2d_reference_style(nn_backend):
@@ -419,6 +419,49 @@ def test_adam_closed_form(nn_backend):
             w = w - lr * m / (np.sqrt(v) + 1e-7)
         np.testing.assert_allclose(w_t.np(), w, rtol=2e-5, atol=1e-6)
         w_t._set_trainable(False)
+
+
+def test_random_initializers_fill_on_device(nn_backend):
+    """InitRandomUniform_test / InitRandomNormal_test and the He / Glorot lines of the reference's own test
+    (test.py:237-242), plus what the seed draw promises: np.random.seed fixes the weights, and they equal the
+    counter-hash stream of that seed (initializer/RandomUniform.py:17-27, RandomNormal.py:14-30)."""
+    nn = nn_backend
+    for init in [nn.initializer.GlorotUniform(1.0, 1.0, 1.0), nn.initializer.GlorotNormal(1.0, 1.0, 1.0),
+                 nn.initializer.HeUniform(1.0, 1.0), nn.initializer.HeNormal(1.0, 1.0),
+                 nn.initializer.RandomNormal(), nn.initializer.RandomUniform()]:
+        v = nn.Tensor((128,), init=init).np()
+        assert v.shape == (128,) and np.isfinite(v).all() and v.std() > 0.05
+
+    def seeds(k, n):
+        np.random.seed(k)
+        return [int(np.random.randint(2147483648)) for _ in range(n)]
+
+    np.random.seed(5)
+    u = nn.Tensor((3, 1000), init=nn.initializer.RandomUniform(-0.5, 1.5)).np()
+    z = nn.Tensor((4096,), init=nn.initializer.RandomNormal(0.25, 2.0)).np()
+    s0, s1 = seeds(5, 2)
+    assert np.allclose(u.reshape(-1), hash_rng.random_uniform(3000, s0, -0.5, 1.5), rtol=0, atol=3e-7)
+    assert np.allclose(z, hash_rng.random_normal(4096, s1, 0.25, 2.0), rtol=0, atol=2e-5)
+    assert u.min() >= -0.5 and u.max() <= 1.5
+
+    # default construction of the layers draws their kernels on the device, each with its own bound
+    np.random.seed(11)
+    conv = nn.Conv2D(8, 16, 3)
+    dense = nn.Dense(32, 64)
+    k, w = conv.kernel.np(), dense.weight.np()
+    a_conv = np.sqrt(3.0) * np.sqrt(2.0 / (8 * 9 + 16 * 9))
+    a_dense = np.sqrt(3.0) * np.sqrt(2.0 / (32 + 64))
+    assert np.abs(k).max() <= a_conv and np.abs(k).max() > 0.9 * a_conv
+    assert np.abs(w).max() <= a_dense and np.abs(w).max() > 0.9 * a_dense
+    s0 = seeds(11, 1)[0]
+    assert np.allclose(k.reshape(-1), hash_rng.random_uniform(k.size, s0, -a_conv, a_conv), rtol=0, atol=1e-7)
+    np.random.seed(11)
+    assert np.array_equal(nn.Conv2D(8, 16, 3).kernel.np(), k)
+
+    with pytest.raises(ValueError):
+        nn.Tensor((4,), init=nn.initializer.HeNormal()).np()          # fan_in never set
+    with pytest.raises(ValueError):
+        nn.Tensor((4,), init=nn.initializer.GlorotUniform(fan_in=3)).np()
 
 
 def test_pointwise_broadcast_and_reduce(nn_backend):

@@ -11,7 +11,7 @@ import itertools
 import numpy as np
 import pytest
 
-from oracle import depthwise_all
+from oracle import depthwise_all, hash_rng
 from oracle import (info_conv2d, conv2d_all, conv2d_fwd, conv2d_dx, conv2d_dw, unfold_index_map,
                     unfold_T_index_map, matmul_fwd)
 from tests.gpu_util import DevArr, rel_err, say
@@ -424,6 +424,35 @@ def test_conv_benchmark_geometries_float(hip, name):
     errs = (rel_err(y, ry), rel_err(dx, rdx), rel_err(dw, rdw))
     say(f'  normalised errors fwd/dX/dW = {errs}')
     assert max(errs) <= TOL
+
+
+def test_random_initialisers_match_the_counter_hash(hip):
+    """Integer stream bit for bit: with low 0 and span 1 the output IS (float)hash * 2^-32.  The affine map is in
+    double on both sides (one float ulp for a fused multiply-add); Box-Muller goes through single-precision
+    log / cos, whose last bits differ between libraries: 2e-6 of stddev-scaled absolute error."""
+    for n, seed in [(1, 0), (255, 1), (100003, 2147483647), (1 << 20, 123456789), (70000, 0xFFFFFFF0)]:
+        say(f'random n={n} seed={seed}')
+        out = DevArr(hip, shape=(n,), fill=np.nan)
+        hip.random_uniform(0, out.ptr, n, seed, 0.0, 1.0)
+        assert np.array_equal(out.get(), hash_rng.random_uniform(n, seed, 0.0, 1.0))
+        hip.random_uniform(0, out.ptr, n, seed, -0.3, 0.9)
+        ref = hash_rng.random_uniform(n, seed, -0.3, 0.9)
+        got = out.get()
+        assert np.abs(got - ref).max() <= np.spacing(np.float32(0.9))
+        assert (got == ref).mean() > 0.999
+        hip.random_normal(0, out.ptr, n, seed, 0.0, 1.0)
+        got, ref = out.get(), hash_rng.random_normal(n, seed, 0.0, 1.0)
+        ok = np.isfinite(ref)
+        assert np.array_equal(np.isfinite(got), ok)
+        assert np.abs(got[ok] - ref[ok]).max() <= 2e-6 * max(1.0, np.abs(ref[ok]).max())
+        hip.random_normal(0, out.ptr, n, seed, -2.0, 0.01)
+        got, ref = out.get(), hash_rng.random_normal(n, seed, -2.0, 0.01)
+        assert np.abs(got[ok] - ref[ok]).max() <= 5e-7
+    # a guard element after the end stays untouched
+    g = DevArr(hip, np.full(130, 7.0, np.float32))
+    hip.random_uniform(0, g.ptr, 129, 5, 0.0, 1.0)
+    assert g.get()[129] == 7.0
+    hip.random_normal(0, g.ptr, 0, 5, 0.0, 1.0)       # n = 0 is a no-op
 
 
 def test_conv_descriptor_errors(hip):

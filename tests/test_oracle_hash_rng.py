@@ -1,0 +1,107 @@
+"""Checks that pin oracle/hash_rng.py without retyping its formulas: both hashes are permutations (inverted
+here with modular inverses from pow() and by undoing each xor-shift), no collisions, avalanche, and the two
+float distributions against scipy.stats."""
+import numpy as np
+import pytest
+from scipy import stats
+
+from oracle import hash_rng
+
+M = 1 << 32
+
+
+def _unxorshift(y, s):
+    """Inverse of x -> x ^ (x >> s) on 32 bits."""
+    x = y
+    for _ in range(32 // s + 1):
+        x = y ^ (x >> s)
+    return x
+
+
+def _invert_hash_u32(h):
+    word = _unxorshift(h, 22)
+    mixed = (word * pow(277803737, -1, M)) % M
+    # the data-dependent shift is at least 4, so the top four bits of the state survive it
+    state = _unxorshift(mixed, (mixed >> 28) + 4)
+    return ((state - 2891336453) * pow(747796405, -1, M)) % M
+
+
+def _invert_hash_u32x2(x, y):
+    k, c = 1664525, 1013904223
+    kinv = pow(k, -1, M)
+    x, y = _unxorshift(x, 16), _unxorshift(y, 16)
+    y = (y - x * k) % M
+    x = (x - y * k) % M
+    x, y = _unxorshift(x, 16), _unxorshift(y, 16)
+    y = (y - x * k) % M
+    x = (x - y * k) % M
+    return ((x - c) * kinv) % M, ((y - c) * kinv) % M
+
+
+def test_hash_u32_is_inverted_by_the_permutation_steps():
+    rng = np.random.default_rng(1)
+    vs = np.concatenate([np.array([0, 1, 2, M - 1, M // 2]), rng.integers(0, M, 2000)]).astype(np.uint64)
+    hs = hash_rng.hash_u32(vs)
+    for v, h in zip(vs.tolist(), hs.tolist()):
+        assert _invert_hash_u32(int(h)) == int(v)
+
+
+def test_hash_u32x2_is_inverted_by_the_permutation_steps():
+    rng = np.random.default_rng(2)
+    xs = rng.integers(0, M, 2000).astype(np.uint64)
+    ys = np.concatenate([np.ones(1000, dtype=np.uint64), rng.integers(0, M, 1000).astype(np.uint64)])
+    hx, hy = hash_rng.hash_u32x2(xs, ys)
+    for x, y, a, b in zip(xs.tolist(), ys.tolist(), hx.tolist(), hy.tolist()):
+        assert _invert_hash_u32x2(int(a), int(b)) == (int(x), int(y))
+
+
+def test_hash_u32_has_no_collisions_on_consecutive_counters():
+    # a random function on 32 bits would collide about n^2 / 2^33 = 2048 times here
+    n = 1 << 22
+    h = hash_rng.hash_u32(np.arange(n, dtype=np.uint64) + np.uint64(0xFFF00000))   # spans the 2^32 wrap
+    assert np.unique(h).size == n
+
+
+@pytest.mark.parametrize('bit', [0, 7, 16, 31])
+def test_single_bit_avalanche(bit):
+    v = np.arange(1 << 16, dtype=np.uint64) * np.uint64(2654435761) & np.uint64(M - 1)
+    a, b = hash_rng.hash_u32(v), hash_rng.hash_u32(v ^ np.uint64(1 << bit))
+    flipped = np.unpackbits((a ^ b).view(np.uint8)).sum() / v.size
+    assert 13.0 < flipped < 19.0
+    ax, ay = hash_rng.hash_u32x2(v, np.ones_like(v))
+    bx, by = hash_rng.hash_u32x2(v ^ np.uint64(1 << bit), np.ones_like(v))
+    # the 2-D hash mixes less in its low bits than the 1-D one; a changed counter must still move both halves
+    assert np.unpackbits((ax ^ bx).view(np.uint8)).sum() / v.size > 8.0
+    assert np.unpackbits((ay ^ by).view(np.uint8)).sum() / v.size > 8.0
+
+
+def test_counter_wraps_modulo_2_32():
+    seed = 0xFFFFFFF0
+    a = hash_rng.random_uniform(64, seed)
+    b = hash_rng.random_uniform(48, 0)
+    assert np.array_equal(a[16:], b)          # element 16 has counter (16 + seed) mod 2^32 = 0
+
+
+def test_uniform_distribution_and_affine_map():
+    n = 1 << 20
+    u = hash_rng.random_uniform(n, 12345)
+    assert u.dtype == np.float32 and u.min() >= 0.0 and u.max() <= 1.0
+    assert abs(u.mean() - 0.5) < 2e-3 and abs(u.var() - 1 / 12) < 1e-3
+    assert stats.kstest(u[:200000].astype(np.float64), 'uniform').pvalue > 1e-3
+    w = hash_rng.random_uniform(n, 12345, -0.25, 0.75)
+    assert np.allclose(w, u.astype(np.float64) - 0.25, rtol=0, atol=1e-7)
+    # neighbouring seeds shift the stream by one element: the value depends on counter + seed only
+    assert np.array_equal(hash_rng.random_uniform(100, 8)[:-1], hash_rng.random_uniform(100, 7)[1:])
+
+
+def test_normal_distribution_and_affine_map():
+    n = 1 << 20
+    z = hash_rng.random_normal(n, 999)
+    z = z[np.isfinite(z)]
+    assert z.size >= n - 2
+    assert abs(z.mean()) < 4e-3 and abs(z.std() - 1.0) < 4e-3
+    assert abs(stats.skew(z.astype(np.float64))) < 0.02 and abs(stats.kurtosis(z.astype(np.float64))) < 0.05
+    assert stats.kstest(z[:200000].astype(np.float64), 'norm').pvalue > 1e-3
+    w = hash_rng.random_normal(n, 999, 1.5, 0.1)
+    ok = np.isfinite(w)
+    assert np.allclose(w[ok], 1.5 + 0.1 * hash_rng.random_normal(n, 999)[ok].astype(np.float64), rtol=0, atol=1e-6)
