@@ -108,6 +108,14 @@ int lnn_conv2d_fwd_f32(int dev, const lnn_conv2d_desc* d, const float* X, const 
 #define LNN_ACT_LEAKY_RELU 1
 int lnn_conv2d_fwd_bias_act_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* W,
                                 const float* bias, int act, float slope, float* Y);
+/* Backward of that epilogue in one pass over y and dy, both [N][O][HW] (the layer's bias add is
+ * dual_wise_op.py:110-130 for the broadcast operand, the activation gradient element_wise_op.py:211):
+ *   dpre = dy * (y >= 0 ? 1 : slope)       (act == LNN_ACT_LEAKY_RELU; slope > 0 so y has the sign of the
+ *                                            pre-activation)   or   dpre = dy   (LNN_ACT_NONE, y unused)
+ *   dbias[o] = (beta_bias ? dbias[o] : 0) + sum over n and pixels of dpre
+ * dpre may be NULL (only the bias gradient is wanted) or equal dy (in place); dbias may be NULL. */
+int lnn_bias_act_bwd_f32(int dev, int N, int O, int HW, const float* y, const float* dy, int act, float slope,
+                         float* dpre, float* dbias, int beta_bias);
 /* dX (+)= dgrad(dY, W)                   conv2D.py:46-50 (the reference always accumulates) */
 int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* W,
                          float* dX, int beta);

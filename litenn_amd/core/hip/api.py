@@ -79,6 +79,7 @@ SIGNATURES = {
     'lnn_reduce_sum_bwd_f32': [_c_int, _c_int, _i32arr, _c_u32, _c_f32, _ptr, _ptr],
     'lnn_sgd_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int],
     'lnn_adam_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32],
+    'lnn_bias_act_bwd_f32': [_c_int, _c_int, _c_int, _c_int, _ptr, _ptr, _c_int, _c_f32, _ptr, _ptr, _c_int],
     'lnn_random_uniform_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
     'lnn_random_normal_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
 }
@@ -285,3 +286,7 @@ def random_uniform(dev, out, n, seed, low, high):
 
 def random_normal(dev, out, n, seed, mean, stddev):
     check(lib.lnn_random_normal_f32(dev, out, int(n), int(seed), float(mean), float(stddev)))
+
+
+def bias_act_bwd(dev, N, O, HW, y, dy, act, slope, dpre, dbias, beta_bias):
+    check(lib.lnn_bias_act_bwd_f32(dev, N, O, HW, y, dy, act, float(slope), dpre, dbias, beta_bias))

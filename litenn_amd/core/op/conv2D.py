@@ -45,44 +45,65 @@ def conv2D_bias_act(input_t, kernel_t, bias_t=None, stride=1, dilation=1, paddin
     alpha = 0.0 if leaky_relu_alpha is None else float(leaky_relu_alpha)
     output_t = nn.Tensor(op.output_shape)
     output_t._set_op_name('conv2D_bias_act')
-    pre_grad = _PreActivationGrad(act, alpha)
-    output_t._assign_gradfn(input_t, lambda O_t, dO_t: conv2D_dI_gradfn(op, input_t, kernel_t, pre_grad(O_t, dO_t)))
-    output_t._assign_gradfn(kernel_t, lambda O_t, dO_t: conv2D_dK_gradfn(op, input_t, kernel_t, pre_grad(O_t, dO_t)))
+    epi = _EpilogueGrad(act, alpha)
+    # the bias comes first: when its gradient is wanted, the one pass that forms the pre-activation gradient also
+    # sums it per channel
+    if bias_t is not None:
+        output_t._assign_gradfn(bias_t, lambda O_t, dO_t: epi.bias(O_t, dO_t, bias_t))
+    output_t._assign_gradfn(input_t, lambda O_t, dO_t: conv2D_dI_gradfn(op, input_t, kernel_t, epi.pre(O_t, dO_t)))
+    output_t._assign_gradfn(kernel_t, lambda O_t, dO_t: conv2D_dK_gradfn(op, input_t, kernel_t, epi.pre(O_t, dO_t)))
     if bias_t is None:
         launch(lambda dev, x, w, y: api.conv2d_fwd_bias_act(dev, op.desc, x, w, None, act, alpha, y),
                input_t, kernel_t, (output_t, 'w'))
     else:
-        output_t._assign_gradfn(bias_t, lambda O_t, dO_t: _bias_gradfn(bias_t, pre_grad(O_t, dO_t)))
         launch(lambda dev, x, w, b, y: api.conv2d_fwd_bias_act(dev, op.desc, x, w, b, act, alpha, y),
                input_t, kernel_t, bias_t, (output_t, 'w'))
     return output_t
 
 
-class _PreActivationGrad:
-    """dO * f'(pre-activation), computed once per backward pass and shared by
-    the gradient functions of the fused op.  For leaky ReLU with alpha > 0 the
-    output has the sign of the pre-activation, so f' is read off the output."""
+class _EpilogueGrad:
+    """Backward of the fused epilogue, shared by the gradient functions of one conv2D_bias_act result.
+
+    pre(): dO * f'(pre-activation), formed once per backward pass.  For leaky ReLU with alpha > 0 the output has
+    the sign of the pre-activation, so f' is read off the output.
+    bias(): bias.grad[o] += sum of that over batch and pixels (dual_wise_op.py:110-130 for the broadcast
+    operand) - in the same launch as pre() when it runs first, which it does whenever the bias gradient is
+    wanted at all."""
 
     def __init__(self, act, alpha):
         self.act, self.alpha = act, alpha
         self.key, self.value = None, None
 
-    def __call__(self, O_t, dO_t):
+    def _run(self, O_t, dO_t, want_pre, bias_grad):
+        N, O, H, W = tuple(dO_t.shape)
+        pre = None
+        if want_pre:
+            pre = nn.Tensor(dO_t.shape)
+            self.key, self.value = dO_t, pre
+        args = [O_t, dO_t]
+        if pre is not None:
+            args.append((pre, 'w'))
+        beta = 0
+        if bias_grad is not None:
+            target, beta = nc.op.accumulate_target(bias_grad)
+            args.append(target)
+
+        def run(dev, y, dy, *outs):
+            outs = list(outs)
+            dpre = outs.pop(0) if pre is not None else None
+            dbias = outs.pop(0) if bias_grad is not None else None
+            api.bias_act_bwd(dev, N, O, H * W, y, dy, self.act, self.alpha, dpre, dbias, beta)
+        launch(run, *args)
+
+    def pre(self, O_t, dO_t):
         if self.act == api.ACT_NONE:
             return dO_t
         if self.key is not dO_t:
-            pre = nn.Tensor(dO_t.shape)
-            n = dO_t.shape.size
-            launch(lambda dev, o, do, di: api.ew_bwd(dev, api.EW_LEAKY_RELU, n, o, do, di, self.alpha),
-                   O_t, dO_t, pre)   # a fresh tensor is zero-filled on first use; the kernel adds into it
-            self.key, self.value = dO_t, pre
+            self._run(O_t, dO_t, True, None)
         return self.value
 
-
-def _bias_gradfn(bias_t, dpre_t):
-    """bias.grad[o] += sum over batch and pixels   (dual_wise_op.py:110-130 for the broadcast operand)."""
-    shape = tuple(dpre_t.shape)
-    launch(lambda dev, s, g: api.reduce_sum(dev, shape, (0, 2, 3), 1.0, s, g, 1), dpre_t, bias_t.get_grad())
+    def bias(self, O_t, dO_t, bias_t):
+        self._run(O_t, dO_t, self.act != api.ACT_NONE and self.key is not dO_t, bias_t.get_grad())
 
 
 def conv2D_dI_gradfn(op, input_t, kernel_t, dO_t):

@@ -18,6 +18,7 @@ int launch_unfold2d(DeviceCtx*, int, int, int, int, int, int, int, int, int, int
 int launch_sgd(DeviceCtx*, uint64_t, float*, const float*, float*, float, float, int);
 int launch_adam(DeviceCtx*, uint64_t, float*, const float*, float*, float*, float, float, float);
 int launch_random_uniform(DeviceCtx*, float*, uint64_t, uint32_t, double, double);
+int launch_bias_act_bwd(DeviceCtx*, int, int, int, const float*, const float*, int, float, float*, float*, int);
 int launch_random_normal(DeviceCtx*, float*, uint64_t, uint32_t, double, double);
 
 static thread_local std::string g_error;
@@ -383,6 +384,12 @@ int lnn_adam_update_f32(int dev, uint64_t n, float* t, const float* g, float* m,
                         float lr) {
   CTX(dev);
   return launch_adam(ctx, n, t, g, m, v, beta1, beta2, lr);
+}
+
+int lnn_bias_act_bwd_f32(int dev, int N, int O, int HW, const float* y, const float* dy, int act, float slope,
+                         float* dpre, float* dbias, int beta_bias) {
+  CTX(dev);
+  return launch_bias_act_bwd(ctx, N, O, HW, y, dy, act, slope, dpre, dbias, beta_bias);
 }
 
 int lnn_random_uniform_f32(int dev, float* out, uint64_t n, uint32_t seed, double low, double high) {

@@ -402,6 +402,100 @@ int launch_sgd(DeviceCtx* ctx, uint64_t n, float* v, const float* g, float* acc,
   return LNN_OK;
 }
 
+// ---- backward of the fused conv epilogue --------------------------------------------------------------------
+// One pass over Y and dY (both [N][O][HW]) gives the gradient before the activation, dpre = dY * f'(Y), and the
+// bias gradient dbias[o] (+)= sum over n and pixels of dpre: the separate activation-gradient kernel and the
+// reduction that follow it in the reference (element_wise_op.py:211, dual_wise_op.py:110-130) read dpre again.
+// Channel o's elements are cut into pieces of 2048 consecutive floats of one plane; block (slice, o) walks a
+// contiguous range of pieces, so the sums are formed in a fixed order whatever the grid.
+constexpr int kEpiPiece = 2048;
+
+__global__ __launch_bounds__(256) void bias_act_bwd_kernel(int N, int O, int HW, int ppp, int slices,
+                                                           const float* __restrict__ y, const float* dy,
+                                                           int act, float slope, float* dpre,
+                                                           float* __restrict__ part, int vec) {
+  const int o = blockIdx.y, sl = blockIdx.x;
+  const long long total = (long long)N * ppp;
+  const long long p0 = total * sl / slices, p1 = total * (sl + 1) / slices;
+  float acc = 0.0f;
+  for (long long p = p0; p < p1; ++p) {
+    const int n = (int)(p / ppp), piece = (int)(p - (long long)n * ppp);
+    const size_t base = ((size_t)n * O + o) * HW + (size_t)piece * kEpiPiece;
+    const int len = HW - piece * kEpiPiece < kEpiPiece ? HW - piece * kEpiPiece : kEpiPiece;
+    if (vec) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int e = (h * 256 + threadIdx.x) * 4;
+        if (e < len) {
+          f32x4 g = *reinterpret_cast<const f32x4*>(dy + base + e);
+          if (act == LNN_ACT_LEAKY_RELU) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(y + base + e);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) g[c] *= v[c] >= 0.0f ? 1.0f : slope;
+          }
+          if (dpre) *reinterpret_cast<f32x4*>(dpre + base + e) = g;
+          acc += (g[0] + g[1]) + (g[2] + g[3]);
+        }
+      }
+    } else {
+      for (int e = threadIdx.x; e < len; e += 256) {
+        float g = dy[base + e];
+        if (act == LNN_ACT_LEAKY_RELU) g *= y[base + e] >= 0.0f ? 1.0f : slope;
+        if (dpre) dpre[base + e] = g;
+        acc += g;
+      }
+    }
+  }
+  if (!part) return;
+  __shared__ float red[4];
+#pragma unroll
+  for (int s = 32; s > 0; s >>= 1) acc += __shfl_xor(acc, s, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) part[(size_t)o * slices + sl] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__global__ void bias_act_bwd_finish_kernel(int O, int slices, const float* __restrict__ part, float* __restrict__ dbias,
+                                           int beta) {
+  const int o = blockIdx.x * blockDim.x + threadIdx.x;
+  if (o >= O) return;
+  float v = 0.0f;
+  for (int s = 0; s < slices; ++s) v += part[(size_t)o * slices + s];
+  dbias[o] = beta ? dbias[o] + v : v;
+}
+
+int launch_bias_act_bwd(DeviceCtx* ctx, int N, int O, int HW, const float* y, const float* dy, int act, float slope,
+                        float* dpre, float* dbias, int beta) {
+  if (N <= 0 || O <= 0 || HW <= 0) return set_error(LNN_ERR_INVALID, "bias_act_bwd: non-positive dimension");
+  if (act != LNN_ACT_NONE && act != LNN_ACT_LEAKY_RELU) return set_error(LNN_ERR_INVALID, "bias_act_bwd: unknown activation");
+  if (!dy || (act != LNN_ACT_NONE && !y)) return set_error(LNN_ERR_INVALID, "bias_act_bwd: null pointer");
+  if (!dpre && !dbias) return set_error(LNN_ERR_INVALID, "bias_act_bwd: nothing to compute");
+  if ((uint64_t)N * O * HW * 4 > kMaxTensorBytes) return set_error(LNN_ERR_UNSUPPORTED, "bias_act_bwd: a tensor of 2 GiB or more");
+  if (O > 65535) return set_error(LNN_ERR_UNSUPPORTED, "bias_act_bwd: more than 65535 channels");
+  const int ppp = (HW + kEpiPiece - 1) / kEpiPiece;
+  const long long total = (long long)N * ppp;
+  long long slices = ((long long)ctx->cus * 8 + O - 1) / O;
+  if (slices > total) slices = total;
+  if (slices < 1) slices = 1;
+  float* part = nullptr;
+  if (dbias) {
+    int st = ensure_workspace(ctx, (size_t)O * slices * sizeof(float));
+    if (st != LNN_OK) return st;
+    part = static_cast<float*>(ctx->ws);
+  }
+  auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const int vec = HW % 4 == 0 && aligned(dy) && aligned(y) && aligned(dpre);
+  hipLaunchKernelGGL(bias_act_bwd_kernel, dim3((unsigned)slices, (unsigned)O), dim3(256), 0, ctx->stream, N, O, HW, ppp,
+                     (int)slices, y, dy, act, slope, dpre, part, vec);
+  LNN_HIP(hipGetLastError());
+  if (dbias) {
+    hipLaunchKernelGGL(bias_act_bwd_finish_kernel, dim3((O + 255) / 256), dim3(256), 0, ctx->stream, O, (int)slices, part,
+                       dbias, beta ? 1 : 0);
+    LNN_HIP(hipGetLastError());
+  }
+  return LNN_OK;
+}
+
 // ---- on-device random initialisers ------------------------------------------------------------------------
 // The reference fills a fresh parameter tensor on the device from a counter hash: element i draws from
 // hash(i + seed), seed a host-side 31-bit integer (initializer/RandomUniform.py:13-27, RandomNormal.py:10-30).

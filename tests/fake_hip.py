@@ -13,7 +13,7 @@ from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
          'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
-         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal']
+         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal', 'bias_act_bwd']
 
 
 class FakeHip:
@@ -192,6 +192,19 @@ class FakeHip:
         M[:] = b1 * M + (np.float32(1) - b1) * G
         V[:] = b2 * V + (np.float32(1) - b2) * G * G
         T[:] = T - np.float32(lr) * M / (np.sqrt(V) + np.float32(1e-7))
+
+    def bias_act_bwd(self, dev, N, O, HW, y, dy, act, slope, dpre, dbias, beta_bias):
+        self.launches += 1
+        n = N * O * HW
+        g = self.f(dy)[:n].copy()
+        if act == real_api.ACT_LEAKY_RELU:
+            g *= np.where(self.f(y)[:n] >= 0, np.float32(1), np.float32(slope))
+        if dpre is not None:
+            self.f(dpre)[:n] = g
+        if dbias is not None:
+            db = g.reshape(N, O, HW).astype(np.float64).sum(axis=(0, 2)).astype(np.float32)
+            B = self.f(dbias)[:O]
+            B[:] = B + db if beta_bias else db
 
     def random_uniform(self, dev, out, n, seed, low, high):
         from oracle import hash_rng

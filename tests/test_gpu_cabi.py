@@ -426,6 +426,46 @@ def test_conv_benchmark_geometries_float(hip, name):
     assert max(errs) <= TOL
 
 
+def test_bias_act_bwd_one_pass(hip):
+    """dpre = dy * f'(y) and dbias[o] (+)= sum dpre: exact on small integers with a power-of-two slope, <= 1e-5 of
+    the largest |dbias| on floats (fp32 sums against fp64)."""
+    rs = np.random.RandomState(21)
+    cases = [(1, 1, 1), (2, 3, 7), (4, 8, 56 * 56), (3, 5, 2048), (2, 4, 2049 * 4), (1, 2, 5000), (5, 130, 36),
+             (64, 16, 32 * 32), (1, 300, 3)]
+    for N, O, HW in cases:
+        for act, slope in [(hip.ACT_LEAKY_RELU, 0.25), (hip.ACT_NONE, 0.0)]:
+            say(f'bias_act_bwd N={N} O={O} HW={HW} act={act}')
+            y = rs.randint(-8, 8, size=(N, O, HW)).astype(np.float32)
+            dy = rs.randint(-8, 8, size=(N, O, HW)).astype(np.float32)
+            b0 = rs.randint(-8, 8, size=(O,)).astype(np.float32)
+            ref = dy * (np.where(y >= 0, 1.0, slope).astype(np.float32) if act == hip.ACT_LEAKY_RELU else 1.0)
+            rb = ref.astype(np.float64).sum(axis=(0, 2))
+            Y, DY = DevArr(hip, y), DevArr(hip, dy)
+            P, B = DevArr(hip, shape=y.shape, fill=np.nan), DevArr(hip, b0)
+            hip.bias_act_bwd(0, N, O, HW, Y.ptr, DY.ptr, act, slope, P.ptr, B.ptr, 1)
+            assert np.array_equal(P.get(), ref)
+            assert np.array_equal(B.get(), (rb + b0).astype(np.float32))
+            hip.bias_act_bwd(0, N, O, HW, Y.ptr, DY.ptr, act, slope, None, B.ptr, 0)       # bias gradient only
+            assert np.array_equal(B.get(), rb.astype(np.float32))
+            hip.bias_act_bwd(0, N, O, HW, Y.ptr, DY.ptr, act, slope, DY.ptr, None, 0)      # in place, no bias
+            assert np.array_equal(DY.get(), ref)
+    N, O, HW = 32, 128, 56 * 56
+    y = rs.standard_normal((N, O, HW)).astype(np.float32)
+    dy = rs.standard_normal((N, O, HW)).astype(np.float32)
+    ref = dy.astype(np.float64) * np.where(y >= 0, 1.0, np.float64(np.float32(0.2)))
+    Y, DY = DevArr(hip, y), DevArr(hip, dy)
+    P, B = DevArr(hip, shape=y.shape, fill=np.nan), DevArr(hip, shape=(O,), fill=np.nan)
+    hip.bias_act_bwd(0, N, O, HW, Y.ptr, DY.ptr, hip.ACT_LEAKY_RELU, 0.2, P.ptr, B.ptr, 0)
+    assert rel_err(P.get(), ref) <= 1e-6
+    assert rel_err(B.get(), ref.sum(axis=(0, 2))) <= 1e-5
+    for bad in [lambda: hip.bias_act_bwd(0, 0, 1, 1, Y.ptr, DY.ptr, hip.ACT_NONE, 0.0, P.ptr, B.ptr, 0),
+                lambda: hip.bias_act_bwd(0, 1, 1, 1, Y.ptr, DY.ptr, 7, 0.0, P.ptr, B.ptr, 0),
+                lambda: hip.bias_act_bwd(0, 1, 1, 1, Y.ptr, DY.ptr, hip.ACT_NONE, 0.0, None, None, 0),
+                lambda: hip.bias_act_bwd(0, 1, 1, 1, None, DY.ptr, hip.ACT_LEAKY_RELU, 0.1, P.ptr, None, 0)]:
+        with pytest.raises(hip.HipException):
+            bad()
+
+
 def test_random_initialisers_match_the_counter_hash(hip):
     """Integer stream bit for bit: with low 0 and span 1 the output IS (float)hash * 2^-32.  The affine map is in
     double on both sides (one float ulp for a fused multiply-add); Box-Muller goes through single-precision
