@@ -71,8 +71,81 @@ struct DwFilter {
 };
 constexpr int kDwMaxTaps = 1024;   // runtime-sized filters of up to 32 x 32 taps
 
+// Stride 1, dilation 1, compile-time filter: dst[r][c] = sum over (a, b) of src[r - pt + a][c - pl + b] * w(a, b).
+// A thread keeps one column and a contiguous run of the band's rows, and slides a KS x KS window of source values
+// down the column: a produced element costs KS LDS reads instead of KS * KS.  A source element outside the plane
+// reads element 0 of the band and is replaced by zero.
+template <int KS>
+struct DwColumn {
+  int cw[KS > 0 ? KS : 1];
+  bool okw[KS > 0 ? KS : 1];
+  __device__ __forceinline__ void init(int c, int pl, int srcW) {
+#pragma unroll
+    for (int b = 0; b < KS; ++b) {
+      const int s = c - pl + b;
+      okw[b] = (uint32_t)s < (uint32_t)srcW;
+      cw[b] = okw[b] ? s : 0;
+    }
+  }
+  __device__ __forceinline__ void load_row(const float* lds, int lo, int srcH, int srcW, int sr, float* out) const {
+    const bool okh = (uint32_t)sr < (uint32_t)srcH;
+    const float* row = lds + (okh ? (sr - lo) * srcW : 0);
+    // the reads stay unconditional (the empty statement uses every value), so a row's reads are in flight together
+    float x[KS > 0 ? KS : 1];
+#pragma unroll
+    for (int b = 0; b < KS; ++b) x[b] = row[cw[b]];
+#pragma unroll
+    for (int b = 0; b < KS; ++b) asm volatile("" : "+v"(x[b]));
+#pragma unroll
+    for (int b = 0; b < KS; ++b) out[b] = (okh && okw[b]) ? x[b] : 0.0f;
+  }
+};
+
+// rows [ra, rb) of the band for this thread's row group, and whether the thread takes part at all
+__device__ __forceinline__ bool dw_row_group(int width, int r0, int r1, int& tc, int& ncol, int& ra, int& rb) {
+  ncol = width < 256 ? width : 256;
+  const int ngrp = 256 / ncol, tg = threadIdx.x / ncol;
+  tc = threadIdx.x - tg * ncol;
+  const int rpg = (r1 - r0 + ngrp - 1) / ngrp;
+  ra = r0 + tg * rpg;
+  rb = ra + rpg < r1 ? ra + rpg : r1;
+  return tg < ngrp && ra < rb;
+}
+
+template <int KS, bool FLIP>
+__device__ __forceinline__ void dw_unit_rows(const float* lds, int lo, int srcH, int srcW, int dstW, int r0, int r1,
+                                             int pt, int pl, const float* k, float* __restrict__ dst, int beta) {
+  constexpr int T = KS > 0 ? KS : 1;
+  int tc, ncol, ra, rb;
+  if (!dw_row_group(dstW, r0, r1, tc, ncol, ra, rb)) return;
+  float w[T * T];
+#pragma unroll
+  for (int i = 0; i < KS * KS; ++i) w[i] = FLIP ? k[KS * KS - 1 - i] : k[i];
+  for (int c = tc; c < dstW; c += ncol) {
+    DwColumn<KS> col;
+    col.init(c, pl, srcW);
+    float win[T][T];
+#pragma unroll
+    for (int j = 0; j + 1 < KS; ++j) col.load_row(lds, lo, srcH, srcW, ra - pt + j, win[j + 1]);
+    for (int r = ra; r < rb; ++r) {
+#pragma unroll
+      for (int j = 0; j + 1 < KS; ++j)
+#pragma unroll
+        for (int b = 0; b < KS; ++b) win[j][b] = win[j + 1][b];
+      col.load_row(lds, lo, srcH, srcW, r - pt + KS - 1, win[KS - 1]);
+      float v = 0.0f;
+#pragma unroll
+      for (int a = 0; a < KS; ++a)
+#pragma unroll
+        for (int b = 0; b < KS; ++b) v += win[a][b] * w[a * KS + b];
+      const int o = r * dstW + c;
+      dst[o] = beta ? dst[o] + v : v;
+    }
+  }
+}
+
 // forward: Y rows [r0, r1) of the plane from X rows [lo, hi]
-template <int KS, int LDSF>
+template <int KS, int LDSF, bool UNIT>
 __global__ __launch_bounds__(256) void dw_fwd_kernel(DwGeom g, const float* __restrict__ X, const float* __restrict__ K,
                                                      float* __restrict__ Y, int bands, int TH, int beta) {
   __shared__ __attribute__((aligned(16))) float lds[LDSF];
@@ -89,6 +162,10 @@ __global__ __launch_bounds__(256) void dw_fwd_kernel(DwGeom g, const float* __re
   dw_copy_wait();
   __syncthreads();
   float* yp = Y + (size_t)plane * g.OH * g.OW;
+  if (KS > 0 && UNIT) {
+    dw_unit_rows<KS, false>(lds, lo, g.IH, g.IW, g.OW, r0, r1, g.PADT, g.PADL, f.k, yp, beta);
+    return;
+  }
   if (KS > 0) {
     // A thread keeps one output column and walks down the band's rows: the column tests and offsets of the
     // KS taps are computed once, a row costs KS row tests and KS*KS guarded multiply-adds.
@@ -148,7 +225,7 @@ __global__ __launch_bounds__(256) void dw_fwd_kernel(DwGeom g, const float* __re
     yp[o] = beta ? yp[o] + v : v;
   }
 }
-template <int KS, int LDSF>
+template <int KS, int LDSF, bool UNIT>
 __global__ __launch_bounds__(256) void dw_dgrad_kernel(DwGeom g, const float* __restrict__ dY,
                                                        const float* __restrict__ K, float* __restrict__ dX, int bands,
                                                        int TH, int beta) {
@@ -167,6 +244,11 @@ __global__ __launch_bounds__(256) void dw_dgrad_kernel(DwGeom g, const float* __
   dw_copy_wait();
   __syncthreads();
   float* xp = dX + (size_t)plane * g.IH * g.IW;
+  if (KS > 0 && UNIT) {
+    // dX[ih][iw] = sum dY[ih + PADT - kh][iw + PADL - kw] * k[kh][kw]: the same walk with the filter turned by 180 degrees
+    dw_unit_rows<KS, true>(lds, lo, g.OH, g.OW, g.IW, r0, r1, KS - 1 - g.PADT, KS - 1 - g.PADL, f.k, xp, beta);
+    return;
+  }
   if (KS > 0) {
     // column walk as in the forward kernel: the output column of each tap and whether it exists are fixed per thread
     const int ncol = g.IW < 256 ? g.IW : 256, ngrp = 256 / ncol;
@@ -226,34 +308,38 @@ __global__ __launch_bounds__(256) void dw_dgrad_kernel(DwGeom g, const float* __
   }
 }
 
-// kernel gradient: block (plane, band) holds dY rows [r0, r1) and the X rows under them and writes, per tap,
-// the sum of X * dY over the band to part[(plane*bands + band)*KK + tap]
-template <int KS, int LDSF, int LDSY>
-__global__ __launch_bounds__(256) void dw_wgrad_kernel(DwGeom g, const float* __restrict__ X,
-                                                       const float* __restrict__ dY, float* __restrict__ part,
-                                                       int bands, int TH) {
-  __shared__ __attribute__((aligned(16))) float ldsx[LDSF];
-  __shared__ __attribute__((aligned(16))) float ldsy[LDSY];
-  __shared__ float red[4];
-  const int plane = blockIdx.x / bands, band = blockIdx.x - plane * bands;
-  const int r0 = band * TH, r1 = r0 + TH < g.OH ? r0 + TH : g.OH;
-  int lo = r0 * g.S - g.PADT, hi = (r1 - 1) * g.S - g.PADT + (g.KH - 1) * g.D;
-  lo = lo < 0 ? 0 : lo;
-  hi = hi >= g.IH ? g.IH - 1 : hi;
-  if (hi >= lo) dw_copy_rows(ldsx, X + (size_t)plane * g.IH * g.IW, lo, hi, g.IW);
-  dw_copy_rows(ldsy, dY + (size_t)plane * g.OH * g.OW, r0, r1 - 1, g.OW);
-  dw_copy_wait();
-  __syncthreads();
-  const int n = (r1 - r0) * g.OW, KK = g.KH * g.KW;
-  float* out = part + ((size_t)plane * bands + band) * KK;
-  if (KS > 0) {
-    // every thread keeps one running sum per tap over its pixels, then the taps are reduced over the block
-    constexpr int T = KS > 0 ? KS * KS : 1;
-    float acc[T];
+// Kernel gradient, compile-time filter: adds X * dY of the dY rows [r0, r1) held in ldsy (row r0 first) and the X
+// rows from lo on held in ldsx to the thread's running sum per tap.
+template <int KS, bool UNIT>
+__device__ __forceinline__ void dw_wgrad_accumulate(const DwGeom& g, const float* ldsx, const float* ldsy, int r0, int r1,
+                                                    int lo, float* acc) {
+  constexpr int T = KS > 0 ? KS * KS : 1;
+  int tc, ncol, ra, rb;
+  const bool active = dw_row_group(g.OW, r0, r1, tc, ncol, ra, rb);
+  if (UNIT && active) {
+    // the window of X slides down the column with the output row; each of its elements meets the row's dY value
+    for (int ow = tc; ow < g.OW; ow += ncol) {
+      DwColumn<KS> col;
+      col.init(ow, g.PADL, g.IW);
+      float win[KS > 0 ? KS : 1][KS > 0 ? KS : 1];
 #pragma unroll
-    for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-    const int ncol = g.OW < 256 ? g.OW : 256, ngrp = 256 / ncol;
-    const int tc = threadIdx.x % ncol, tg = threadIdx.x / ncol;
+      for (int j = 0; j + 1 < KS; ++j) col.load_row(ldsx, lo, g.IH, g.IW, ra - g.PADT + j, win[j + 1]);
+      for (int oh = ra; oh < rb; ++oh) {
+#pragma unroll
+        for (int j = 0; j + 1 < KS; ++j)
+#pragma unroll
+          for (int b = 0; b < KS; ++b) win[j][b] = win[j + 1][b];
+        col.load_row(ldsx, lo, g.IH, g.IW, oh - g.PADT + KS - 1, win[KS - 1]);
+        const float dyv = ldsy[(oh - r0) * g.OW + ow];
+#pragma unroll
+        for (int a = 0; a < KS; ++a)
+#pragma unroll
+          for (int b = 0; b < KS; ++b) acc[a * KS + b] += win[a][b] * dyv;
+      }
+    }
+  }
+  if (!UNIT) {
+    const int ngrp = 256 / ncol, tg = threadIdx.x / ncol;
     for (int ow = tc; ow < g.OW; ow += ncol) {
       if (tg >= ngrp) break;
       int iw[T];
@@ -283,22 +369,57 @@ __global__ __launch_bounds__(256) void dw_wgrad_kernel(DwGeom g, const float* __
           for (int kw = 0; kw < KS; ++kw) acc[kh * KS + kw] += (okh[kh] && okw[kw]) ? x[kh * KS + kw] * dyv : 0.0f;
       }
     }
-    // wavefront butterflies of all taps side by side (their exchanges overlap), then the four wavefront sums
-    __shared__ float red2[4][T];
+  }
+}
+
+// Sum of every tap's running sums over the block, in a fixed order: wavefront butterflies of all taps side by side
+// (their exchanges overlap), then the four wavefront sums.
+template <int T>
+__device__ __forceinline__ void dw_reduce_taps(float* acc, float* out) {
+  __shared__ float red2[4][T];
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      float got[T];
+  for (int o = 32; o > 0; o >>= 1) {
+    float got[T];
 #pragma unroll
-      for (int t = 0; t < T; ++t) got[t] = __shfl_xor(acc[t], o, 64);
+    for (int t = 0; t < T; ++t) got[t] = __shfl_xor(acc[t], o, 64);
 #pragma unroll
-      for (int t = 0; t < T; ++t) acc[t] += got[t];
-    }
-    if ((threadIdx.x & 63) == 0) {
+    for (int t = 0; t < T; ++t) acc[t] += got[t];
+  }
+  if ((threadIdx.x & 63) == 0) {
 #pragma unroll
-      for (int t = 0; t < T; ++t) red2[threadIdx.x >> 6][t] = acc[t];
-    }
-    __syncthreads();
-    if (threadIdx.x < T) out[threadIdx.x] = (red2[0][threadIdx.x] + red2[1][threadIdx.x]) + (red2[2][threadIdx.x] + red2[3][threadIdx.x]);
+    for (int t = 0; t < T; ++t) red2[threadIdx.x >> 6][t] = acc[t];
+  }
+  __syncthreads();
+  if (threadIdx.x < T) out[threadIdx.x] = (red2[0][threadIdx.x] + red2[1][threadIdx.x]) + (red2[2][threadIdx.x] + red2[3][threadIdx.x]);
+}
+
+// kernel gradient: block (plane, band) holds dY rows [r0, r1) and the X rows under them and writes, per tap,
+// the sum of X * dY over the band to part[(plane*bands + band)*KK + tap]
+template <int KS, int LDSF, int LDSY, bool UNIT>
+__global__ __launch_bounds__(256) void dw_wgrad_kernel(DwGeom g, const float* __restrict__ X,
+                                                       const float* __restrict__ dY, float* __restrict__ part,
+                                                       int bands, int TH) {
+  __shared__ __attribute__((aligned(16))) float ldsx[LDSF];
+  __shared__ __attribute__((aligned(16))) float ldsy[LDSY];
+  __shared__ float red[4];
+  const int plane = blockIdx.x / bands, band = blockIdx.x - plane * bands;
+  const int r0 = band * TH, r1 = r0 + TH < g.OH ? r0 + TH : g.OH;
+  int lo = r0 * g.S - g.PADT, hi = (r1 - 1) * g.S - g.PADT + (g.KH - 1) * g.D;
+  lo = lo < 0 ? 0 : lo;
+  hi = hi >= g.IH ? g.IH - 1 : hi;
+  if (hi >= lo) dw_copy_rows(ldsx, X + (size_t)plane * g.IH * g.IW, lo, hi, g.IW);
+  dw_copy_rows(ldsy, dY + (size_t)plane * g.OH * g.OW, r0, r1 - 1, g.OW);
+  dw_copy_wait();
+  __syncthreads();
+  const int n = (r1 - r0) * g.OW, KK = g.KH * g.KW;
+  float* out = part + ((size_t)plane * bands + band) * KK;
+  if (KS > 0) {
+    constexpr int T = KS > 0 ? KS * KS : 1;
+    float acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+    dw_wgrad_accumulate<KS, UNIT>(g, ldsx, ldsy, r0, r1, lo, acc);
+    dw_reduce_taps<T>(acc, out);
   } else {
     for (int kh = 0; kh < g.KH; ++kh)
       for (int kw = 0; kw < g.KW; ++kw) {
@@ -317,6 +438,37 @@ __global__ __launch_bounds__(256) void dw_wgrad_kernel(DwGeom g, const float* __
         __syncthreads();
       }
   }
+}
+
+
+// Kernel gradient when a whole X plane and dY plane fit in LDS twice: block (slice, channel) walks its images'
+// planes of that channel, the transfers of the next plane running while the current one is accumulated, and reduces
+// once at the end: part[(slice*C + c)*KK + tap].  stage = floats per LDS stage, xf = floats reserved for the X plane.
+template <int KS, bool UNIT>
+__global__ __launch_bounds__(256) void dw_wgrad_planes_kernel(DwGeom g, const float* __restrict__ X,
+                                                              const float* __restrict__ dY, float* __restrict__ part,
+                                                              int slices, int stage, int xf) {
+  extern __shared__ __attribute__((aligned(16))) float dw_lds[];
+  constexpr int T = KS > 0 ? KS * KS : 1;
+  const int c = blockIdx.x % g.C, sl = blockIdx.x / g.C;
+  const int n0 = (int)((long long)g.N * sl / slices), n1 = (int)((long long)g.N * (sl + 1) / slices);
+  float acc[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+  auto fetch = [&](int n, int st) {
+    const size_t plane = (size_t)n * g.C + c;
+    dw_copy_rows(dw_lds + st * stage, X + plane * g.IH * g.IW, 0, g.IH - 1, g.IW);
+    dw_copy_rows(dw_lds + st * stage + xf, dY + plane * g.OH * g.OW, 0, g.OH - 1, g.OW);
+  };
+  if (n0 < n1) fetch(n0, 0);
+  for (int n = n0; n < n1; ++n) {
+    const int st = (n - n0) & 1;
+    dw_copy_wait();
+    __syncthreads();   // plane n has landed for every wavefront, and every wavefront is done with plane n - 1
+    if (n + 1 < n1) fetch(n + 1, st ^ 1);
+    dw_wgrad_accumulate<KS, UNIT>(g, dw_lds + st * stage, dw_lds + st * stage + xf, 0, g.OH, 0, acc);
+  }
+  dw_reduce_taps<T>(acc, part + ((size_t)sl * g.C + c) * T);
 }
 
 // dK[c][tap] (+)= sum over images and bands, in a fixed order.  One block per channel: thread (j, tap) adds every
@@ -384,15 +536,16 @@ int launch_dw_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, cons
   if (g.KH * g.KW > kDwMaxTaps) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d: more than 1024 taps");
   const dim3 grid((unsigned)(g.N * g.C * bands)), block(256);
   const int b = beta ? 1 : 0;
-#define LNN_DW_LAUNCH(KS)                                                                                  \
+#define LNN_DW_LAUNCH(KS, UNIT)                                                                                  \
   do {                                                                                                     \
-    if (small) hipLaunchKernelGGL((dw_fwd_kernel<KS, kDwSmall>), grid, block, 0, ctx->stream, g, X, K, Y, bands, TH, b); \
-    else hipLaunchKernelGGL((dw_fwd_kernel<KS, kDwLarge>), grid, block, 0, ctx->stream, g, X, K, Y, bands, TH, b);       \
+    if (small) hipLaunchKernelGGL((dw_fwd_kernel<KS, kDwSmall, UNIT>), grid, block, 0, ctx->stream, g, X, K, Y, bands, TH, b); \
+    else hipLaunchKernelGGL((dw_fwd_kernel<KS, kDwLarge, UNIT>), grid, block, 0, ctx->stream, g, X, K, Y, bands, TH, b);       \
   } while (0)
-  if (g.KH == g.KW && g.KH == 3) LNN_DW_LAUNCH(3);
-  else if (g.KH == g.KW && g.KH == 5) LNN_DW_LAUNCH(5);
-  else if (g.KH == g.KW && g.KH == 1) LNN_DW_LAUNCH(1);
-  else LNN_DW_LAUNCH(0);
+  const bool unit = g.S == 1 && g.D == 1;   // sliding-window kernels
+  if (g.KH == g.KW && g.KH == 3) { if (unit) LNN_DW_LAUNCH(3, true); else LNN_DW_LAUNCH(3, false); }
+  else if (g.KH == g.KW && g.KH == 5) { if (unit) LNN_DW_LAUNCH(5, true); else LNN_DW_LAUNCH(5, false); }
+  else if (g.KH == g.KW && g.KH == 1) { if (unit) LNN_DW_LAUNCH(1, true); else LNN_DW_LAUNCH(1, false); }
+  else LNN_DW_LAUNCH(0, false);
 #undef LNN_DW_LAUNCH
   LNN_HIP(hipGetLastError());
   return LNN_OK;
@@ -412,15 +565,16 @@ int launch_dw_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, c
   if (g.KH * g.KW > kDwMaxTaps) return set_error(LNN_ERR_UNSUPPORTED, "depthwise_conv2d: more than 1024 taps");
   const dim3 grid((unsigned)(g.N * g.C * bands)), block(256);
   const int b = beta ? 1 : 0;
-#define LNN_DW_LAUNCH(KS)                                                                                    \
+#define LNN_DW_LAUNCH(KS, UNIT)                                                                                    \
   do {                                                                                                       \
-    if (small) hipLaunchKernelGGL((dw_dgrad_kernel<KS, kDwSmall>), grid, block, 0, ctx->stream, g, dY, K, dX, bands, TH, b); \
-    else hipLaunchKernelGGL((dw_dgrad_kernel<KS, kDwLarge>), grid, block, 0, ctx->stream, g, dY, K, dX, bands, TH, b);       \
+    if (small) hipLaunchKernelGGL((dw_dgrad_kernel<KS, kDwSmall, UNIT>), grid, block, 0, ctx->stream, g, dY, K, dX, bands, TH, b); \
+    else hipLaunchKernelGGL((dw_dgrad_kernel<KS, kDwLarge, UNIT>), grid, block, 0, ctx->stream, g, dY, K, dX, bands, TH, b);       \
   } while (0)
-  if (g.KH == g.KW && g.KH == 3) LNN_DW_LAUNCH(3);
-  else if (g.KH == g.KW && g.KH == 5) LNN_DW_LAUNCH(5);
-  else if (g.KH == g.KW && g.KH == 1) LNN_DW_LAUNCH(1);
-  else LNN_DW_LAUNCH(0);
+  const bool unit = g.S == 1 && g.D == 1;   // sliding-window kernels
+  if (g.KH == g.KW && g.KH == 3) { if (unit) LNN_DW_LAUNCH(3, true); else LNN_DW_LAUNCH(3, false); }
+  else if (g.KH == g.KW && g.KH == 5) { if (unit) LNN_DW_LAUNCH(5, true); else LNN_DW_LAUNCH(5, false); }
+  else if (g.KH == g.KW && g.KH == 1) { if (unit) LNN_DW_LAUNCH(1, true); else LNN_DW_LAUNCH(1, false); }
+  else LNN_DW_LAUNCH(0, false);
 #undef LNN_DW_LAUNCH
   LNN_HIP(hipGetLastError());
   return LNN_OK;
@@ -432,6 +586,36 @@ int launch_dw_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   if (st != LNN_OK) return st;
   if (!X || !dY || !dK) return set_error(LNN_ERR_INVALID, "depthwise_conv2d_wgrad: null pointer");
   const int KK = g.KH * g.KW;
+  // Whole planes twice in LDS (at most 64 KB): the pipelined kernel, one reduction per block
+  const int xf = (g.IH * g.IW + 255) / 256 * 256, yf = (g.OH * g.OW + 255) / 256 * 256, stage = xf + yf;
+  const bool square = g.KH == g.KW && (g.KH == 1 || g.KH == 3 || g.KH == 5);
+  if (square && (long long)g.IH * g.IW <= 8192 && (long long)g.OH * g.OW <= 8192 && 2 * stage * 4 <= 65536) {
+    // as many blocks as the LDS holds at once (160 KB per compute unit), each walking several planes
+    int per_cu = 160 * 1024 / (2 * stage * 4);
+    per_cu = per_cu > 8 ? 8 : per_cu;
+    int slices = (per_cu * ctx->cus + g.C - 1) / g.C;
+    slices = slices > g.N ? g.N : slices;
+    st = ensure_workspace(ctx, (size_t)slices * g.C * KK * sizeof(float));
+    if (st != LNN_OK) return st;
+    float* part = static_cast<float*>(ctx->ws);
+    const dim3 grid((unsigned)(g.C * slices)), block(256);
+    const size_t lds_bytes = (size_t)2 * stage * sizeof(float);
+    const bool unit = g.S == 1 && g.D == 1;
+#define LNN_DW_LAUNCH(KS)                                                                                          \
+  do {                                                                                                             \
+    if (unit) hipLaunchKernelGGL((dw_wgrad_planes_kernel<KS, true>), grid, block, lds_bytes, ctx->stream, g, X, dY, part, slices, stage, xf); \
+    else hipLaunchKernelGGL((dw_wgrad_planes_kernel<KS, false>), grid, block, lds_bytes, ctx->stream, g, X, dY, part, slices, stage, xf);    \
+  } while (0)
+    if (g.KH == 3) LNN_DW_LAUNCH(3);
+    else if (g.KH == 5) LNN_DW_LAUNCH(5);
+    else LNN_DW_LAUNCH(1);
+#undef LNN_DW_LAUNCH
+    LNN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(dw_wgrad_finish_kernel, dim3((unsigned)g.C), dim3(256), 0, ctx->stream, dK, part, g.C, KK, slices, 1,
+                       beta ? 1 : 0);
+    LNN_HIP(hipGetLastError());
+    return LNN_OK;
+  }
   auto rows = [&](int xfloats, int yfloats) {
     int th = dw_band_rows(g.OH, g.IW, g.S, 1, (long long)(g.KH - 1) * g.D, xfloats);
     while (th >= 1 && (long long)th * g.OW > yfloats) --th;
@@ -448,15 +632,16 @@ int launch_dw_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   if (st != LNN_OK) return st;
   const dim3 grid((unsigned)(g.N * g.C * bands)), block(256);
   float* part = static_cast<float*>(ctx->ws);
-#define LNN_DW_LAUNCH(KS)                                                                                      \
+#define LNN_DW_LAUNCH(KS, UNIT)                                                                                      \
   do {                                                                                                         \
-    if (small) hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwSmall, kDwSmall>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
-    else hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwWgradX, kDwWgradY>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
+    if (small) hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwSmall, kDwSmall, UNIT>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
+    else hipLaunchKernelGGL((dw_wgrad_kernel<KS, kDwWgradX, kDwWgradY, UNIT>), grid, block, 0, ctx->stream, g, X, dY, part, bands, TH); \
   } while (0)
-  if (g.KH == g.KW && g.KH == 3) LNN_DW_LAUNCH(3);
-  else if (g.KH == g.KW && g.KH == 5) LNN_DW_LAUNCH(5);
-  else if (g.KH == g.KW && g.KH == 1) LNN_DW_LAUNCH(1);
-  else LNN_DW_LAUNCH(0);
+  const bool unit = g.S == 1 && g.D == 1;   // sliding-window kernels
+  if (g.KH == g.KW && g.KH == 3) { if (unit) LNN_DW_LAUNCH(3, true); else LNN_DW_LAUNCH(3, false); }
+  else if (g.KH == g.KW && g.KH == 5) { if (unit) LNN_DW_LAUNCH(5, true); else LNN_DW_LAUNCH(5, false); }
+  else if (g.KH == g.KW && g.KH == 1) { if (unit) LNN_DW_LAUNCH(1, true); else LNN_DW_LAUNCH(1, false); }
+  else LNN_DW_LAUNCH(0, false);
 #undef LNN_DW_LAUNCH
   LNN_HIP(hipGetLastError());
   hipLaunchKernelGGL(dw_wgrad_finish_kernel, dim3((unsigned)g.C), dim3(256), 0, ctx->stream, dK,
