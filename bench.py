@@ -103,6 +103,20 @@ def rel_err(got, ref):
     return float(np.abs(np.asarray(got, np.float64) - ref).max() / max(np.abs(ref).max(), 1e-30))
 
 
+SETTLE_S = 0.25
+
+
+def settle(step, sync):
+    """Untimed: repeat the step for about SETTLE_S seconds before the warm-up steps.  An idle MI355X needs some
+    20-30 ms of sustained load to leave its low-power clocks (the first kernels of a process run ~25 % longer than
+    the same kernels a few dozen launches later); a 5-step warm-up of sub-millisecond steps ends inside that ramp."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < SETTLE_S:
+        for _ in range(10):
+            step()
+        sync()
+
+
 def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
     xs, ws, s, d, padding, seed = CONV_CONFIGS[name]
     x, w, dy, ci = conv_tensors(xs, ws, s, d, padding, seed)
@@ -124,6 +138,7 @@ def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
         for fn in passes.values():
             fn()
 
+    settle(step, lambda: api.synchronize(0))
     for _ in range(warmup):
         step()
     api.synchronize(0)
@@ -158,7 +173,7 @@ def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
     got = (Y.get(), dX.get(), dW.get())
     result = {
         'metric': 'conv2D fwd+bwd fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
-        'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True,
+        'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
         'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
         'config': {'workload': f'{name}: x{list(xs)} w{list(ws)} stride {s} dilation {d} padding {padding!r}, '
                                'step = fwd + dX(+=) + dW(+=)'},
@@ -208,6 +223,7 @@ def bench_matmul(api, steps, warmup, n=4096, cpu=True):
         for fn in passes.values():
             fn()
 
+    settle(step, lambda: api.synchronize(0))
     for _ in range(warmup):
         step()
     api.synchronize(0)
@@ -225,7 +241,7 @@ def bench_matmul(api, steps, warmup, n=4096, cpu=True):
     dB.zero()
     step()
     res = {'metric': 'matmul fwd+dA+dB fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
-           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True,
+           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
            'config': {'workload': f'cfg2_matmul: [{n}x{n}] @ [{n}x{n}], step = C + dA(+=) + dB(+=)'},
            'roofline': {'bound': 'mfma', 'kernel': dom, 'achieved': per_pass[dom]['tflops'],
@@ -288,6 +304,7 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
         for fn in passes.values():
             fn()
 
+    settle(step, lambda: api.synchronize(0))
     for _ in range(warmup):
         step()
     api.synchronize(0)
@@ -305,7 +322,7 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
     dK.zero()
     step()
     res = {'metric': 'conv2DTranspose fwd+bwd fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
-           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True,
+           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
            'config': {'workload': f'cfgT_decoder: conv2DTranspose x[{N}, {IC}, {IH}, {IW}] k[{OC}, {IC}, {KS}, {KS}] '
                                   f"stride {S} 'same', step = fwd + dI(+=) + dK(+=)"},
@@ -352,6 +369,7 @@ def bench_depthwise(api, steps, warmup, cpu=True):
         for fn in passes.values():
             fn()
 
+    settle(step, lambda: api.synchronize(0))
     for _ in range(warmup):
         step()
     api.synchronize(0)
@@ -371,7 +389,7 @@ def bench_depthwise(api, steps, warmup, cpu=True):
     step()
     total_bytes = sum(bytes_pass.values())
     res = {'metric': 'depthwise_conv2D fwd+bwd algorithmic GB/s', 'value': total_bytes / wall_ms / 1e6, 'unit': 'GB/s',
-           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True,
+           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
            'config': {'workload': f"cfgD_depthwise: x[{N}, {C}, {H}, {H}] k[{C}, {KS}, {KS}] stride 1 'same', "
                                   'step = fwd + dX(+=) + dK(+=)'},
@@ -431,6 +449,7 @@ def bench_encoder(steps, warmup):
         opt.step()
         return loss
 
+    settle(step, nn.devices.wait)
     for _ in range(warmup):
         step()
     nn.devices.wait()
@@ -441,7 +460,7 @@ def bench_encoder(steps, warmup):
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     flops = 61.66e9
     res = {'metric': 'encoder training step images/s', 'value': 16 / wall_ms * 1e3, 'unit': 'images/s', 'n_gpus': 1,
-           'steps': steps, 'warmup': warmup, 'ms_per_step': wall_ms, 'higher_is_better': True, 'scaling': 'weak',
+           'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True, 'scaling': 'weak',
            'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
            'config': {'workload': 'cfg5_encoder: 16x3x128x128, 3->64->128->256->512, 5x5 s2 p2, leaky_relu(0.1), '
                                   'loss mean(square), SGD lr 1e-3; forward + backward + update'},
@@ -453,8 +472,8 @@ def bench_encoder(steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=20)
-    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--all', action='store_true', help='also measure every benchmark configuration')
     ap.add_argument('--out-dir', default='.', help='where --all writes bench_all.jsonl')
