@@ -160,9 +160,10 @@ enum {
 };
 /* out (+)= f(in) */
 int lnn_ew_fwd_f32(int dev, int op, uint64_t n, const float* in, float* out, float p0, int beta);
-/* din += f'(in, out_fwd) * dout     (always accumulates, element_wise_op.py:108) */
+/* din (+)= f'(in) * dout.  The reference always accumulates (element_wise_op.py:108) into a gradient that
+ * starts as zeros; beta = 0 is that first contribution without the zero fill and the read. */
 int lnn_ew_bwd_f32(int dev, int op, uint64_t n, const float* in, const float* dout, float* din,
-                   float p0);
+                   float p0, int beta);
 /* out (+)= a (op) b with numpy broadcasting; shapes already left-padded with
  * ones to `rank` <= 8 (dual_wise_op.py:138-152).  op: 0 add, 1 sub, 2 mul. */
 int lnn_binary_bcast_f32(int dev, int op, int rank, const int32_t* out_shape,
@@ -172,9 +173,9 @@ int lnn_binary_bcast_f32(int dev, int op, int rank, const int32_t* out_shape,
  * set = axis i is summed.  rank <= 8. */
 int lnn_reduce_sum_f32(int dev, int rank, const int32_t* shape, uint32_t reduce_mask,
                        float scale, const float* in, float* out, int beta);
-/* din[idx] += scale * dout[idx with reduced axes set to 0]   (reduce.py:243-255) */
+/* din[idx] (+)= scale * dout[idx with reduced axes set to 0]   (reduce.py:243-255; beta as above) */
 int lnn_reduce_sum_bwd_f32(int dev, int rank, const int32_t* shape, uint32_t reduce_mask,
-                           float scale, const float* dout, float* din);
+                           float scale, const float* dout, float* din, int beta);
 /* SGD.py:42-74: acc = momentum*acc - lr*g;  v += nesterov ? momentum*acc - lr*g : acc */
 int lnn_sgd_update_f32(int dev, uint64_t n, float* v, const float* g, float* acc, float momentum,
                        float lr, int nesterov);

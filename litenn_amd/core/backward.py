@@ -1,5 +1,7 @@
 import operator
 
+import numpy as np
+
 import litenn_amd as nn
 import litenn_amd.core as nc
 
@@ -37,8 +39,14 @@ def backward(loss, stop_grad=None, grad_for_non_trainables=False, keep_gradient_
     roots = [t for t in loss if t._get_seq_id() not in blocked]
     for t in roots:
         g = t.get_grad()
+        fresh = all(not b.has_ptr() for b in g._get_buffers())   # still the implicit zeros: the seed may overwrite
         if t in seeds:
-            nc.op.add(g, nn.Tensor_from_value(seeds[t]), output_t=g)
+            if fresh and isinstance(seeds[t], np.ndarray) and seeds[t].size == g.shape.size:
+                g.set(seeds[t])
+            else:
+                nc.op.add(g, nn.Tensor_from_value(seeds[t]), output_t=g)
+        elif fresh:
+            g.fill(1.0)
         else:
             nc.op.add_const(g, 1.0, output_t=g)
 

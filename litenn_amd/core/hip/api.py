@@ -73,10 +73,10 @@ SIGNATURES = {
     'lnn_unfold2d_f32': [_c_int] + [_c_int] * 14 + [_ptr, _ptr, _c_int],
     'lnn_transpose_f32': [_c_int, _c_int, _i32arr, _i32arr, _ptr, _ptr, _c_int],
     'lnn_ew_fwd_f32': [_c_int, _c_int, _c_u64, _ptr, _ptr, _c_f32, _c_int],
-    'lnn_ew_bwd_f32': [_c_int, _c_int, _c_u64, _ptr, _ptr, _ptr, _c_f32],
+    'lnn_ew_bwd_f32': [_c_int, _c_int, _c_u64, _ptr, _ptr, _ptr, _c_f32, _c_int],
     'lnn_binary_bcast_f32': [_c_int, _c_int, _c_int, _i32arr, _i32arr, _i32arr, _ptr, _ptr, _ptr, _c_int],
     'lnn_reduce_sum_f32': [_c_int, _c_int, _i32arr, _c_u32, _c_f32, _ptr, _ptr, _c_int],
-    'lnn_reduce_sum_bwd_f32': [_c_int, _c_int, _i32arr, _c_u32, _c_f32, _ptr, _ptr],
+    'lnn_reduce_sum_bwd_f32': [_c_int, _c_int, _i32arr, _c_u32, _c_f32, _ptr, _ptr, _c_int],
     'lnn_sgd_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int],
     'lnn_adam_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32],
     'lnn_bias_act_bwd_f32': [_c_int, _c_int, _c_int, _c_int, _ptr, _ptr, _c_int, _c_f32, _ptr, _ptr, _c_int],
@@ -248,8 +248,8 @@ def ew_fwd(dev, op, n, src, dst, p0=0.0, beta=0):
     check(lib.lnn_ew_fwd_f32(dev, op, n, src, dst, float(p0), int(beta)))
 
 
-def ew_bwd(dev, op, n, src, dout, din, p0=0.0):
-    check(lib.lnn_ew_bwd_f32(dev, op, n, src, dout, din, float(p0)))
+def ew_bwd(dev, op, n, src, dout, din, p0=0.0, beta=1):
+    check(lib.lnn_ew_bwd_f32(dev, op, n, src, dout, din, float(p0), beta))
 
 
 def binary_bcast(dev, op, out_shape, a_shape, b_shape, a, b, out, beta=0):
@@ -268,8 +268,8 @@ def reduce_sum(dev, shape, axes, scale, src, dst, beta=0):
     check(lib.lnn_reduce_sum_f32(dev, len(shape), _ints(shape), _mask(axes), float(scale), src, dst, int(beta)))
 
 
-def reduce_sum_bwd(dev, shape, axes, scale, dout, din):
-    check(lib.lnn_reduce_sum_bwd_f32(dev, len(shape), _ints(shape), _mask(axes), float(scale), dout, din))
+def reduce_sum_bwd(dev, shape, axes, scale, dout, din, beta=1):
+    check(lib.lnn_reduce_sum_bwd_f32(dev, len(shape), _ints(shape), _mask(axes), float(scale), dout, din, beta))
 
 
 def sgd_update(dev, n, v, g, acc, momentum, lr, nesterov):

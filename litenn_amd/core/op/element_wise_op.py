@@ -36,7 +36,8 @@ def element_wise_op(kind, param, input_t, output_t=None, is_add_to_output=False)
 
 def _input_gradfn(code, param, input_t, dO_t):
     n = input_t.shape.size
-    launch(lambda dev, i, do, di: api.ew_bwd(dev, code, n, i, do, di, param), input_t, dO_t, input_t.get_grad())
+    grad_t, beta = nc.op.accumulate_target(input_t.get_grad())
+    launch(lambda dev, i, do, di: api.ew_bwd(dev, code, n, i, do, di, param, beta), input_t, dO_t, grad_t)
 
 
 def add_const_op(input_t, value, output_t=None, is_add_to_output=False):

@@ -26,7 +26,8 @@ def reduce_op(op_type, input_t, axes=None, keepdims=False, output_t=None, is_add
 
 def reduce_dI_gradfn(op, input_t, O_t, dO_t):
     # in.grad[idx] += dO[idx with reduced axes dropped] (/ count for mean)   (reduce.py:243-255)
-    launch(lambda dev, do, di: api.reduce_sum_bwd(dev, op.shape, op.axes, op.scale, do, di), dO_t, input_t.get_grad())
+    grad_t, beta = nc.op.accumulate_target(input_t.get_grad())
+    launch(lambda dev, do, di: api.reduce_sum_bwd(dev, op.shape, op.axes, op.scale, do, di, beta), dO_t, grad_t)
 
 
 class _ReduceOp:

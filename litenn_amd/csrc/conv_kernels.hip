@@ -101,7 +101,7 @@ struct ReduceArgs {
   OutMap om;
   PostOp post;
 };
-__global__ __launch_bounds__(256) void reduce_partials(float* out, const float* part, ReduceArgs a) {
+__device__ __forceinline__ void reduce_body(float* out, const float* part, const ReduceArgs& a) {
   __shared__ float red[8][33];
   const int li = threadIdx.x & 31, ls = threadIdx.x >> 5;
   const int i = blockIdx.x * 32 + li;
@@ -124,10 +124,13 @@ __global__ __launch_bounds__(256) void reduce_partials(float* out, const float* 
     out[o] = a.beta ? out[o] + s : s;
   }
 }
+__global__ __launch_bounds__(256) void reduce_partials(float* out, const float* part, ReduceArgs a) {
+  reduce_body(out, part, a);
+}
 
 // The same for ncols % 4 == 0 with 128-bit reads: a block covers 128 consecutive
 // elements, 8 lanes per group of 4 striding over the slices.
-__global__ __launch_bounds__(256) void reduce_partials4(float* out, const float* part, ReduceArgs a) {
+__device__ __forceinline__ void reduce_body4(float* out, const float* part, const ReduceArgs& a) {
   __shared__ float red[8][128];
   const int q = threadIdx.x & 31, ls = threadIdx.x >> 5;
   const int i4 = (blockIdx.x * 32 + q) * 4;
@@ -151,6 +154,25 @@ __global__ __launch_bounds__(256) void reduce_partials4(float* out, const float*
     out[o] = a.beta ? out[o] + t : t;
   }
 }
+__global__ __launch_bounds__(256) void reduce_partials4(float* out, const float* part, ReduceArgs a) {
+  reduce_body4(out, part, a);
+}
+
+// The reductions of the pixel classes of one strided dgrad in one launch: blockIdx.y = class.
+constexpr int kMaxReduceBatch = 4;
+struct ReduceBatch {
+  ReduceArgs r[kMaxReduceBatch];
+  float* out[kMaxReduceBatch];
+  const float* part[kMaxReduceBatch];
+  int vec[kMaxReduceBatch];
+};
+__global__ __launch_bounds__(256) void reduce_partials_batch(ReduceBatch b) {
+  const int c = blockIdx.y;
+  const int per_block = b.vec[c] ? 128 : 32;
+  if ((long long)blockIdx.x * per_block >= b.r[c].n) return;   // the whole block leaves together
+  if (b.vec[c]) reduce_body4(b.out[c], b.part[c], b.r[c]);
+  else reduce_body(b.out[c], b.part[c], b.r[c]);
+}
 
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
 enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5 };
@@ -158,8 +180,8 @@ enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRA
 // Wp[a][tap][b] = W[..] so that the tap-major K index tap*CH + ch is contiguous:
 //   mode 0 (forward): Wp[o][tap][c] = W[o][c][tap]
 //   mode 1 (dgrad):   Wp[c][t][o] = W[o][c][tap_t], t over the taps of the pixel class
-__global__ void permute_weights(float* wp, const float* w, int O, int C, int KK, int mode, ConvGeom g, PixelClass pc) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void permute_one(float* wp, const float* w, int O, int C, int KK, int mode, const ConvGeom& g,
+                                            const PixelClass& pc, int i) {
   if (mode == 0) {
     if (i >= O * C * KK) return;
     const int b = i % C, tap = (i / C) % KK, a = i / (C * KK);
@@ -172,6 +194,17 @@ __global__ void permute_weights(float* wp, const float* w, int O, int C, int KK,
     const int tap = nth_tap(g.KH, g.D, g.S, pc.rh, jh) * g.KW + nth_tap(g.KW, g.D, g.S, pc.rw, jw);
     wp[i] = w[((size_t)b * C + a) * KK + tap];
   }
+}
+__global__ void permute_weights(float* wp, const float* w, int O, int C, int KK, int mode, ConvGeom g, PixelClass pc) {
+  permute_one(wp, w, O, C, KK, mode, g, pc, blockIdx.x * blockDim.x + threadIdx.x);
+}
+// mode 1 for up to four pixel classes at once: blockIdx.y = class
+struct PermuteBatch {
+  float* wp[4];
+  PixelClass pc[4];
+};
+__global__ void permute_weights_classes(PermuteBatch b, const float* w, int O, int C, int KK, ConvGeom g) {
+  permute_one(b.wp[blockIdx.y], w, O, C, KK, 1, g, b.pc[blockIdx.y], blockIdx.x * blockDim.x + threadIdx.x);
 }
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
@@ -424,7 +457,7 @@ static int permuted_weights(DeviceCtx* ctx, const ConvGeom& g, const float* W, i
 
 // Slice reduction of a split-K problem into its final tensor.
 template <int PASS, int WM>
-static int launch_reduce(DeviceCtx* ctx, const ConvArgs& a, float* final_out, int final_beta) {
+static ReduceArgs reduce_args(const ConvArgs& a, int final_beta) {
   constexpr int WN = 4 / WM;
   ReduceArgs r;
   r.n = a.M * a.Ncols; r.slices = a.ksplit; r.slices_last = a.ksplit; r.beta = final_beta; r.ncols = a.Ncols;
@@ -438,6 +471,12 @@ static int launch_reduce(DeviceCtx* ctx, const ConvArgs& a, float* final_out, in
   r.dN = make_fastdiv((uint32_t)a.Ncols);
   r.om = final_map<PASS>(a);
   r.post = a.post;
+  return r;
+}
+
+template <int PASS, int WM>
+static int launch_reduce(DeviceCtx* ctx, const ConvArgs& a, float* final_out, int final_beta) {
+  const ReduceArgs r = reduce_args<PASS, WM>(a, final_beta);
   if (a.Ncols % 4 == 0)   // partial buffers start 256-byte aligned
     hipLaunchKernelGGL(reduce_partials4, dim3((r.n + 127) / 128), dim3(256), 0, ctx->stream, final_out,
                        static_cast<const float*>(a.Out), r);
@@ -600,11 +639,28 @@ static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_
     hipLaunchKernelGGL((conv_kernel_batch<PASS, WM, NTMAX>), dim3(gx, gy, nb), dim3(512, 1, 1), 0, ctx->stream, b);
     LNN_HIP(hipGetLastError());
   }
+  // the K-split classes' reductions, kMaxReduceBatch per launch
+  ReduceBatch rb;
+  int nr = 0;
+  unsigned gx = 1;
+  auto flush = [&]() {
+    if (nr == 0) return;
+    hipLaunchKernelGGL(reduce_partials_batch, dim3(gx, nr), dim3(256), 0, ctx->stream, rb);
+    nr = 0;
+    gx = 1;
+  };
   for (int i = 0; i < n; ++i)
     if (cls[i].ksplit > 1) {
-      int st = launch_reduce<PASS, WM>(ctx, cls[i], final_out[i], final_beta[i]);
-      if (st != LNN_OK) return st;
+      rb.r[nr] = reduce_args<PASS, WM>(cls[i], final_beta[i]);
+      rb.out[nr] = final_out[i];
+      rb.part[nr] = cls[i].Out;
+      rb.vec[nr] = cls[i].Ncols % 4 == 0;
+      const unsigned blocks = (unsigned)((rb.r[nr].n + (rb.vec[nr] ? 127 : 31)) / (rb.vec[nr] ? 128 : 32));
+      gx = blocks > gx ? blocks : gx;
+      if (++nr == kMaxReduceBatch) flush();
     }
+  flush();
+  LNN_HIP(hipGetLastError());
   return LNN_OK;
 }
 
@@ -737,18 +793,26 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   }
   st = ensure_workspace(ctx, w_bytes + part_bytes);
   if (st != LNN_OK) return st;
-  if (tap)
-    for (int i = 0; i < nc; ++i) {
-      ConvArgs& a = cls[i];
-      float* wp = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + w_off[i]);
-      const int n = full.O * full.C * pcs[i].nkh * pcs[i].nkw;
-      if (n > 0) {
-        hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, wp, W, full.O, full.C,
-                           full.KK, 1, full, pcs[i]);
-        LNN_HIP(hipGetLastError());
+  if (tap) {
+    // every class's weights in one launch (nc <= kMaxBatch <= 4 here)
+    PermuteBatch pb;
+    int most = 0;
+    for (int i = 0; i < 4; ++i) {
+      const int j = i < nc ? i : 0;
+      pb.wp[i] = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + w_off[j]);
+      pb.pc[i] = pcs[j];
+      if (i < nc) {
+        const int n = full.O * full.C * pcs[i].nkh * pcs[i].nkw;
+        most = n > most ? n : most;
+        cls[i].W = pb.wp[i];
       }
-      a.W = wp;
     }
+    if (most > 0) {
+      hipLaunchKernelGGL(permute_weights_classes, dim3((most + 255) / 256, nc), dim3(256), 0, ctx->stream, pb, W, full.O,
+                         full.C, full.KK, full);
+      LNN_HIP(hipGetLastError());
+    }
+  }
   return tap ? launch_classes_by_m<PASS_DGRAD_TAP>(ctx, cls, w_bytes) : launch_classes_by_m<PASS_DGRAD>(ctx, cls, w_bytes);
 }
 

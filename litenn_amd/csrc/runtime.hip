@@ -7,11 +7,11 @@ namespace lnn {
 
 int launch_fill_u32(DeviceCtx*, void*, uint32_t, uint64_t);
 int launch_ew_fwd(DeviceCtx*, int, uint64_t, const float*, float*, float, int);
-int launch_ew_bwd(DeviceCtx*, int, uint64_t, const float*, const float*, float*, float);
+int launch_ew_bwd(DeviceCtx*, int, uint64_t, const float*, const float*, float*, float, int);
 int launch_binary_bcast(DeviceCtx*, int, int, const int32_t*, const int32_t*, const int32_t*, const float*,
                         const float*, float*, int);
 int launch_reduce_sum(DeviceCtx*, int, const int32_t*, uint32_t, float, const float*, float*, int);
-int launch_reduce_sum_bwd(DeviceCtx*, int, const int32_t*, uint32_t, float, const float*, float*);
+int launch_reduce_sum_bwd(DeviceCtx*, int, const int32_t*, uint32_t, float, const float*, float*, int);
 int launch_transpose(DeviceCtx*, int, const int32_t*, const int32_t*, const float*, float*, int);
 int launch_unfold2d(DeviceCtx*, int, int, int, int, int, int, int, int, int, int, int, int, int, int, const float*,
                     float*, int);
@@ -344,12 +344,12 @@ int lnn_ew_fwd_f32(int dev, int op, uint64_t n, const float* in, float* out, flo
   return launch_ew_fwd(ctx, op, n, in, out, p0, beta);
 }
 
-int lnn_ew_bwd_f32(int dev, int op, uint64_t n, const float* in, const float* dout, float* din, float p0) {
+int lnn_ew_bwd_f32(int dev, int op, uint64_t n, const float* in, const float* dout, float* din, float p0, int beta) {
   if (n && (!in || !dout || !din)) return set_error(LNN_ERR_INVALID, "ew_bwd: null pointer");
   int st = check_count(n, "ew_bwd");
   if (st != LNN_OK) return st;
   CTX(dev);
-  return launch_ew_bwd(ctx, op, n, in, dout, din, p0);
+  return launch_ew_bwd(ctx, op, n, in, dout, din, p0, beta);
 }
 
 int lnn_binary_bcast_f32(int dev, int op, int rank, const int32_t* out_shape, const int32_t* a_shape,
@@ -367,10 +367,10 @@ int lnn_reduce_sum_f32(int dev, int rank, const int32_t* shape, uint32_t reduce_
 }
 
 int lnn_reduce_sum_bwd_f32(int dev, int rank, const int32_t* shape, uint32_t reduce_mask, float scale,
-                           const float* dout, float* din) {
+                           const float* dout, float* din, int beta) {
   if (!shape || !dout || !din) return set_error(LNN_ERR_INVALID, "reduce_sum_bwd: null pointer");
   CTX(dev);
-  return launch_reduce_sum_bwd(ctx, rank, shape, reduce_mask, scale, dout, din);
+  return launch_reduce_sum_bwd(ctx, rank, shape, reduce_mask, scale, dout, din, beta);
 }
 
 int lnn_sgd_update_f32(int dev, uint64_t n, float* v, const float* g, float* acc, float momentum, float lr,

@@ -54,9 +54,11 @@ __global__ void ew_fwd_kernel(int op, uint64_t n, const float* in, float* out, f
   }
 }
 
-__global__ void ew_bwd_kernel(int op, uint64_t n, const float* in, const float* dout, float* din, float p0) {
-  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x)
-    din[i] += dout[i] * ew_df(op, in[i], p0);
+__global__ void ew_bwd_kernel(int op, uint64_t n, const float* in, const float* dout, float* din, float p0, int beta) {
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const float g = dout[i] * ew_df(op, in[i], p0);
+    din[i] = beta ? din[i] + g : g;
+  }
 }
 
 __global__ void binary_bcast_kernel(int op, Dims d, uint64_t n, const float* a, const float* b, float* out, int beta) {
@@ -121,17 +123,22 @@ __global__ void reduce_sum_kernel(RedPlan p, const float* in, float* dst, int pa
   }
 }
 
-__global__ void reduce_finish_kernel(const float* part, float* out, uint64_t outs, int parts, float scale, int beta) {
-  const uint64_t o = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x;
-  if (o >= outs) return;
+// one wavefront per output: lane l adds parts l, l + 64, ..., then a butterfly (fixed order)
+__global__ __launch_bounds__(64) void reduce_finish_kernel(const float* part, float* out, uint64_t outs, int parts,
+                                                           float scale, int beta) {
+  const uint64_t o = blockIdx.x;
   float s = 0.0f;
-  for (int k = 0; k < parts; ++k) s += part[o * parts + k];
-  s *= scale;
-  out[o] = beta ? out[o] + s : s;
+  for (int k = threadIdx.x; k < parts; k += 64) s += part[o * parts + k];
+#pragma unroll
+  for (int w = 32; w > 0; w >>= 1) s += __shfl_xor(s, w, 64);
+  if (threadIdx.x == 0) {
+    s *= scale;
+    out[o] = beta ? out[o] + s : s;
+  }
 }
 
-// din[idx] += scale * dout[kept part of idx]
-__global__ void reduce_bwd_kernel(Dims d, uint64_t n, float scale, const float* dout, float* din) {
+// din[idx] (+)= scale * dout[kept part of idx]
+__global__ void reduce_bwd_kernel(Dims d, uint64_t n, float scale, const float* dout, float* din, int beta) {
   for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     uint32_t g = (uint32_t)i;
     long long oa = 0;
@@ -140,7 +147,8 @@ __global__ void reduce_bwd_kernel(Dims d, uint64_t n, float scale, const float* 
       g /= (uint32_t)d.shape[ax];
       oa += (long long)x * d.sa[ax];
     }
-    din[i] += scale * dout[oa];
+    const float v = scale * dout[oa];
+    din[i] = beta ? din[i] + v : v;
   }
 }
 
@@ -240,10 +248,11 @@ int launch_ew_fwd(DeviceCtx* ctx, int op, uint64_t n, const float* in, float* ou
   return LNN_OK;
 }
 
-int launch_ew_bwd(DeviceCtx* ctx, int op, uint64_t n, const float* in, const float* dout, float* din, float p0) {
+int launch_ew_bwd(DeviceCtx* ctx, int op, uint64_t n, const float* in, const float* dout, float* din, float p0,
+                  int beta) {
   if (op < 0 || op > LNN_EW_RELU) return set_error(LNN_ERR_INVALID, "ew_bwd: unknown op");
   if (n == 0) return LNN_OK;
-  hipLaunchKernelGGL(ew_bwd_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, op, n, in, dout, din, p0);
+  hipLaunchKernelGGL(ew_bwd_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, op, n, in, dout, din, p0, beta ? 1 : 0);
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }
@@ -324,7 +333,7 @@ int launch_reduce_sum(DeviceCtx* ctx, int rank, const int32_t* shape, uint32_t m
                      scale, beta ? 1 : 0);
   LNN_HIP(hipGetLastError());
   if (parts > 1) {
-    hipLaunchKernelGGL(reduce_finish_kernel, dim3((unsigned)((p.outs + 255) / 256)), dim3(256), 0, ctx->stream,
+    hipLaunchKernelGGL(reduce_finish_kernel, dim3((unsigned)p.outs), dim3(64), 0, ctx->stream,
                        static_cast<const float*>(dst), out, p.outs, parts, scale, beta ? 1 : 0);
     LNN_HIP(hipGetLastError());
   }
@@ -332,7 +341,7 @@ int launch_reduce_sum(DeviceCtx* ctx, int rank, const int32_t* shape, uint32_t m
 }
 
 int launch_reduce_sum_bwd(DeviceCtx* ctx, int rank, const int32_t* shape, uint32_t mask, float scale,
-                          const float* dout, float* din) {
+                          const float* dout, float* din, int beta) {
   int st = check_rank(rank, shape, "reduce_sum_bwd");
   if (st != LNN_OK) return st;
   Dims d;
@@ -347,7 +356,7 @@ int launch_reduce_sum_bwd(DeviceCtx* ctx, int rank, const int32_t* shape, uint32
     if (!red) c *= shape[ax];
     n *= (uint64_t)shape[ax];
   }
-  hipLaunchKernelGGL(reduce_bwd_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, d, n, scale, dout, din);
+  hipLaunchKernelGGL(reduce_bwd_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, d, n, scale, dout, din, beta ? 1 : 0);
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }

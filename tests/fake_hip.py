@@ -155,10 +155,10 @@ class FakeHip:
         x = self.f(src)[:n].astype(np.float64)
         self._put(self.f(dst)[:n], self._F[op](x, p0), beta)
 
-    def ew_bwd(self, dev, op, n, src, dout, din, p0=0.0):
+    def ew_bwd(self, dev, op, n, src, dout, din, p0=0.0, beta=1):
         self.launches += 1
         x = self.f(src)[:n].astype(np.float64)
-        self._put(self.f(din)[:n], self.f(dout)[:n].astype(np.float64) * self._DF[op](x, p0), 1)
+        self._put(self.f(din)[:n], self.f(dout)[:n].astype(np.float64) * self._DF[op](x, p0), beta)
 
     def binary_bcast(self, dev, op, out_shape, a_shape, b_shape, a, b, out, beta=0):
         self.launches += 1
@@ -172,11 +172,11 @@ class FakeHip:
         r = np.asarray(r).reshape(-1)
         self._put(self.f(dst)[:r.size], r, beta)
 
-    def reduce_sum_bwd(self, dev, shape, axes, scale, dout, din):
+    def reduce_sum_bwd(self, dev, shape, axes, scale, dout, din, beta=1):
         self.launches += 1
         kd = tuple(1 if i in axes else s for i, s in enumerate(shape))
         g = self.f(dout, kd).astype(np.float64) * scale
-        self._put(self.f(din, shape), np.broadcast_to(g, shape), 1)
+        self._put(self.f(din, shape), np.broadcast_to(g, shape), beta)
 
     def sgd_update(self, dev, n, v, g, acc, momentum, lr, nesterov):
         self.launches += 1
