@@ -184,6 +184,14 @@ int lnn_sgd_update_f32(int dev, uint64_t n, float* v, const float* g, float* acc
 int lnn_adam_update_f32(int dev, uint64_t n, float* t, const float* g, float* m, float* v,
                         float beta1, float beta2, float lr);
 
+/* The same two updates for `count` tensors in one launch (an optimizer step over a model's parameters,
+ * Optimizer.py:117-147 walks them one by one).  n, v/t, g, acc/m, v: host arrays of `count` element counts and
+ * device pointers; tensors with n[i] == 0 are skipped. */
+int lnn_sgd_update_multi_f32(int dev, int count, const uint64_t* n, float* const* v, const float* const* g,
+                             float* const* acc, float momentum, float lr, int nesterov);
+int lnn_adam_update_multi_f32(int dev, int count, const uint64_t* n, float* const* t, const float* const* g,
+                              float* const* m, float* const* v, float beta1, float beta2, float lr);
+
 /* On-device random initialisers: element i is drawn from a counter hash of (uint32)(i + seed), so a tensor
  * is filled in place without host staging (initializer/RandomUniform.py:13-27, RandomNormal.py:10-30; the PCG
  * hashes of CLKernelHelper.py:210-228).  The reference draws seed = np.random.randint(2^31) on the host.

@@ -79,6 +79,8 @@ SIGNATURES = {
     'lnn_reduce_sum_bwd_f32': [_c_int, _c_int, _i32arr, _c_u32, _c_f32, _ptr, _ptr, _c_int],
     'lnn_sgd_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int],
     'lnn_adam_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32],
+    'lnn_sgd_update_multi_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int],
+    'lnn_adam_update_multi_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32],
     'lnn_bias_act_bwd_f32': [_c_int, _c_int, _c_int, _c_int, _ptr, _ptr, _c_int, _c_f32, _ptr, _ptr, _c_int],
     'lnn_random_uniform_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
     'lnn_random_normal_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
@@ -290,3 +292,21 @@ def random_normal(dev, out, n, seed, mean, stddev):
 
 def bias_act_bwd(dev, N, O, HW, y, dy, act, slope, dpre, dbias, beta_bias):
     check(lib.lnn_bias_act_bwd_f32(dev, N, O, HW, y, dy, act, float(slope), dpre, dbias, beta_bias))
+
+
+def _ptr_array(ptrs):
+    return (ctypes.c_void_p * len(ptrs))(*ptrs)
+
+
+def sgd_update_multi(dev, ns, vs, gs, accs, momentum, lr, nesterov):
+    """One launch for the SGD update of len(ns) tensors."""
+    count = len(ns)
+    check(lib.lnn_sgd_update_multi_f32(dev, count, (ctypes.c_uint64 * count)(*ns), _ptr_array(vs), _ptr_array(gs),
+                                       _ptr_array(accs), float(momentum), float(lr), 1 if nesterov else 0))
+
+
+def adam_update_multi(dev, ns, ts, gs, ms, vs, beta1, beta2, lr):
+    """One launch for the Adam update of len(ns) tensors."""
+    count = len(ns)
+    check(lib.lnn_adam_update_multi_f32(dev, count, (ctypes.c_uint64 * count)(*ns), _ptr_array(ts), _ptr_array(gs),
+                                        _ptr_array(ms), _ptr_array(vs), float(beta1), float(beta2), float(lr)))

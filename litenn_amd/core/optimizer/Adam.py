@@ -19,9 +19,11 @@ class Adam(Optimizer):
 
     def _on_step(self):
         lr = self._current_lr()
-        for t in self.get_trainable_tensors():
-            if not t.has_grad():
-                continue
-            n = t.shape.size
-            launch(lambda dev, v, g, m, s: api.adam_update(dev, n, v, g, m, s, self.beta_1, self.beta_2, lr),
-                   t, t.get_grad(), self._ms[t.get_name()], self._vs[t.get_name()])
+        ts = [t for t in self.get_trainable_tensors() if t.has_grad()]
+        if not ts:
+            return
+        k, ns = len(ts), [t.shape.size for t in ts]
+        launch(lambda dev, *p: api.adam_update_multi(dev, ns, p[:k], p[k:2 * k], p[2 * k:3 * k], p[3 * k:],
+                                                     self.beta_1, self.beta_2, lr),
+               *ts, *[t.get_grad() for t in ts], *[self._ms[t.get_name()] for t in ts],
+               *[self._vs[t.get_name()] for t in ts])

@@ -7,7 +7,7 @@ class SGD(Optimizer):
     """Stochastic gradient descent (same constructor as optimizer/SGD.py:29):
       acc = momentum*acc - lr*g
       v  += nesterov ? momentum*acc - lr*g : acc          (SGD.py:52,68-72)
-    fused into one launch per tensor."""
+    fused into one launch for all tensors."""
 
     def __init__(self, tensors_list, momentum=0.0, nesterov=False, lr=0.001, lr_decay=0.0, lr_dropout=0.0,
                  clipnorm=0.0):
@@ -19,10 +19,10 @@ class SGD(Optimizer):
 
     def _on_step(self):
         lr = self._current_lr()
-        for t in self.get_trainable_tensors():
-            if not t.has_grad():
-                continue
-            acc_t = self._accs[t.get_name()]
-            n = t.shape.size
-            launch(lambda dev, v, g, a: api.sgd_update(dev, n, v, g, a, self.momentum, lr, self.nesterov),
-                   t, t.get_grad(), acc_t)
+        ts = [t for t in self.get_trainable_tensors() if t.has_grad()]
+        if not ts:
+            return
+        k, ns = len(ts), [t.shape.size for t in ts]
+        # every tensor's update in one launch per device: pointers arrive as (values, gradients, accumulators)
+        launch(lambda dev, *p: api.sgd_update_multi(dev, ns, p[:k], p[k:2 * k], p[2 * k:], self.momentum, lr, self.nesterov),
+               *ts, *[t.get_grad() for t in ts], *[self._accs[t.get_name()] for t in ts])

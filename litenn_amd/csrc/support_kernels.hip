@@ -229,6 +229,45 @@ __global__ void adam_kernel(uint64_t n, float* t, const float* g, float* m, floa
   }
 }
 
+// The optimizer step of up to kMultiMax tensors in one launch: blockIdx.y = tensor.  A model has a handful of
+// parameter tensors, most of them small, and one launch per tensor costs more than the update itself.
+constexpr int kMultiMax = 16;
+struct MultiArgs {
+  uint64_t n[kMultiMax];
+  float* t[kMultiMax];          // the parameter
+  const float* g[kMultiMax];    // its gradient
+  float* s0[kMultiMax];         // optimizer state (SGD: accumulator; Adam: m)
+  float* s1[kMultiMax];         // Adam: v
+};
+__global__ void sgd_multi_kernel(MultiArgs a, float momentum, float lr, int nesterov) {
+  const int k = blockIdx.y;
+  const uint64_t n = a.n[k];
+  float* v = a.t[k];
+  const float* g = a.g[k];
+  float* acc = a.s0[k];
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const float x = momentum * acc[i] - lr * g[i];
+    acc[i] = x;
+    v[i] += nesterov ? momentum * x - lr * g[i] : x;
+  }
+}
+__global__ void adam_multi_kernel(MultiArgs a, float beta1, float beta2, float lr) {
+  const int k = blockIdx.y;
+  const uint64_t n = a.n[k];
+  float* t = a.t[k];
+  const float* g = a.g[k];
+  float* m = a.s0[k];
+  float* v2 = a.s1[k];
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    const float gi = g[i];
+    const float mi = beta1 * m[i] + (1.0f - beta1) * gi;
+    const float vi = beta2 * v2[i] + (1.0f - beta2) * gi * gi;
+    m[i] = mi;
+    v2[i] = vi;
+    t[i] += -lr * mi / (sqrtf(vi) + 1e-7f);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host launchers (called from the C ABI)
 // ---------------------------------------------------------------------------
@@ -562,6 +601,33 @@ int launch_random_normal(DeviceCtx* ctx, float* out, uint64_t n, uint32_t seed, 
   if (!out) return set_error(LNN_ERR_INVALID, "random_normal: null pointer");
   hipLaunchKernelGGL(random_normal_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, out, n, seed, mean, stddev);
   LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+// kind 0: SGD (p0 momentum, p1 unused, flag nesterov), kind 1: Adam (p0 beta1, p1 beta2)
+int launch_update_multi(DeviceCtx* ctx, int kind, int count, const uint64_t* n, float* const* t, const float* const* g,
+                        float* const* s0, float* const* s1, float p0, float p1, float lr, int flag) {
+  const char* who = kind ? "adam_update_multi" : "sgd_update_multi";
+  if (count < 0) return set_error(LNN_ERR_INVALID, std::string(who) + ": negative count");
+  if (count == 0) return LNN_OK;
+  if (!n || !t || !g || !s0 || (kind && !s1)) return set_error(LNN_ERR_INVALID, std::string(who) + ": null array");
+  for (int i0 = 0; i0 < count; i0 += kMultiMax) {
+    const int nb = count - i0 < kMultiMax ? count - i0 : kMultiMax;
+    MultiArgs a = {};
+    uint64_t most = 0;
+    for (int i = 0; i < nb; ++i) {
+      a.n[i] = n[i0 + i];
+      a.t[i] = t[i0 + i]; a.g[i] = g[i0 + i]; a.s0[i] = s0[i0 + i]; a.s1[i] = kind ? s1[i0 + i] : nullptr;
+      if (a.n[i] && (!a.t[i] || !a.g[i] || !a.s0[i] || (kind && !a.s1[i])))
+        return set_error(LNN_ERR_INVALID, std::string(who) + ": null pointer");
+      most = a.n[i] > most ? a.n[i] : most;
+    }
+    if (most == 0) continue;
+    const dim3 grid(grid_for(most, ctx->cus / 2).x, (unsigned)nb);
+    if (kind) hipLaunchKernelGGL(adam_multi_kernel, grid, dim3(256), 0, ctx->stream, a, p0, p1, lr);
+    else hipLaunchKernelGGL(sgd_multi_kernel, grid, dim3(256), 0, ctx->stream, a, p0, lr, flag ? 1 : 0);
+    LNN_HIP(hipGetLastError());
+  }
   return LNN_OK;
 }
 

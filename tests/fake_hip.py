@@ -13,7 +13,7 @@ from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
          'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
-         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal', 'bias_act_bwd']
+         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal', 'bias_act_bwd', 'sgd_update_multi', 'adam_update_multi']
 
 
 class FakeHip:
@@ -192,6 +192,16 @@ class FakeHip:
         M[:] = b1 * M + (np.float32(1) - b1) * G
         V[:] = b2 * V + (np.float32(1) - b2) * G * G
         T[:] = T - np.float32(lr) * M / (np.sqrt(V) + np.float32(1e-7))
+
+    def sgd_update_multi(self, dev, ns, vs, gs, accs, momentum, lr, nesterov):
+        for n, v, g, a in zip(ns, vs, gs, accs):
+            self.sgd_update(dev, n, v, g, a, momentum, lr, nesterov)
+        self.launches -= len(ns) - 1
+
+    def adam_update_multi(self, dev, ns, ts, gs, ms, vs, beta1, beta2, lr):
+        for n, t, g, m, v in zip(ns, ts, gs, ms, vs):
+            self.adam_update(dev, n, t, g, m, v, beta1, beta2, lr)
+        self.launches -= len(ns) - 1
 
     def bias_act_bwd(self, dev, N, O, HW, y, dy, act, slope, dpre, dbias, beta_bias):
         self.launches += 1

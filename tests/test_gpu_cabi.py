@@ -426,6 +426,35 @@ def test_conv_benchmark_geometries_float(hip, name):
     assert max(errs) <= TOL
 
 
+def test_multi_tensor_updates_equal_single_launches(hip):
+    """lnn_sgd_update_multi_f32 / lnn_adam_update_multi_f32 against one call per tensor: the same bits, for more
+    tensors than one launch holds and with an empty tensor among them."""
+    rs = np.random.RandomState(77)
+    sizes = [1, 7, 0, 300, 4097, 64 * 9, 33, 1 << 16] + [11 + 3 * i for i in range(14)]   # 22 tensors
+    mk = lambda: [rs.standard_normal(max(n, 1)).astype(np.float32) for n in sizes]
+    v0, g0, a0, b0 = mk(), mk(), mk(), [np.abs(x) for x in mk()]
+    for kind in ('sgd', 'sgd_nesterov', 'adam'):
+        say(f'multi-tensor update {kind}')
+        one = [[DevArr(hip, x) for x in arrs] for arrs in (v0, g0, a0, b0)]
+        many = [[DevArr(hip, x) for x in arrs] for arrs in (v0, g0, a0, b0)]
+        for i, n in enumerate(sizes):
+            if kind == 'adam':
+                hip.adam_update(0, n, one[0][i].ptr, one[1][i].ptr, one[2][i].ptr, one[3][i].ptr, 0.9, 0.999, 1e-2)
+            else:
+                hip.sgd_update(0, n, one[0][i].ptr, one[1][i].ptr, one[2][i].ptr, 0.9, 1e-2, kind == 'sgd_nesterov')
+        ptrs = [[d.ptr for d in col] for col in many]
+        if kind == 'adam':
+            hip.adam_update_multi(0, sizes, ptrs[0], ptrs[1], ptrs[2], ptrs[3], 0.9, 0.999, 1e-2)
+        else:
+            hip.sgd_update_multi(0, sizes, ptrs[0], ptrs[1], ptrs[2], 0.9, 1e-2, kind == 'sgd_nesterov')
+        for col_one, col_many in zip(one, many):
+            for x, y in zip(col_one, col_many):
+                assert np.array_equal(x.get(), y.get())
+    hip.sgd_update_multi(0, [], [], [], [], 0.9, 1e-2, False)      # nothing to do
+    with pytest.raises(hip.HipException):
+        hip.sgd_update_multi(0, [4], [None], [many[1][0].ptr], [many[2][0].ptr], 0.9, 1e-2, False)
+
+
 def test_bias_act_bwd_one_pass(hip):
     """dpre = dy * f'(y) and dbias[o] (+)= sum dpre: exact on small integers with a power-of-two slope, <= 1e-5 of
     the largest |dbias| on floats (fp32 sums against fp64)."""
