@@ -175,7 +175,9 @@ __global__ __launch_bounds__(256) void reduce_partials_batch(ReduceBatch b) {
 }
 
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
-enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5 };
+// PASS_WGRAD_TAP4: PASS_WGRAD_TAP with 128-bit transfers of the pixel gather too (stride 1, OW % 4 == 0, no padded columns)
+enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5, PASS_WGRAD_TAP4 = 6 };
+constexpr bool wgrad_tap(int pass) { return pass == PASS_WGRAD_TAP || pass == PASS_WGRAD_TAP4; }
 
 // Wp[a][tap][b] = W[..] so that the tap-major K index tap*CH + ch is contiguous:
 //   mode 0 (forward): Wp[o][tap][c] = W[o][c][tap]
@@ -211,12 +213,12 @@ template <int PASS, int WM, int NTMAX, bool FLAG>
 struct ConvCfg {
   static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
   // the tap-major passes send both operands straight into unpadded LDS tiles, three stages deep
-  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || PASS == PASS_DGRAD_TAP || PASS == PASS_WGRAD_TAP;
+  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || PASS == PASS_DGRAD_TAP || wgrad_tap(PASS);
   // A side is K-contiguous in LDS for all passes.
   static constexpr int SA = DIRECT ? BM * BK : LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
   static constexpr int SB = DIRECT ? BNMAX * BK : LdsSize<PASS == PASS_WGRAD, BNMAX>::value;
-  static constexpr int STAGES = !DIRECT ? 2 : (PASS == PASS_WGRAD_TAP ? LNN_STAGES_WGRAD : LNN_STAGES_FD);
+  static constexpr int STAGES = !DIRECT ? 2 : (wgrad_tap(PASS) ? LNN_STAGES_WGRAD : LNN_STAGES_FD);
 };
 
 // Loader selection and initialisation per pass.  FLAG:
@@ -284,6 +286,15 @@ struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A& la) const { l.init(rx, g, col0, la, kend, kbeg); }
 };
 
+template <bool FLAG, int ST>
+struct ConvProblem<PASS_WGRAD_TAP4, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
+  template <int R> using LA = ConvWgradTapA4Direct<R>;
+  template <int R> using LB = ConvWgradTapB4Direct<R>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A& la) const { l.init(rx, g, col0, la, kend, kbeg); }
+};
+
 // Where GEMM element (m, column) of a pass lives in its output tensor.
 __host__ __device__ inline OutMap plain_map(int ncols) {
   OutMap om;
@@ -299,7 +310,7 @@ __host__ __device__ inline OutMap final_map(const ConvArgs& a) {
   } else if (PASS == PASS_DGRAD || PASS == PASS_DGRAD_TAP) {
     om.nchw = 3; om.ld = a.full_IHW; om.mtot = a.g.C; om.dHW = a.g.dIHW;
     om.dCW = a.g.dIW; om.s = a.cls_s; om.iw = a.full_IW; om.org = a.cls_org;
-  } else if (PASS == PASS_WGRAD_TAP) {
+  } else if (wgrad_tap(PASS)) {
     // GEMM column tap*C + c lands in dW[o][c][tap]
     om.nchw = 2; om.ld = a.Ncols; om.mtot = a.g.KK; om.dHW = a.dC;
   }
@@ -325,7 +336,7 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a) {
     // K slice of this workgroup: slices are in gridDim.y, except that the tap-major wgrad pass has a flat
     // grid in which the last chunk, if it holds less work, is cut into proportionally fewer slices
     int slice = blockIdx.y, ns = a.ksplit;
-    if (PASS == PASS_WGRAD_TAP) {
+    if (wgrad_tap(PASS)) {
       const int b = blockIdx.x, nfull = (a.n_chunks - 1) * a.ksplit;
       if (b < nfull) {
         chunk_i = b / a.ksplit;
@@ -348,7 +359,7 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a) {
   p.om = a.ksplit > 1 ? plain_map(a.Ncols) : final_map<PASS>(a);
   p.post = a.post;
   if (a.ksplit > 1) { p.post.bias = nullptr; p.post.act = 0; }   // applied by the slice reduction
-  if (PASS == PASS_WGRAD_TAP)
+  if (wgrad_tap(PASS))
     walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.g.KK, a.total_units,
                               a.chunk_units, chunk_i);
   else
@@ -463,7 +474,7 @@ static ReduceArgs reduce_args(const ConvArgs& a, int final_beta) {
   r.n = a.M * a.Ncols; r.slices = a.ksplit; r.slices_last = a.ksplit; r.beta = final_beta; r.ncols = a.Ncols;
   r.bm_log = WM == 4 ? 7 : (WM == 2 ? 6 : 5); r.uw_log = WN == 4 ? 7 : (WN == 2 ? 6 : 5);
   r.per_mt = 0; r.last_unit0 = 0x7fffffff;
-  if (PASS == PASS_WGRAD_TAP) {
+  if (wgrad_tap(PASS)) {
     r.slices_last = a.ks_last;
     r.per_mt = a.g.KK * a.n_units;
     r.last_unit0 = (a.n_chunks - 1) * a.chunk_units;
@@ -526,12 +537,12 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   float* final_out = a.Out;
   const int final_beta = a.beta;
   int grid_y = 1;
-  if (PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP) {
+  if (PASS == PASS_WGRAD || wgrad_tap(PASS)) {
     const int m_tiles = (a.M + BM - 1) / BM;
     a.n_units = (a.Ncols + 32 * WN - 1) / (32 * WN);
     long long total = (long long)m_tiles * a.n_units;
     a.chunk_units = 0;
-    if (PASS == PASS_WGRAD_TAP) {
+    if (wgrad_tap(PASS)) {
       // columns are tap-major: KK segments of C / (32*WN) units per M tile; a workgroup
       // takes one sub-tile's worth of whole segments (or of one segment's halves)
       a.n_units = a.g.C / (32 * WN);
@@ -545,16 +556,16 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     a.n_chunks = 1;
     a.ks_last = 1;
     // one full-width sub-tile per workgroup, then as many K slices as fill the chip
-    const int chunk = PASS == PASS_WGRAD_TAP ? a.chunk_units : 2 * NTMAX;
+    const int chunk = wgrad_tap(PASS) ? a.chunk_units : 2 * NTMAX;
     int grid = (int)((total + chunk - 1) / chunk);
     const int nkt = (a.K + BK - 1) / BK;
-    long long s = PASS == PASS_WGRAD_TAP ? slots * chunk / total : slots / grid;
+    long long s = wgrad_tap(PASS) ? slots * chunk / total : slots / grid;
     if (s > nkt / 4) s = nkt / 4;
     if (s > 1024) s = 1024;
     if (s < 1) s = 1;
     int ksplit = (int)s;
     grid_y = ksplit;
-    if (PASS == PASS_WGRAD_TAP) {
+    if (wgrad_tap(PASS)) {
       // the last chunk holds rem <= chunk units: give it the matching share of the slices.  A K step of u
       // units costs about (o + u) with a fixed part o worth an eighth of a full chunk (measured: a half
       // chunk's step takes 0.56 of a full one), so that is the ratio of the slice counts.
@@ -838,7 +849,12 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   const int unit = g.O > 64 ? 32 : (g.O > 32 ? 64 : 128);
   // ... and a K step of pixels never wraps around an image more than once
   const bool vec = g.OHW % 4 == 0 && aligned16(dY);
-  if (g.C % unit == 0 && BK / g.OW + 1 <= g.OH) return launch_by_m<PASS_WGRAD_TAP>(ctx, a, vec);
+  if (g.C % unit == 0 && BK / g.OW + 1 <= g.OH) {
+    // every tap of every output pixel reads a column inside the image: the gather can move four pixels at a time
+    const bool cols_inside = g.PADL == 0 && g.OW - 1 + (g.KW - 1) * g.D <= g.IW - 1;
+    if (vec && g.S == 1 && g.OW % 4 == 0 && cols_inside) return launch_by_m<PASS_WGRAD_TAP4>(ctx, a, true);
+    return launch_by_m<PASS_WGRAD_TAP>(ctx, a, vec);
+  }
   return launch_by_m<PASS_WGRAD>(ctx, a, vec);
 }
 

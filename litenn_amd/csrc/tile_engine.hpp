@@ -1020,6 +1020,56 @@ struct ConvWgradTapBDirect {
   }
 };
 
+// The pixel gather with 128-bit transfers, for stride 1, OW % 4 == 0 and no padding at the left or right edge
+// (1x1 kernels, 'valid' convolutions): the four pixels p..p+3 (p % 4 == 0) of a lane sit in one output row, so the
+// input pixels under a tap are four consecutive floats of one input row (at any 4-byte alignment), all inside the
+// image or - above / below it - all outside.  Same block / lane layout as ConvWgradTapA4Direct: lane l carries
+// 4-pixel group (l % 8) ^ (l / 8) for channel l / 8 of an 8-channel block, wavefront w the blocks w, w+4, ...
+// With padded columns one group per image row and off-centre tap hangs over the edge; repairing it after the
+// transfer (zeros over the outside elements) was measured and cost more than the wider transfers gain.
+template <int R>
+struct ConvWgradTapB4Direct {
+  static constexpr bool KC = true, DIRECT = true;
+  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int NB = R / 8, E = (NB + 3) / 4;
+  static constexpr int NLD = NB % 4 == 0 ? E : -1;
+  static_assert(R % 8 == 0, "whole 8-row blocks");
+  rsrc_t rs;
+  int IH, IHW, OH, OW, kend;
+  int p, oh, ow, ih, xoff;
+  int qh, rw, x_step, xwrap_w, xwrap_h;
+  template <class LA>
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int col0, const LA&, int kend_, int k0) {
+    rs = r;
+    IH = g.IH; IHW = g.IHW; OH = g.OH; OW = g.OW;
+    kend = kend_;
+    const int tap = col0 / g.C, c0 = col0 - tap * g.C;
+    const int kh = tap / g.KW, kw = tap - kh * g.KW;
+    qh = BK / g.OW; rw = BK - qh * g.OW;
+    x_step = qh * g.IW + rw;
+    xwrap_w = g.IW - g.OW;
+    xwrap_h = g.C * g.IHW - g.OH * g.IW;
+    const int lane = threadIdx.x & 63, rb = lane >> 3;
+    p = k0 + 4 * ((lane & 7) ^ rb);
+    const uint32_t img = g.dOHW.div((uint32_t)p), rem = (uint32_t)p - img * g.OHW;
+    oh = (int)g.dOW.div(rem);
+    ow = (int)rem - oh * g.OW;
+    ih = oh + kh * g.D - g.PADT;
+    xoff = ((int)img * g.C + c0 + 8 * gwave() + rb) * g.IHW + ih * g.IW + ow + kw * g.D;
+  }
+  __device__ __forceinline__ void issue(int, float* lds, int, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+    const uint32_t voff = p < kend && (uint32_t)ih < (uint32_t)IH ? (uint32_t)xoff * 4u : OOB;
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      if (NB % 4 == 0 || wave + 4 * e < NB)
+        buf_load_lds16(rs, lds + (off + (wave + 4 * e) * 8) * BK, voff, (uint32_t)(32 * e * IHW) * 4u);
+    p += BK; oh += qh; ow += rw; ih += qh; xoff += x_step;
+    if (ow >= OW) { ow -= OW; ++oh; ++ih; xoff += xwrap_w; }
+    if (oh >= OH) { oh -= OH; ih -= OH; xoff += xwrap_h; }
+  }
+};
+
 // Optional per-row bias and activation applied to a finished element before
 // it is stored ('=' only): y = f(acc + bias[m]), f = identity or leaky ReLU
 // (x >= 0 ? x : slope * x, the same selection the pointwise kernel makes).

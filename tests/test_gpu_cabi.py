@@ -275,6 +275,36 @@ def test_conv_wide_images_pixel_walk_integer_exact(hip):
                 assert np.array_equal(dw, rdw), ('dW', xs, oc, s, d, ks, padding)
 
 
+def test_conv_wgrad_128bit_pixel_gather_integer_exact(hip):
+    """Stride 1, an output width that is a multiple of 4 and no padded columns (1x1 kernels, 'valid' convolutions,
+    padding at the top / bottom only) send the wgrad pixel gather as 128-bit transfers of four consecutive input
+    pixels at any 4-byte alignment; rows above / below the image arrive as zeros.  The same geometries with padded
+    columns take the 32-bit gather and are checked beside them."""
+    rs = np.random.RandomState(31)
+    cases = [((2, 32, 12, 12), 3, 1, 'same'), ((1, 32, 58, 58), 3, 1, 'valid'), ((2, 64, 9, 16), 5, 1, 'same'),
+             ((2, 32, 10, 20), 3, 2, 'same'), ((1, 32, 7, 10), 3, 1, 2), ((2, 32, 6, 6), 3, 1, 4),
+             ((3, 32, 5, 14), 2, 1, (2, 0, 1, 1)), ((1, 96, 8, 9), 3, 1, (3, 1, 2, 0)), ((2, 32, 6, 8), 7, 1, 'same'),
+             ((1, 32, 20, 44), 3, 3, 'same'), ((4, 32, 8, 8), 1, 1, 'same'), ((1, 32, 9, 4), 3, 1, 'same'),
+             ((2, 128, 28, 28), 3, 1, 'same'), ((1, 32, 33, 36), 4, 1, (1, 1, 2, 2)),
+             ((2, 32, 8, 18), 3, 1, (0, 1, 0, 1)), ((1, 64, 10, 12), 1, 1, (0, 2, 0, 2)), ((2, 32, 9, 20), 3, 2, 'valid'),
+             ((3, 32, 6, 11), 4, 1, (0, 3, 0, 3)), ((2, 256, 28, 28), 1, 1, 'same'), ((1, 32, 40, 35), 4, 1, 'valid')]
+    for xs, ks, d, padding in cases:
+        ci = info_conv2d(xs[2], xs[3], ks, ks, 1, d, padding)
+        assert ci.OW % 4 == 0, (xs, ks, d, padding, ci.OW)
+        for oc in (32, 72, 130):
+            say(f'wgrad gather x={xs} oc={oc} ks={ks} d={d} pad={padding}')
+            x = rs.randint(-5, 6, size=xs).astype(np.float32)
+            w = rs.randint(-5, 6, size=(oc, xs[1], ks, ks)).astype(np.float32)
+            dy = rs.randint(-5, 6, size=(xs[0], oc, ci.OH, ci.OW)).astype(np.float32)
+            rdw = conv2d_dw(x, dy, w.shape, 1, d, padding)
+            desc, _ = _desc(hip, xs, w.shape, 1, d, padding)
+            X, dY = DevArr(hip, x), DevArr(hip, dy)
+            for beta, fill in ((0, np.nan), (1, 3.0)):
+                dW = DevArr(hip, shape=w.shape, fill=fill)
+                hip.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW.ptr, beta)
+                assert np.array_equal(dW.get() - (3.0 if beta else 0.0), rdw), (xs, oc, ks, d, padding, beta)
+
+
 def test_conv_few_tiles_split_k_integer_exact(hip):
     """Deep layers on small images have a long K and few output tiles: forward
     and dgrad then split K over the idle compute units and a second kernel
