@@ -19,6 +19,9 @@
 #ifndef LNN_FD_B_DIRECT
 #define LNN_FD_B_DIRECT 1
 #endif
+#ifndef LNN_CLASS_SHARES
+#define LNN_CLASS_SHARES 1
+#endif
 #ifndef LNN_WGRAD_B_DIRECT
 #define LNN_WGRAD_B_DIRECT 1
 #endif
@@ -618,12 +621,38 @@ template <int PASS, int WM, int NTMAX>
 static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_off) {
   const int n = (int)cls.size();
   const int per_batch = n < kMaxBatch ? n : kMaxBatch;
-  const long long slots = ctx->cus / per_batch > 0 ? ctx->cus / per_batch : 1;   // equal shares of the chip
+  const long long equal = ctx->cus / per_batch > 0 ? ctx->cus / per_batch : 1;   // equal shares of the chip
+  // The classes of one launch differ in their number of taps (5x5 stride 2: 9, 6, 6 and 4): with the tap-major
+  // kernels, whose time follows the multiply-adds, each gets workgroups in proportion to its work instead
+  // (256 -> 512 channels at 16 x 16: 77 -> 63 us).
+  std::vector<long long> share(n, equal);
+  if (LNN_CLASS_SHARES && PASS == PASS_DGRAD_TAP && n <= kMaxBatch) {
+    std::vector<long long> prop(n, equal);
+    long long total = 0, given = 0;
+    for (int i = 0; i < n; ++i) total += (long long)cls[i].K * cls[i].Ncols;
+    for (int i = 0; i < n && total > 0; ++i) {
+      prop[i] = (long long)ctx->cus * cls[i].K * cls[i].Ncols / total;
+      prop[i] = prop[i] < 1 ? 1 : prop[i];
+      given += prop[i];
+    }
+    for (int i = 0; given > ctx->cus && i < n; ++i)
+      if (prop[i] > 1) { --prop[i]; --given; }
+    // Only where every class is cut along K anyway (few output tiles: any share divides into whole sub-tiles times
+    // K slices).  Classes with many tiles and no K split lose more to the narrow sub-tiles of an odd share than
+    // they gain (64 -> 128 channels at 64 x 64: 82 -> 121 us).
+    bool all_split = true;
+    for (int i = 0; i < n; ++i) {
+      ConvArgs a = cls[i];
+      plan_tiles<WM, NTMAX>(a, equal);
+      all_split = all_split && a.total_units >= 0 && a.ksplit > 1;
+    }
+    if (all_split) share = prop;
+  }
   std::vector<float*> final_out(n);
   std::vector<int> final_beta(n);
   for (int i = 0; i < n; ++i) {
     ConvArgs& a = cls[i];
-    const size_t need = plan_tiles<WM, NTMAX>(a, slots);
+    const size_t need = plan_tiles<WM, NTMAX>(a, share[i]);
     if (a.total_units < 0) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
     final_out[i] = a.Out;
     final_beta[i] = a.beta;
