@@ -33,7 +33,9 @@ PEAK_HBM_GBS = 8000.0
 # copy of known size), measured separately under rocprofv3 --pmc; keyed by workload and pass.  A pass that has
 # not been measured reports null.
 MEASURED_TRAFFIC_BYTES = {
-    'cfg3_vgg3x3': {'fwd': 340.0e6, 'dX': 360.9e6, 'dW': 236.4e6 + 40.5e6},   # dW = wgrad kernel + slice reduction
+    'cfg3_vgg3x3': {'fwd': 316.5e6 + 4.5e6, 'dX': 384.6e6 + 4.5e6, 'dW': 236.3e6 + 40.5e6},   # + weight permutation / slice reduction
+    'cfg2_matmul': {'fwd': 1208.2e6, 'dA': 1275.5e6, 'dB': 1275.3e6},
+    'cfgD_depthwise': {'fwd': 206.1e6, 'dX': 309.8e6, 'dK': 205.7e6 + 0.2e6},
 }
 
 CONV_CONFIGS = {
@@ -246,7 +248,7 @@ def bench_matmul(api, steps, warmup, n=4096, cpu=True):
            'config': {'workload': f'cfg2_matmul: [{n}x{n}] @ [{n}x{n}], step = C + dA(+=) + dB(+=)'},
            'roofline': {'bound': 'mfma', 'kernel': dom, 'achieved': per_pass[dom]['tflops'],
                         'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s', 'frac': per_pass[dom]['frac_mfma'],
-                        'traffic': None},
+                        'traffic': MEASURED_TRAFFIC_BYTES['cfg2_matmul'].get(dom) if n == 4096 else None},
            'passes': per_pass}
     if cpu:
         from oracle import refpath
@@ -395,7 +397,8 @@ def bench_depthwise(api, steps, warmup, cpu=True):
                                   'step = fwd + dX(+=) + dK(+=)'},
            'images_per_s': N / wall_ms * 1e3,
            'roofline': {'bound': 'hbm', 'kernel': dom, 'achieved': per_pass[dom]['alg_gbs'], 'peak': PEAK_HBM_GBS,
-                        'unit': 'GB/s', 'frac': per_pass[dom]['frac_hbm'], 'traffic': None},
+                        'unit': 'GB/s', 'frac': per_pass[dom]['frac_hbm'],
+                        'traffic': MEASURED_TRAFFIC_BYTES['cfgD_depthwise'].get(dom)},
            'passes': per_pass}
     if cpu:
         from oracle import depthwise_all
