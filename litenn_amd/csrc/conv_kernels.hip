@@ -22,6 +22,9 @@
 #ifndef LNN_CLASS_SHARES
 #define LNN_CLASS_SHARES 1
 #endif
+#ifndef LNN_SMALL_DGRAD
+#define LNN_SMALL_DGRAD 1
+#endif
 #ifndef LNN_WGRAD_B_DIRECT
 #define LNN_WGRAD_B_DIRECT 1
 #endif
@@ -210,6 +213,165 @@ struct PermuteBatch {
 };
 __global__ void permute_weights_classes(PermuteBatch b, const float* w, int O, int C, int KK, ConvGeom g) {
   permute_one(b.wp[blockIdx.y], w, O, C, KK, 1, g, b.pc[blockIdx.y], blockIdx.x * blockDim.x + threadIdx.x);
+}
+
+// ---- data gradient for very few input channels (image stems, the last layer of a decoder) ----------------------
+// With C <= 4 the GEMM of the data gradient has at most 4 rows, and an MFMA tile would work on 32.  This kernel
+// computes it on the vector ALU instead.  Stride S, dilation 1, square K x K kernel: the input pixels with the same
+// rh = (ih + PADT) % S, rw = (iw + PADW) % S form a class that sees the taps kh = rh, rh + S, ... (NKH of them) and
+// kw = rw, rw + S, ..., spaced one output pixel apart:
+//   dX[n][c][h0 + S*y][w0 + S*x] (+)= sum over o, jh, jw of dY[n][o][y + ah - jh][x + aw - jw] * W[o][c][rh + S*jh][rw + S*jw]
+// A block owns the 32 x 32 pixels (y, x) of ALL S*S classes of one image, i.e. one region of dY, which it brings to
+// LDS once per chunk of kDsOC output channels (row by row with global -> LDS transfers, all in flight together)
+// beside the chunk's weights (4 floats per tap, channels past C zero).  A thread owns 2 x 2 pixels of every class:
+// per output channel and class it reads its (NKH+1) x (NKW+1) window and each tap's weights (a broadcast read) once
+// for 4 * NKH * NKW * C multiply-adds.
+constexpr int kDsOC = 8, kDsTile = 32;
+struct SmallDgradArgs {
+  const float* dY;
+  const float* wc;        // [O][K*K taps, class by class][4]
+  float* dX;
+  int N, O, C, OH, OW, IH, IW;
+  int h0[4], w0[4];       // per class (rh*S + rw): origin, ...
+  int ph[4], pw[4];       // ... plane size (0: no such pixels), ...
+  int dh[4], dw[4];       // ... and tile row / column of output pixel (y + ah, x + aw) for y = x = 0
+  int oh_base, ow_base;   // output pixel under tile element (0, 0) of block (0, 0)
+  int th, tw;             // tile rows / columns in use
+  int tiles_x, beta;
+};
+// number of taps k < K with k % S == r, and the number of taps in the classes before class (rh, rw)
+constexpr int ds_nk(int K, int S, int r) { return r < K ? (K - r + S - 1) / S : 0; }
+constexpr int ds_tap_base(int K, int S, int cls) {
+  int n = 0;
+  for (int q = 0; q < cls; ++q) n += ds_nk(K, S, q / S) * ds_nk(K, S, q % S);
+  return n;
+}
+// Wc[o][t][c]: t runs over the classes' taps in class order, c < 4 (zero for c >= C)
+__global__ void small_dgrad_weights(float* wc, const float* w, int O, int C, int K, int S) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x, KK = K * K;
+  if (i >= O * KK * 4) return;
+  const int c = i & 3, t = (i >> 2) % KK, o = (i >> 2) / KK;
+  int rest = t, kh = 0, kw = 0;
+  for (int cls = 0; cls < S * S; ++cls) {
+    const int rh = cls / S, rw = cls % S;
+    const int nh = rh < K ? (K - rh + S - 1) / S : 0, nw = rw < K ? (K - rw + S - 1) / S : 0;
+    if (rest < nh * nw) {
+      kh = rh + S * (rest / nw);
+      kw = rw + S * (rest % nw);
+      break;
+    }
+    rest -= nh * nw;
+  }
+  wc[i] = c < C ? w[((size_t)o * C + c) * KK + kh * K + kw] : 0.0f;
+}
+
+template <int S, int K, int CN, int CLS>
+struct SmallDgradClass {
+  static constexpr int RH = CLS / S, RW = CLS % S, NKH = ds_nk(K, S, RH), NKW = ds_nk(K, S, RW);
+  static constexpr int TAP0 = ds_tap_base(K, S, CLS);
+  // adds output channel o's contribution to the 2 x 2 pixels of this class
+  static __device__ __forceinline__ void accumulate(const SmallDgradArgs& a, const float* tile, int pitch, const float* wo,
+                                                    int ty, int tx, float (&acc)[2][2][CN]) {
+    if constexpr (NKH > 0 && NKW > 0) {
+      // tile element of output pixel (y + ah - jh, x + aw - jw): row dh + y - jh
+      const float* base = tile + (a.dh[CLS] + 2 * ty - (NKH - 1)) * pitch + a.dw[CLS] + 2 * tx - (NKW - 1);
+      float win[NKH + 1][NKW + 1];
+#pragma unroll
+      for (int i = 0; i <= NKH; ++i)
+#pragma unroll
+        for (int j = 0; j <= NKW; ++j) win[i][j] = base[i * pitch + j];
+#pragma unroll
+      for (int jh = 0; jh < NKH; ++jh)
+#pragma unroll
+        for (int jw = 0; jw < NKW; ++jw) {
+          const f32x4 w4 = *reinterpret_cast<const f32x4*>(wo + (TAP0 + jh * NKW + jw) * 4);
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const float v = win[i + NKH - 1 - jh][j + NKW - 1 - jw];
+#pragma unroll
+              for (int c = 0; c < CN; ++c) acc[i][j][c] += v * w4[c];
+            }
+        }
+    }
+  }
+  static __device__ __forceinline__ void store(const SmallDgradArgs& a, int n, int y0, int x0, int ty, int tx,
+                                               const float (&acc)[2][2][CN]) {
+    if constexpr (NKH > 0 && NKW > 0) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int y = y0 + 2 * ty + i, x = x0 + 2 * tx + j;
+          if (y >= a.ph[CLS] || x >= a.pw[CLS]) continue;
+#pragma unroll
+          for (int c = 0; c < CN; ++c) {
+            if (c >= a.C) continue;
+            float* dst = a.dX + ((size_t)n * a.C + c) * a.IH * a.IW + (size_t)(a.h0[CLS] + S * y) * a.IW + a.w0[CLS] + S * x;
+            *dst = a.beta ? *dst + acc[i][j][c] : acc[i][j][c];
+          }
+        }
+    }
+  }
+};
+
+template <int S, int K, int CN>
+__global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
+  constexpr int NCLS = S * S, KK = K * K;
+  constexpr int TMAX = kDsTile + (K + S - 1) / S + 1, PITCH = TMAX | 1, PLANE = (TMAX * PITCH + 63) / 64 * 64;
+  __shared__ float tile[kDsOC * PLANE + 64];
+  __shared__ __attribute__((aligned(16))) float wl[kDsOC * KK * 4];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int by = blockIdx.x / a.tiles_x, bx = blockIdx.x - by * a.tiles_x, n = blockIdx.y;
+  const int y0 = by * kDsTile, x0 = bx * kDsTile;
+  const int oh0 = a.oh_base + y0, ow0 = a.ow_base + x0;
+  float acc[NCLS][2][2][CN];
+#pragma unroll
+  for (int q = 0; q < NCLS; ++q)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int c = 0; c < CN; ++c) acc[q][i][j][c] = 0.0f;
+  const uint32_t plane = (uint32_t)a.OH * a.OW;
+  const rsrc_t rs = make_rsrc(a.dY, (uint32_t)a.N * a.O * plane * 4u);
+  // this lane's column of a tile row; lanes past the tile width take no part in the transfers
+  const int ow = ow0 + lane;
+  const bool col_lane = lane < a.tw, col_ok = (uint32_t)ow < (uint32_t)a.OW;
+  for (int o0 = 0; o0 < a.O; o0 += kDsOC) {
+    __syncthreads();
+    if (col_lane) {
+      for (int q = wave; q < kDsOC * a.th; q += 4) {   // (channel, row) pairs of the chunk, one transfer each
+        const int o = q / a.th, r = q - o * a.th, oh = oh0 + r;
+        const bool ok = col_ok && o0 + o < a.O && (uint32_t)oh < (uint32_t)a.OH;
+        const uint32_t voff = ok ? (((uint32_t)n * a.O + o0 + o) * plane + (uint32_t)oh * a.OW + ow) * 4u : OOB;
+        buf_load_lds4(rs, tile + o * PLANE + r * PITCH, voff, 0);
+      }
+    }
+    for (int i = threadIdx.x; i < kDsOC * KK * 4; i += 256)
+      wl[i] = o0 * KK * 4 + i < a.O * KK * 4 ? a.wc[(size_t)o0 * KK * 4 + i] : 0.0f;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+#pragma unroll 1
+    for (int o = 0; o < kDsOC; ++o) {
+      const float* t = tile + o * PLANE;
+      const float* wo = wl + o * KK * 4;
+      SmallDgradClass<S, K, CN, 0>::accumulate(a, t, PITCH, wo, ty, tx, acc[0]);
+      if constexpr (NCLS > 1) {
+        SmallDgradClass<S, K, CN, 1>::accumulate(a, t, PITCH, wo, ty, tx, acc[1]);
+        SmallDgradClass<S, K, CN, 2>::accumulate(a, t, PITCH, wo, ty, tx, acc[2]);
+        SmallDgradClass<S, K, CN, 3>::accumulate(a, t, PITCH, wo, ty, tx, acc[3]);
+      }
+    }
+  }
+  SmallDgradClass<S, K, CN, 0>::store(a, n, y0, x0, ty, tx, acc[0]);
+  if constexpr (NCLS > 1) {
+    SmallDgradClass<S, K, CN, 1>::store(a, n, y0, x0, ty, tx, acc[1]);
+    SmallDgradClass<S, K, CN, 2>::store(a, n, y0, x0, ty, tx, acc[2]);
+    SmallDgradClass<S, K, CN, 3>::store(a, n, y0, x0, ty, tx, acc[3]);
+  }
 }
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
@@ -752,6 +914,74 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   return launch_by_m<PASS_FWD>(ctx, a, a.K % 4 == 0 && aligned16(W));
 }
 
+// The vector-ALU data gradient serves C <= 4, dilation 1, stride 1 (K = 1, 3, 5) or 2 (K = 3, 4, 5, 7), when there
+// are enough tiles to occupy the chip (a small problem is quicker on the MFMA path, whose tiles are finer).
+static bool small_dgrad_applies(const DeviceCtx* ctx, const ConvGeom& g) {
+  if (!LNN_SMALL_DGRAD || g.C > 4 || g.D != 1 || g.KH != g.KW) return false;
+  const int K = g.KH;
+  const bool shape = (g.S == 1 && (K == 1 || K == 3 || K == 5)) || (g.S == 2 && (K == 3 || K == 4 || K == 5 || K == 7));
+  if (!shape) return false;
+  const long long ph = (g.IH + g.S - 1) / g.S, pw = (g.IW + g.S - 1) / g.S;
+  const long long blocks = ((ph + kDsTile - 1) / kDsTile) * ((pw + kDsTile - 1) / kDsTile) * g.N;
+  if ((uint64_t)g.N * g.O * g.OHW * 4 > kMaxTensorBytes) return false;
+  return blocks * 2 >= ctx->cus;
+}
+
+constexpr int kNotHere = 1;   // launch_small_dgrad: a geometry it leaves to the general path (no error)
+static int launch_small_dgrad(DeviceCtx* ctx, const ConvGeom& g, const float* dY, const float* W, float* dX, int beta) {
+  const int K = g.KH, S = g.S, n_w = g.O * K * K * 4;
+  int st = ensure_workspace(ctx, (size_t)n_w * sizeof(float));
+  if (st != LNN_OK) return st;
+  float* wc = static_cast<float*>(ctx->ws);
+  hipLaunchKernelGGL(small_dgrad_weights, dim3((n_w + 255) / 256), dim3(256), 0, ctx->stream, wc, W, g.O, g.C, K, S);
+  LNN_HIP(hipGetLastError());
+  SmallDgradArgs a;
+  a.dY = dY; a.wc = wc; a.dX = dX;
+  a.N = g.N; a.O = g.O; a.C = g.C; a.OH = g.OH; a.OW = g.OW; a.IH = g.IH; a.IW = g.IW;
+  int ah[4], aw[4], lo_h = 1 << 30, lo_w = 1 << 30, hi_h = -(1 << 30), hi_w = -(1 << 30), max_ph = 0, max_pw = 0;
+  for (int cls = 0; cls < 4; ++cls) {
+    a.h0[cls] = a.w0[cls] = a.ph[cls] = a.pw[cls] = a.dh[cls] = a.dw[cls] = 0;
+    ah[cls] = aw[cls] = 0;
+  }
+  for (int cls = 0; cls < S * S; ++cls) {
+    const int rh = cls / S, rw = cls % S;
+    const int nkh = rh < K ? (K - rh + S - 1) / S : 0, nkw = rw < K ? (K - rw + S - 1) / S : 0;
+    const int h0 = ((rh - g.PADT) % S + S) % S, w0 = ((rw - g.PADL) % S + S) % S;
+    a.h0[cls] = h0; a.w0[cls] = w0;
+    a.ph[cls] = h0 < g.IH ? (g.IH - h0 + S - 1) / S : 0;
+    a.pw[cls] = w0 < g.IW ? (g.IW - w0 + S - 1) / S : 0;
+    if (nkh == 0 || nkw == 0) {
+      if (!beta && a.ph[cls] > 0 && a.pw[cls] > 0) return kNotHere;   // a class without taps would need a zero fill
+      a.ph[cls] = a.pw[cls] = 0;
+      continue;
+    }
+    ah[cls] = (h0 + g.PADT - rh) / S;   // exact: h0 + PADT = rh (mod S)
+    aw[cls] = (w0 + g.PADL - rw) / S;
+    lo_h = std::min(lo_h, ah[cls] - (nkh - 1)); hi_h = std::max(hi_h, ah[cls]);
+    lo_w = std::min(lo_w, aw[cls] - (nkw - 1)); hi_w = std::max(hi_w, aw[cls]);
+    max_ph = std::max(max_ph, a.ph[cls]); max_pw = std::max(max_pw, a.pw[cls]);
+  }
+  if (max_ph == 0 || max_pw == 0) return LNN_OK;
+  for (int cls = 0; cls < S * S; ++cls) { a.dh[cls] = ah[cls] - lo_h; a.dw[cls] = aw[cls] - lo_w; }
+  a.oh_base = lo_h; a.ow_base = lo_w;
+  a.th = kDsTile + hi_h - lo_h; a.tw = kDsTile + hi_w - lo_w;
+  const int tmax = kDsTile + (K + S - 1) / S + 1;
+  if (a.th > tmax || a.tw > tmax || a.tw > 64) return kNotHere;
+  a.tiles_x = (max_pw + kDsTile - 1) / kDsTile;
+  a.beta = beta ? 1 : 0;
+  const dim3 grid((unsigned)(a.tiles_x * ((max_ph + kDsTile - 1) / kDsTile)), (unsigned)g.N), block(256);
+#define LNN_DS(S_, K_)                                                                                        \
+  do {                                                                                                        \
+    if (g.C == 3) hipLaunchKernelGGL((small_dgrad_kernel<S_, K_, 3>), grid, block, 0, ctx->stream, a);         \
+    else hipLaunchKernelGGL((small_dgrad_kernel<S_, K_, 4>), grid, block, 0, ctx->stream, a);                  \
+  } while (0)
+  if (S == 1) { if (K == 1) LNN_DS(1, 1); else if (K == 3) LNN_DS(1, 3); else LNN_DS(1, 5); }
+  else { if (K == 3) LNN_DS(2, 3); else if (K == 4) LNN_DS(2, 4); else if (K == 5) LNN_DS(2, 5); else LNN_DS(2, 7); }
+#undef LNN_DS
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
 int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta) {
   ConvGeom full;
   int st = fill_geom(d, full);
@@ -759,6 +989,10 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   if (!dY || !W || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
   const int S = full.S;
   if (S > 15) return set_error(LNN_ERR_UNSUPPORTED, "conv2d_dgrad: stride > 15");
+  if (small_dgrad_applies(ctx, full)) {
+    st = launch_small_dgrad(ctx, full, dY, W, dX, beta);
+    if (st != kNotHere) return st;
+  }
   st = reserve_tables(ctx, (size_t)S * S);
   if (st != LNN_OK) return st;
   const bool tap = full.O % BK == 0;

@@ -305,6 +305,33 @@ def test_conv_wgrad_128bit_pixel_gather_integer_exact(hip):
                 assert np.array_equal(dW.get() - (3.0 if beta else 0.0), rdw), (xs, oc, ks, d, padding, beta)
 
 
+def test_conv_dgrad_few_input_channels_vector_kernel_integer_exact(hip):
+    """C <= 4, dilation 1, stride 1 (K = 1, 3, 5) or 2 (K = 3, 4, 5, 7) with enough tiles for the chip takes the
+    vector-ALU data gradient (all pixel classes of a 32 x 32 tile in one block).  Image sizes that are not multiples
+    of the tile, every padding kind, '=' and '+=', and the neighbouring shapes that stay on the MFMA path."""
+    rs = np.random.RandomState(41)
+    cases = [(16, 3, 1, 3, 'same', 5), (16, 4, 1, 5, 'valid', 3), (16, 1, 1, 1, 'same', 6), (16, 2, 1, 3, 2, 4),
+             (16, 3, 1, 5, (1, 0, 3, 2), 3), (40, 3, 2, 7, 3, 1), (40, 3, 2, 5, 'same', 3), (40, 4, 2, 4, 1, 3),
+             (40, 1, 2, 3, 'valid', 4), (40, 2, 2, 5, (0, 2, 1, 0), 3), (40, 3, 2, 3, 0, 5), (40, 3, 2, 4, (2, 1, 0, 3), 2),
+             # not covered by the kernel: dilation, stride 3, 7 x 7 at stride 1
+             (16, 3, 1, 3, 'same', 4, 2), (30, 3, 3, 5, 2, 3), (16, 3, 1, 7, 'same', 2)]
+    for case in cases:
+        n, c, s_, k, padding, oc = case[:6]
+        d = case[6] if len(case) > 6 else 1
+        xs = (n, c, 70, 66)
+        ci = info_conv2d(70, 66, k, k, s_, d, padding)
+        say(f'small-C dgrad x={xs} oc={oc} k={k} s={s_} d={d} pad={padding}')
+        w = rs.randint(-4, 5, size=(oc, c, k, k)).astype(np.float32)
+        dy = rs.randint(-4, 5, size=(n, oc, ci.OH, ci.OW)).astype(np.float32)
+        ref = conv2d_dx(dy, w, xs, s_, d, padding)
+        desc, _ = _desc(hip, xs, w.shape, s_, d, padding)
+        W, dY = DevArr(hip, w), DevArr(hip, dy)
+        for beta, fill in ((0, np.nan), (1, -2.0)):
+            dX = DevArr(hip, shape=xs, fill=fill)
+            hip.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, beta)
+            assert np.array_equal(dX.get() - (-2.0 if beta else 0.0), ref), (case, beta)
+
+
 def test_conv_few_tiles_split_k_integer_exact(hip):
     """Deep layers on small images have a long K and few output tiles: forward
     and dgrad then split K over the idle compute units and a second kernel
