@@ -222,10 +222,10 @@ __global__ void permute_weights_classes(PermuteBatch b, const float* w, int O, i
 // kw = rw, rw + S, ..., spaced one output pixel apart:
 //   dX[n][c][h0 + S*y][w0 + S*x] (+)= sum over o, jh, jw of dY[n][o][y + ah - jh][x + aw - jw] * W[o][c][rh + S*jh][rw + S*jw]
 // A block owns the 32 x 32 pixels (y, x) of ALL S*S classes of one image, i.e. one region of dY, which it brings to
-// LDS once per chunk of kDsOC output channels (row by row with global -> LDS transfers, all in flight together)
-// beside the chunk's weights (4 floats per tap, channels past C zero).  A thread owns 2 x 2 pixels of every class:
-// per output channel and class it reads its (NKH+1) x (NKW+1) window and each tap's weights (a broadcast read) once
-// for 4 * NKH * NKW * C multiply-adds.
+// LDS once per chunk of kDsOC output channels (row by row with global -> LDS transfers, all in flight together).
+// A thread owns 2 x 2 pixels of every class: per output channel and class it reads its (NKH+1) x (NKW+1) window once;
+// the weights (4 floats per tap, channels past C zero) have the same address in every lane and come through the
+// scalar cache.  4 * NKH * NKW * C multiply-adds per window.
 constexpr int kDsOC = 8, kDsTile = 32;
 struct SmallDgradArgs {
   const float* dY;
@@ -321,7 +321,6 @@ __global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
   constexpr int NCLS = S * S, KK = K * K;
   constexpr int TMAX = kDsTile + (K + S - 1) / S + 1, PITCH = TMAX | 1, PLANE = (TMAX * PITCH + 63) / 64 * 64;
   __shared__ float tile[kDsOC * PLANE + 64];
-  __shared__ __attribute__((aligned(16))) float wl[kDsOC * KK * 4];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int by = blockIdx.x / a.tiles_x, bx = blockIdx.x - by * a.tiles_x, n = blockIdx.y;
   const int y0 = by * kDsTile, x0 = bx * kDsTile;
@@ -350,14 +349,14 @@ __global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
         buf_load_lds4(rs, tile + o * PLANE + r * PITCH, voff, 0);
       }
     }
-    for (int i = threadIdx.x; i < kDsOC * KK * 4; i += 256)
-      wl[i] = o0 * KK * 4 + i < a.O * KK * 4 ? a.wc[(size_t)o0 * KK * 4 + i] : 0.0f;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    const int on = a.O - o0 < kDsOC ? a.O - o0 : kDsOC;
 #pragma unroll 1
-    for (int o = 0; o < kDsOC; ++o) {
+    for (int o = 0; o < on; ++o) {
       const float* t = tile + o * PLANE;
-      const float* wo = wl + o * KK * 4;
+      // the same address in every lane: the weights arrive through the scalar cache
+      const float* wo = a.wc + (size_t)(o0 + o) * KK * 4;
       SmallDgradClass<S, K, CN, 0>::accumulate(a, t, PITCH, wo, ty, tx, acc[0]);
       if constexpr (NCLS > 1) {
         SmallDgradClass<S, K, CN, 1>::accumulate(a, t, PITCH, wo, ty, tx, acc[1]);
