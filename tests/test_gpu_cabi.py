@@ -313,6 +313,9 @@ def test_conv_dgrad_few_input_channels_vector_kernel_integer_exact(hip):
     cases = [(16, 3, 1, 3, 'same', 5), (16, 4, 1, 5, 'valid', 3), (16, 1, 1, 1, 'same', 6), (16, 2, 1, 3, 2, 4),
              (16, 3, 1, 5, (1, 0, 3, 2), 3), (40, 3, 2, 7, 3, 1), (40, 3, 2, 5, 'same', 3), (40, 4, 2, 4, 1, 3),
              (40, 1, 2, 3, 'valid', 4), (40, 2, 2, 5, (0, 2, 1, 0), 3), (40, 3, 2, 3, 0, 5), (40, 3, 2, 4, (2, 1, 0, 3), 2),
+             # fewer images, i.e. fewer tiles than half the chip: these stay on the MFMA path
+             (16, 3, 2, 5, 'same', 3), (16, 4, 2, 7, 3, 2), (6, 3, 1, 3, 'same', 4), (6, 2, 1, 5, (2, 0, 1, 3), 3),
+             (16, 1, 2, 4, 1, 3), (16, 3, 2, 3, (1, 0, 0, 1), 4),
              # not covered by the kernel: dilation, stride 3, 7 x 7 at stride 1
              (16, 3, 1, 3, 'same', 4, 2), (30, 3, 3, 5, 2, 3), (16, 3, 1, 7, 'same', 2)]
     for case in cases:
