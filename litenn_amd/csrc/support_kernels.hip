@@ -569,29 +569,32 @@ __device__ __forceinline__ void hash_u32x2(uint32_t& x, uint32_t& y) {
 // (float)h * 2^-32: the reference multiplies by 1.0 / (float)0xffffffffU, and (float)0xffffffffU rounds to 2^32
 constexpr float kUnitScale = 1.0f / 4294967296.0f;
 
-// out[i] = u * (high - low) + low in double, as the reference's double literals make it (RandomUniform.py:17-21)
-__global__ void random_uniform_kernel(float* __restrict__ out, uint64_t n, uint32_t seed, double span, double low) {
+// out[i] = u * (high - low) + low (RandomUniform.py:17-21).  The reference builds every kernel with
+// -cl-single-precision-constant (CLDevice.py:93), so low and high are float literals there and the whole expression
+// is single precision: span = (float)high - (float)low is rounded once, and the multiply-add is contracted into one
+// fused operation, which OpenCL C permits by default and GPU compilers do.
+__global__ void random_uniform_kernel(float* __restrict__ out, uint64_t n, uint32_t seed, float span, float low) {
   for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
     const float u = (float)hash_u32((uint32_t)(i + seed)) * kUnitScale;
-    out[i] = (float)((double)u * span + low);
+    out[i] = __builtin_fmaf(u, span, low);
   }
 }
-// Box-Muller on the two halves of the 2-D hash of (i + seed, 1) (RandomNormal.py:14-24); sqrt, log and cos in
-// single precision, mean + normal * stddev in double
-__global__ void random_normal_kernel(float* __restrict__ out, uint64_t n, uint32_t seed, double mean, double stddev) {
+// Box-Muller on the two halves of the 2-D hash of (i + seed, 1) (RandomNormal.py:14-24), all in single precision:
+// sqrt(-2*log(x)) * cos((2*PI_F)*y), then mean + normal*stddev with float mean / stddev as one fused multiply-add
+__global__ void random_normal_kernel(float* __restrict__ out, uint64_t n, uint32_t seed, float mean, float stddev) {
   for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
     uint32_t x = (uint32_t)(i + seed), y = 1u;
     hash_u32x2(x, y);
     const float fx = (float)x * kUnitScale, fy = (float)y * kUnitScale;
     const float normal = sqrtf(-2.0f * logf(fx)) * cosf((2.0f * 3.14159274101257f) * fy);
-    out[i] = (float)(mean + (double)normal * stddev);
+    out[i] = __builtin_fmaf(normal, stddev, mean);
   }
 }
 
 int launch_random_uniform(DeviceCtx* ctx, float* out, uint64_t n, uint32_t seed, double low, double high) {
   if (n == 0) return LNN_OK;
   if (!out) return set_error(LNN_ERR_INVALID, "random_uniform: null pointer");
-  hipLaunchKernelGGL(random_uniform_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, out, n, seed, high - low, low);
+  hipLaunchKernelGGL(random_uniform_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, out, n, seed, (float)high - (float)low, (float)low);
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }
@@ -599,7 +602,7 @@ int launch_random_uniform(DeviceCtx* ctx, float* out, uint64_t n, uint32_t seed,
 int launch_random_normal(DeviceCtx* ctx, float* out, uint64_t n, uint32_t seed, double mean, double stddev) {
   if (n == 0) return LNN_OK;
   if (!out) return set_error(LNN_ERR_INVALID, "random_normal: null pointer");
-  hipLaunchKernelGGL(random_normal_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, out, n, seed, mean, stddev);
+  hipLaunchKernelGGL(random_normal_kernel, grid_for(n, ctx->cus), dim3(256), 0, ctx->stream, out, n, seed, (float)mean, (float)stddev);
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }

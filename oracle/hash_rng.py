@@ -2,9 +2,12 @@
 
 The reference fills a parameter tensor with a counter hash: element i is a function of (uint32)(i + seed) alone
 (initializer/RandomUniform.py:13-27, RandomNormal.py:10-30), the hashes being the two PCG variants of its device
-helper text (CLKernelHelper.py:210-228).  All integer work is modulo 2**32 and reproduced bit for bit; the float
-stages follow the reference's expression types (single precision up to the Box-Muller value, double for the final
-scale and shift, because the reference formats mean / stddev / low / high as double literals).
+helper text (CLKernelHelper.py:210-228).  All integer work is modulo 2**32 and reproduced bit for bit.  The float
+stages are single precision throughout: the reference builds every kernel with -cl-single-precision-constant
+(minicl/CLDevice.py:93), so the mean / stddev / low / high it formats into the kernel text are float literals, and
+`u*(high-low)+low` (RandomUniform.py:20) and `mean+n*stddev` (RandomNormal.py:24) are float expressions.  The
+multiply-add is taken as contracted into one fused operation (OpenCL C allows it by default, and which one a vendor
+compiler emits cannot be read off the reference: at most one float ulp rides on that choice).
 
 Pinning.  The reference holds no output vector of these kernels and its OpenCL text cannot run here, so the
 integer stream is PARITY UNPINNED against the reference's device output.  What tests/test_oracle_hash_rng.py does
@@ -55,10 +58,28 @@ def _counter(n, seed):
     return (np.arange(n, dtype=np.uint64) + np.uint64(seed)) & M32
 
 
+def fma32(a, b, c):
+    """round_to_float32(a*b + c) with a single rounding, for float32 arrays / scalars.  The product of two
+    floats is exact in double; the double sum is corrected to round-to-odd with the exact error of the addition
+    (two-sum), after which the narrowing to float32 rounds as if it had seen the exact value."""
+    a, b, c = (np.asarray(v, np.float32).astype(np.float64) for v in (a, b, c))
+    p = a * b
+    s = p + c
+    bb = s - p
+    e = (p - (s - bb)) + (c - bb)
+    bits = np.atleast_1d(s).copy().view(np.int64)
+    inexact = (np.atleast_1d(e) != 0) & ((bits & 1) == 0) & np.isfinite(np.atleast_1d(s))
+    away = np.signbit(np.atleast_1d(e)) == np.signbit(np.atleast_1d(s))   # the exact value lies farther from zero than s
+    bits += np.where(inexact, np.where(away, 1, -1), 0)
+    return bits.view(np.float64).reshape(np.shape(s)).astype(np.float32)
+
+
 def random_uniform(n, seed, low=0.0, high=1.0):
-    """O[gid] = hash_float_uint(gid+seed)*(high-low)+low (RandomUniform.py:17-21)."""
+    """O[gid] = hash_float_uint(gid+seed)*(high-low)+low in single precision (RandomUniform.py:17-21,
+    CLDevice.py:93): span = (float)high - (float)low, then one fused multiply-add."""
     u = _unit(hash_u32(_counter(n, seed)))
-    return (u.astype(np.float64) * (float(high) - float(low)) + float(low)).astype(np.float32)
+    span = np.float32(high) - np.float32(low)
+    return fma32(u, span, np.float32(low))
 
 
 def random_normal(n, seed, mean=0.0, stddev=1.0):
@@ -68,4 +89,4 @@ def random_normal(n, seed, mean=0.0, stddev=1.0):
     with np.errstate(divide='ignore'):
         r = np.sqrt(np.float32(-2.0) * np.log(fx, dtype=np.float32), dtype=np.float32)
     normal = r * np.cos(np.float32(2.0 * np.float32(3.14159274101257)) * fy, dtype=np.float32)
-    return (float(mean) + normal.astype(np.float64) * float(stddev)).astype(np.float32)
+    return fma32(normal, np.float32(stddev), np.float32(mean))

@@ -90,6 +90,7 @@ def test_uniform_distribution_and_affine_map():
     assert stats.kstest(u[:200000].astype(np.float64), 'uniform').pvalue > 1e-3
     w = hash_rng.random_uniform(n, 12345, -0.25, 0.75)
     assert np.allclose(w, u.astype(np.float64) - 0.25, rtol=0, atol=1e-7)
+    assert w.dtype == np.float32
     # neighbouring seeds shift the stream by one element: the value depends on counter + seed only
     assert np.array_equal(hash_rng.random_uniform(100, 8)[:-1], hash_rng.random_uniform(100, 7)[1:])
 
@@ -105,3 +106,30 @@ def test_normal_distribution_and_affine_map():
     w = hash_rng.random_normal(n, 999, 1.5, 0.1)
     ok = np.isfinite(w)
     assert np.allclose(w[ok], 1.5 + 0.1 * hash_rng.random_normal(n, 999)[ok].astype(np.float64), rtol=0, atol=1e-6)
+
+
+def test_fma32_rounds_once():
+    """The single-precision affine stage of both initialisers is one fused multiply-add: compare the helper with
+    exact rational arithmetic, including products that sit exactly half-way between two floats before the addend
+    breaks the tie (where rounding the product or the double sum first would go the other way)."""
+    from fractions import Fraction
+    rng = np.random.default_rng(7)
+    a = rng.standard_normal(4000).astype(np.float32)
+    b = rng.standard_normal(4000).astype(np.float32)
+    c = (rng.standard_normal(4000) * 10.0 ** rng.integers(-12, 3, 4000)).astype(np.float32)
+    # ties: (1 + 2^-12)^2 = 1 + 2^-11 + 2^-24 is half-way between two floats near 1; a tiny addend decides
+    t = np.float32(1 + 2.0 ** -12)
+    a = np.concatenate([a, np.full(4, t, np.float32)])
+    b = np.concatenate([b, np.full(4, t, np.float32)])
+    c = np.concatenate([c, np.array([2.0 ** -60, -2.0 ** -60, 0.0, 2.0 ** -100], np.float32)])
+    got = hash_rng.fma32(a, b, c)
+
+    def nearest_f32(q):
+        lo = np.float32(float(q))                      # within one ulp of the answer
+        cands = {float(lo), float(np.nextafter(lo, np.float32(np.inf))), float(np.nextafter(lo, np.float32(-np.inf)))}
+        best = min(cands, key=lambda v: (abs(Fraction(v) - q), int(np.float32(v).view(np.uint32)) & 1))
+        return np.float32(best)
+
+    for x, y, z, g in zip(a.tolist(), b.tolist(), c.tolist(), got.tolist()):
+        assert np.float32(g) == nearest_f32(Fraction(x) * Fraction(y) + Fraction(z)), (x, y, z)
+    assert got[-4] != got[-3]      # the 2^-60 addends break the tie in opposite directions
