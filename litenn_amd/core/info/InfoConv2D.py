@@ -30,7 +30,7 @@ class InfoConv2D:
                 self.OH_T, self.OW_T = H * stride, W * stride
             else:
                 raise ValueError('Invalid padding value.')
-        elif isinstance(padding, int) and not isinstance(padding, bool):
+        elif isinstance(padding, int):
             self.PADL = self.PADT = self.PADR = self.PADB = padding
         elif isinstance(padding, Iterable):
             pads = tuple(int(x) for x in padding)

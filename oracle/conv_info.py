@@ -37,7 +37,7 @@ def info_conv2d(H, W, KH, KW, stride, dilation, padding):
         PADB = EKH - 1 - PADT
         OH_T = H * stride
         OW_T = W * stride
-    elif isinstance(padding, int) and not isinstance(padding, bool):
+    elif isinstance(padding, int):   # InfoConv2D.py:59 (a bool counts as an int there too)
         PADL = PADT = PADR = PADB = padding
     elif isinstance(padding, Iterable) and not isinstance(padding, str):
         padding = tuple(int(x) for x in padding)
