@@ -7,6 +7,26 @@ import litenn_amd.core as nc
 
 _seq = operator.methodcaller('_get_seq_id')
 
+# Per-sweep state for gradient functions that share an intermediate result (the fused convolution epilogue forms
+# its pre-activation gradient once for three gradient functions): a counter that identifies the running sweep
+# (None outside one) and callbacks run when the sweep ends, so nothing computed from one sweep's gradients is reused
+# by the next and nothing keeps gradient-sized tensors alive after it.
+_sweep = {'id': 0, 'active': None, 'cleanups': []}
+
+
+def current_sweep():
+    """Identifier of the backward() call in progress, or None outside one."""
+    return _sweep['active']
+
+
+def at_end_of_sweep(fn):
+    """Call fn() when the backward() call in progress returns (at once if none is running)."""
+    if _sweep['active'] is None:
+        fn()
+    else:
+        _sweep['cleanups'].append(fn)
+
+
 
 def backward(loss, stop_grad=None, grad_for_non_trainables=False, keep_gradient_for_non_trainables=False):
     """Reverse-mode sweep (same observable behaviour as backward.py:8-158).
@@ -21,6 +41,19 @@ def backward(loss, stop_grad=None, grad_for_non_trainables=False, keep_gradient_
     Tensors are visited in decreasing creation order; every registered
     gradient function adds into its input's gradient.
     """
+    if _sweep['active'] is not None:
+        raise Exception('backward() called from inside a gradient function')
+    _sweep['id'] += 1
+    _sweep['active'] = _sweep['id']
+    try:
+        _backward(loss, stop_grad, grad_for_non_trainables)
+    finally:
+        cleanups, _sweep['cleanups'], _sweep['active'] = _sweep['cleanups'], [], None
+        for fn in cleanups:
+            fn()
+
+
+def _backward(loss, stop_grad, grad_for_non_trainables):
     seeds = {}
     if isinstance(loss, dict):
         seeds = loss

@@ -81,61 +81,93 @@ class ModuleBase:
             raise Exception('You cannot assign sets to the Module')
 
     # ---- state --------------------------------------------------------------
-    def _state_items(self, prefix=''):
-        """Yields (dotted name, owner, key, value) for every saveable leaf."""
-        saveables = getattr(self, '_saveables', None)
-        for var in list(vars(self)):
-            if saveables is not None:
-                if var not in saveables:
-                    continue
-            elif var[0] == '_':
-                continue
-            yield from ModuleBase._walk(self.__dict__, var, getattr(self, var), f'{prefix}{var}')
+    # Layout of the flat state dict (what ModuleBase.py:131-199 writes, so files are interchangeable):
+    #   tensor      '<owner path>.<attr>'          -> ('np.ndarray', array)        owner path relative to the saved
+    #                                                                              module, '' for itself: '.kernel'
+    #   int, float, complex, str (bool included)
+    #               '<owner path>.<attr>' without a leading dot -> ('python-var', (class name, value))
+    #   list        '<owner path>.<attr>__len' without a leading dot -> bare int; elements follow as '<attr>[i]'
+    #   dict        elements as '<attr>[key]'; nothing for the dict itself
+    # Tuples, None, arrays and anything else are not part of the state.
+    def _visit_state(self, visit):
+        """Calls visit(kind, name, obj, setter) for every saveable leaf under this module; for kind 'list' the
+        return value says whether to descend into the elements."""
+        top = self
 
-    @staticmethod
-    def _walk(owner, key, obj, name):
-        if isinstance(obj, ModuleBase):
-            yield from obj._state_items(name + '.')
-        elif isinstance(obj, (list, tuple)):
-            yield (name + '__len', None, None, len(obj))
-            for i, el in enumerate(obj):
-                yield from ModuleBase._walk(obj, i, el, f'{name}[{i}]')
-        elif isinstance(obj, dict):
-            for k, el in obj.items():
-                yield from ModuleBase._walk(obj, k, el, f'{name}[{k}]')
-        elif isinstance(obj, (nn.Tensor, int, float, str, bool, np.ndarray)) or obj is None:
-            yield (name, owner, key, obj)
+        def walk(owner, obj, attr, setter):
+            if isinstance(obj, ModuleBase):
+                keep = getattr(obj, '_saveables', None)
+                for var in list(vars(obj)):
+                    if (var not in keep) if keep is not None else var[0] == '_':
+                        continue
+                    walk(obj, getattr(obj, var), var, lambda v, o=obj, n=var: setattr(o, n, v))
+            elif isinstance(obj, nn.Tensor):
+                visit('tensor', obj.get_name(top), obj, None)
+            elif isinstance(obj, list):
+                name = f'{owner.get_name(top)}.{attr}'.lstrip('.')
+                if visit('list', name, obj, None):
+                    for i, el in enumerate(obj):
+                        walk(owner, el, f'{attr}[{i}]', lambda v, o=obj, k=i: o.__setitem__(k, v))
+            elif isinstance(obj, dict):
+                for k in list(obj):
+                    walk(owner, obj[k], f'{attr}[{k}]', lambda v, o=obj, k=k: o.__setitem__(k, v))
+            elif isinstance(obj, (int, float, complex, str)):
+                visit('var', f'{owner.get_name(top)}.{attr}'.lstrip('.'), obj, setter)
+
+        walk(None, self, None, None)
 
     def dump_state(self):
-        """{dotted name: ('np.ndarray', array) | ('python-var', value)}."""
+        """{name: ('np.ndarray', array) | ('python-var', (class name, value)) | list length}."""
         state = {}
-        for name, owner, key, obj in self._state_items():
-            if isinstance(obj, nn.Tensor):
+
+        def visit(kind, name, obj, setter):
+            if kind == 'tensor':
                 state[name] = ('np.ndarray', obj.np())
-            elif owner is None:
-                state[name] = ('python-var', obj)
+            elif kind == 'list':
+                state[name + '__len'] = len(obj)
             else:
-                state[name] = ('python-var', obj)
+                state[name] = ('python-var', (obj.__class__.__name__, obj))
+            return True
+
+        self._visit_state(visit)
         return state
 
     def load_state(self, state_dict):
-        """Restore what matches; mismatches only warn."""
-        for name, owner, key, obj in self._state_items():
-            if owner is None:
-                if name in state_dict and state_dict[name][1] != obj:
-                    log.warning(f'{name}: saved length {state_dict[name][1]} != current {obj}')
-                continue
-            if name not in state_dict:
-                log.warning(f'{name} is not found in the saved state')
-                continue
-            kind, value = state_dict[name]
-            if isinstance(obj, nn.Tensor):
-                if kind != 'np.ndarray' or tuple(value.shape) != tuple(obj.shape):
-                    log.warning(f'{name}: saved value does not fit tensor shape {obj.shape}')
-                    continue
-                obj.set(value)
+        """Restores what matches by name, kind and shape / class; everything else only warns
+        (ModuleBase.py:146-199).  A list whose saved length differs is skipped with all its elements."""
+        def visit(kind, name, obj, setter):
+            if kind == 'list':
+                saved = state_dict.get(name + '__len', None)
+                if saved is None or saved != len(obj):
+                    log.warning(f'List {name} is not loaded, because length of list {len(obj)} != saved list len {saved}')
+                    return False
+                return True
+            what = 'Tensor' if kind == 'tensor' else 'Variable'
+            entry = state_dict.get(name, None)
+            if entry is None:
+                log.warning(f'{what} {name} is not loaded, because saved data is not found.')
+                return True
+            saved_kind, value = entry
+            if kind == 'tensor':
+                if saved_kind != 'np.ndarray':
+                    log.warning(f'Tensor {name} is not loaded, because saved type is {saved_kind}, but must be np.ndarray')
+                elif tuple(obj.shape) != value.shape:
+                    log.warning(f'Tensor {name} is not loaded, because saved Tensor shape is {value.shape}, '
+                                f'but must be {tuple(obj.shape)}')
+                else:
+                    obj.set(value)
+            elif saved_kind != 'python-var':
+                log.warning(f'Variable {name} is not loaded, because saved type is {saved_kind}, but must be python-var')
             else:
-                owner[key] = value
+                class_name, value = value
+                if class_name != obj.__class__.__name__:
+                    log.warning(f'Variable {name} is not loaded, because saved class_name is {class_name}, '
+                                f'but must be {obj.__class__.__name__}')
+                else:
+                    setter(value)
+            return True
+
+        self._visit_state(visit)
 
     def save(self, filepath):
         Path(filepath).write_bytes(pickle.dumps(self.dump_state(), 4))

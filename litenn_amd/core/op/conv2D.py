@@ -1,5 +1,6 @@
 import litenn_amd as nn
 import litenn_amd.core as nc
+from ..backward import at_end_of_sweep, current_sweep
 from ..hip import api, launch, ShallowMode
 
 
@@ -72,14 +73,26 @@ class _EpilogueGrad:
 
     def __init__(self, act, alpha):
         self.act, self.alpha = act, alpha
+        self.key, self.value = None, None      # key: (backward sweep, the dO tensor the value was formed from)
+
+    def _drop(self):
         self.key, self.value = None, None
+
+    def _cached(self, dO_t):
+        sweep = current_sweep()
+        return (sweep is not None and self.key is not None and self.key[0] == sweep and self.key[1] is dO_t)
 
     def _run(self, O_t, dO_t, want_pre, bias_grad):
         N, O, H, W = tuple(dO_t.shape)
         pre = None
         if want_pre:
             pre = nn.Tensor(dO_t.shape)
-            self.key, self.value = dO_t, pre
+            self.value = pre
+            # valid for the gradient functions of this sweep only: the next sweep's dO holds other values in the same
+            # tensor object, and the tensors are released when the sweep ends
+            if current_sweep() is not None:
+                self.key = (current_sweep(), dO_t)
+                at_end_of_sweep(self._drop)
         args = [O_t, dO_t]
         if pre is not None:
             args.append((pre, 'w'))
@@ -98,12 +111,18 @@ class _EpilogueGrad:
     def pre(self, O_t, dO_t):
         if self.act == api.ACT_NONE:
             return dO_t
-        if self.key is not dO_t:
-            self._run(O_t, dO_t, True, None)
-        return self.value
+        if self._cached(dO_t):
+            return self.value
+        self._run(O_t, dO_t, True, None)
+        value = self.value
+        if current_sweep() is None:
+            self._drop()
+        return value
 
     def bias(self, O_t, dO_t, bias_t):
-        self._run(O_t, dO_t, self.act != api.ACT_NONE and self.key is not dO_t, bias_t.get_grad())
+        self._run(O_t, dO_t, self.act != api.ACT_NONE and not self._cached(dO_t), bias_t.get_grad())
+        if current_sweep() is None:
+            self._drop()
 
 
 def conv2D_dI_gradfn(op, input_t, kernel_t, dO_t):

@@ -49,3 +49,15 @@ def nn_backend(request, monkeypatch, capsys):
     yield nn
     nn._test_fake = None
     _reset_registry()
+
+
+@pytest.fixture
+def nn_hip(capsys):
+    """`import litenn_amd as nn` on the real library and GPU 0 only (for cases too large for the numpy stand-in)."""
+    import litenn_amd as nn
+    from litenn_amd.core.hip import devices
+    devices._current_devices = None
+    devices._all_devices = None
+    nn._test_fake = None
+    yield nn
+    _reset_registry()

@@ -125,6 +125,40 @@ def test_conv2d_bias_act_equals_separate_ops(nn_backend):
         nc.op.conv2D_bias_act(nn.Tensor((1, 2, 4, 4)), nn.Tensor((3, 2, 3, 3)), leaky_relu_alpha=0.0)
 
 
+def test_fused_epilogue_backward_twice_over_one_graph(nn_backend):
+    """Two backward() sweeps over the same graph with grad_for_non_trainables=True accumulate: the output's own
+    gradient holds 1x then 2x the seed (the same tensor object both times), so the second sweep adds twice the first
+    sweep's contribution and every gradient of the fused node ends at three times a single sweep: its
+    pre-activation gradient must be formed anew from the current dO in each sweep.  (The chain of three separate
+    ops also keeps and re-propagates the gradients of its two intermediate tensors, so it is compared after the
+    first sweep only.)"""
+    nn = nn_backend
+    import litenn_amd.core as nc
+    rs = np.random.RandomState(12)
+    x_n = rs.randint(-3, 4, size=(2, 3, 9, 9)).astype(np.float32)
+    k_n = rs.randint(-3, 4, size=(4, 3, 3, 3)).astype(np.float32)
+    b_n = rs.randint(-3, 4, size=(4,)).astype(np.float32)
+    outs = []
+    for fused in (False, True):
+        x, k, b = nn.Tensor_from_value(x_n), nn.Tensor_from_value(k_n), nn.Tensor_from_value(b_n)
+        if fused:
+            y = nc.op.conv2D_bias_act(x, k, b, 1, 1, 'same', leaky_relu_alpha=0.5)
+        else:
+            y = nn.leaky_relu(nn.conv2D(x, k) + b.reshape((1, -1, 1, 1)), 0.5)
+        g_n = np.random.RandomState(1).randint(-4, 5, size=tuple(y.shape)).astype(np.float32)
+        nn.backward({y: g_n}, grad_for_non_trainables=True)
+        once = (x.get_grad().np().copy(), k.get_grad().np().copy(), b.get_grad().np().copy())
+        nn.backward({y: g_n}, grad_for_non_trainables=True)
+        twice = (x.get_grad().np(), k.get_grad().np(), b.get_grad().np())
+        if fused:
+            for o, t in zip(once, twice):
+                assert np.array_equal(t, 3 * o)
+        outs.append(once)
+        del x, k, b, y
+    for a, f in zip(*outs):
+        assert np.array_equal(a, f)
+
+
 def test_depthwise_conv2d_reference_style(nn_backend):
     """depthwise_conv2D_test (depthwise_conv2D.py:128-…): its grid of paddings,
     dilations, strides, kernel sizes and shapes, exact on integer-valued data,
@@ -554,6 +588,120 @@ def test_module_names_save_and_load(nn_backend, tmp_path):
         nn.optimizer.SGD(net.trainables())                  # already attached
 
 
+def test_state_dict_has_the_reference_layout(nn_backend, caplog):
+    """dump_state() / load_state() use the flat layout of ModuleBase.py:131-199, so checkpoints are
+    interchangeable with the reference: tensors under '<path>.<attr>' as ('np.ndarray', array) - '.attr' with the
+    leading dot for a tensor of the saved module itself -, python values as ('python-var', (class name, value)),
+    list lengths as a bare int under '<name>__len', dict elements under '<name>[key]'.  The expected dict below is
+    written out by hand from that layout, not produced by this package."""
+    nn = nn_backend
+
+    class Net(nn.Module):
+        def __init__(self):
+            self.blocks = [nn.Conv2D(2, 2, 3), nn.Conv2D(2, 2, 1, use_bias=False)]
+            self.head = nn.Dense(8, 3)
+            self.note = 'v1'
+            self.scale = nn.Tensor((2,), init=nn.initializer.Scalar(1.0))
+            self.d = {'a': 3, 'b': [1.5, 'x']}
+            self.flag = True
+            self.tup = (1, 2)            # tuples, None and arrays are not part of the state
+            self.nothing = None
+            self._hidden = 5             # underscore names are skipped unless listed as saveable
+
+    net = Net()
+    state = net.dump_state()
+    expect_vars = {'blocks__len': 2, 'note': ('python-var', ('str', 'v1')), 'd[a]': ('python-var', ('int', 3)),
+                   'd[b]__len': 2, 'd[b][0]': ('python-var', ('float', 1.5)), 'd[b][1]': ('python-var', ('str', 'x')),
+                   'flag': ('python-var', ('bool', True))}
+    expect_tensors = {'blocks[0].kernel': (2, 2, 3, 3), 'blocks[0].bias': (2,), 'blocks[1].kernel': (2, 2, 1, 1),
+                      'head.weight': (8, 3), 'head.bias': (3,), '.scale': (2,)}
+    assert set(state) == set(expect_vars) | set(expect_tensors)
+    for k, v in expect_vars.items():
+        assert state[k] == v and type(state[k]) is type(v), k
+    for k, shape in expect_tensors.items():
+        kind, arr = state[k]
+        assert kind == 'np.ndarray' and isinstance(arr, np.ndarray) and arr.shape == shape and arr.dtype == np.float32, k
+
+    # a state dict as the reference would have written it for the same model
+    rs = np.random.RandomState(3)
+    ref_state = {k: ('np.ndarray', rs.normal(0, 1, shape).astype(np.float32)) for k, shape in expect_tensors.items()}
+    ref_state.update({'blocks__len': 2, 'note': ('python-var', ('str', 'from-reference')),
+                      'd[a]': ('python-var', ('int', 11)), 'd[b]__len': 2, 'd[b][0]': ('python-var', ('float', 2.5)),
+                      'd[b][1]': ('python-var', ('str', 'y')), 'flag': ('python-var', ('bool', False))})
+    net.load_state(ref_state)
+    assert net.note == 'from-reference' and net.d == {'a': 11, 'b': [2.5, 'y']} and net.flag is False
+    assert np.array_equal(net.blocks[1].kernel.np(), ref_state['blocks[1].kernel'][1])
+    assert np.array_equal(net.scale.np(), ref_state['.scale'][1])
+    assert np.array_equal(net.head.weight.np(), ref_state['head.weight'][1])
+
+    # mismatches warn and leave the value alone: class name, tensor shape, kind, list length (elements skipped too)
+    caplog.clear()
+    bad = dict(ref_state)
+    bad['note'] = ('python-var', ('int', 7))
+    bad['d[a]'] = ('np.ndarray', np.zeros(1, np.float32))
+    bad['head.bias'] = ('np.ndarray', np.zeros((4,), np.float32))
+    bad['d[b]__len'] = 3
+    bad['d[b][0]'] = ('python-var', ('float', 99.0))
+    del bad['flag']
+    with caplog.at_level('WARNING', logger='litenn'):
+        net.load_state(bad)
+    assert net.note == 'from-reference' and net.d == {'a': 11, 'b': [2.5, 'y']} and net.flag is False
+    assert np.array_equal(net.head.bias.np(), ref_state['head.bias'][1])
+    text = caplog.text
+    for needle in ('note', 'd[a]', 'head.bias', 'List d[b]', 'flag'):
+        assert needle in text, needle
+
+    # optimizers: the iteration counter and the accumulators, keyed by the tensors' full names
+    opt = nn.optimizer.SGD(net.trainables(), momentum=0.5)
+    ostate = opt.dump_state()
+    assert ostate['iteration'] == ('python-var', ('int', 0))
+    assert set(ostate) == {'iteration'} | {f'._accs[{t.get_name()}]' for t in net.trainables()}
+    assert '._accs[Net.blocks[0].kernel]' in ostate
+    ostate['iteration'] = ('python-var', ('int', 41))
+    acc = np.full((2, 2, 3, 3), 0.25, np.float32)
+    ostate['._accs[Net.blocks[0].kernel]'] = ('np.ndarray', acc)
+    opt.load_state(ostate)
+    assert opt.iteration == 41 and isinstance(opt.iteration, int)
+    assert np.array_equal(opt._accs['Net.blocks[0].kernel'].np(), acc)
+
+
+def test_library_side_out_of_memory_evicts_pooled_blocks(nn_backend):
+    """A library call that reports out-of-memory for its own scratch is repeated after a pooled (idle) block has
+    been released, largest first, like a failed tensor allocation (CLDevice.py:134-164); with an empty pool the
+    error surfaces."""
+    nn = nn_backend
+    from litenn_amd.core.hip import api, launch
+    dev = nn.devices.get_current()[0]
+    for n in (1000, 3000, 2000):
+        nn.Tensor((n,)).np()                      # allocate, then drop: the blocks go to the pool
+    assert dev._total_buffers_pooled == 3
+    t = nn.Tensor_from_value(np.arange(4, dtype=np.float32))
+    calls = []
+
+    def scratch_hungry(device_index, ptr):
+        calls.append(dev._total_memory_pooled)
+        if len(calls) <= 2:
+            raise api.HipException(api.ERR_OOM, 'out of device memory for scratch')
+
+    launch(scratch_hungry, t)
+    assert calls == [24000, 12000, 4000]          # 3000 floats released first, then 2000
+    assert dev._total_buffers_pooled == 1
+
+    def always(device_index, ptr):
+        raise api.HipException(api.ERR_OOM, 'out of device memory for scratch')
+    with pytest.raises(api.HipException) as e:
+        launch(always, t)
+    assert e.value.code == api.ERR_OOM and dev._total_buffers_pooled == 0
+
+    def other(device_index, ptr):
+        raise api.HipException(api.ERR_INVALID, 'bad argument')
+    nn.Tensor((500,)).np()
+    with pytest.raises(api.HipException):
+        launch(other, t)
+    assert dev._total_buffers_pooled == 1         # other errors do not touch the pool
+    del t
+
+
 def test_training_step_matches_numpy(nn_backend):
     """Two-layer version of the encoder benchmark: conv(5x5, s2, p2) + bias ->
     leaky_relu(0.1) -> conv -> mean(square); SGD.  Compared with a float64
@@ -599,6 +747,72 @@ def test_training_step_matches_numpy(nn_backend):
     assert np.abs(c2.kernel.np() - W2).max() <= 1e-4 * np.abs(W2).max()
     assert np.abs(c2.bias.np() - B2).max() <= 1e-4 * max(np.abs(B2).max(), 1e-3)
     assert not x_t.has_grad()                          # the input is not trainable: its dX is skipped
+
+
+@pytest.mark.gpu
+def test_encoder_training_step_at_full_channel_widths(nn_hip):
+    """The 4-layer encoder of the training-step benchmark at its real widths (3 -> 64 -> 128 -> 256 -> 512, 5x5,
+    stride 2, pad 2, leaky_relu(0.1) between layers, loss mean(square), SGD lr 1e-3) on 2 images of 128 x 128: the
+    composition the single-layer tests do not see - fused bias / activation epilogues and their backward, strided
+    data gradients with all pixel classes in one launch, split-K forward / dgrad on the deep layers, the
+    multi-tensor SGD update - against a float64 restatement built from the oracle.  Two steps, so the second runs
+    on updated weights.  Loss, every kernel and bias gradient, and every updated kernel within 1e-4 (normalised)."""
+    from oracle import conv2d_fwd, conv2d_dx, conv2d_dw
+    from tests.gpu_util import say
+    nn = nn_hip
+    rs = np.random.RandomState(0)
+    chans = [3, 64, 128, 256, 512]
+    x = rs.uniform(-1, 1, (2, 3, 128, 128)).astype(np.float32)
+    ws = [rs.normal(0, np.sqrt(2.0 / (chans[i] * 25)), (chans[i + 1], chans[i], 5, 5)).astype(np.float32) for i in range(4)]
+    convs = [nn.Conv2D(chans[i], chans[i + 1], 5, stride=2, padding=2, kernel_initializer=nn.initializer.NumpyArray(ws[i]))
+             for i in range(4)]
+
+    class Enc(nn.Module):
+        def __init__(self):
+            self.convs = convs
+
+        def forward(self, t):
+            for i, c in enumerate(self.convs):
+                t = c(t)
+                if i < 3:
+                    t = nn.leaky_relu(t, 0.1)
+            return t
+
+    enc = Enc()
+    lr = 1e-3
+    opt = nn.optimizer.SGD(enc.trainables(), lr=lr)
+    x_t = nn.Tensor_from_value(x)
+    W = [w.astype(np.float64) for w in ws]
+    B = [np.zeros(c) for c in chans[1:]]
+    for step in range(2):
+        say(f'encoder step {step} at full widths')
+        opt.zero_grad()
+        loss = nn.square(enc(x_t)).mean()
+        loss.backward()
+        got_dw = [c.kernel.get_grad().np() for c in convs]
+        got_db = [c.bias.get_grad().np() for c in convs]
+        opt.step()
+        # float64 restatement
+        acts, zs = [x.astype(np.float64)], []
+        for i in range(4):
+            z = conv2d_fwd(acts[-1], W[i], 2, 1, 2) + B[i].reshape(1, -1, 1, 1)
+            zs.append(z)
+            acts.append(np.where(z >= 0, z, 0.1 * z) if i < 3 else z)
+        ref_loss = (zs[3] ** 2).mean()
+        assert abs(float(loss.np()[0]) - ref_loss) <= 1e-4 * abs(ref_loss)
+        dz = 2 * zs[3] / zs[3].size
+        for i in (3, 2, 1, 0):
+            dW, dB = conv2d_dw(acts[i], dz, W[i].shape, 2, 1, 2), dz.sum((0, 2, 3))
+            assert np.abs(got_dw[i] - dW).max() <= 1e-4 * np.abs(dW).max(), ('dW', step, i)
+            assert np.abs(got_db[i].reshape(-1) - dB).max() <= 1e-4 * np.abs(dB).max(), ('dB', step, i)
+            if i > 0:
+                dz = conv2d_dx(dz, W[i], acts[i].shape, 2, 1, 2) * np.where(zs[i - 1] >= 0, 1.0, 0.1)
+            W[i], B[i] = W[i] - lr * dW, B[i] - lr * dB
+        for i in range(4):
+            assert np.abs(convs[i].kernel.np() - W[i]).max() <= 1e-4 * np.abs(W[i]).max(), ('W', step, i)
+            # the update itself, not hidden under the weights' magnitude: v_new - v_old = -lr * g to fp32 rounding of v
+            assert np.abs(convs[i].bias.np().reshape(-1) - B[i]).max() <= 1e-4 * max(np.abs(B[i]).max(), 1e-12), ('b', step, i)
+    assert not x_t.has_grad()
 
 
 def test_unfold2d_operator(nn_backend):
