@@ -119,6 +119,16 @@ int lnn_bias_act_bwd_f32(int dev, int N, int O, int HW, const float* y, const fl
 /* dX (+)= dgrad(dY, W)                   conv2D.py:46-50 (the reference always accumulates) */
 int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* W,
                          float* dX, int beta);
+/* Which kernel family lnn_conv2d_dgrad_f32 uses for a geometry on a device with `compute_units` compute units
+ * (lnn_device_info reports them).  Host arithmetic only: works without a device.  No counterpart in the reference,
+ * whose data gradient always runs unfold + GeMM + transposes (conv2D.py:46-50); it lets a caller, or a test, see
+ * which code a shape exercises.  For LNN_DGRAD_PATH_VECTOR tile_info (7 values, may be NULL) receives the dY tile of
+ * one block: rows and columns brought to LDS, the largest extent the kernel's LDS plane holds, and the smallest /
+ * largest row and column any thread reads: {rows, cols, max_extent, min_row, min_col, max_row, max_col}. */
+#define LNN_DGRAD_PATH_MFMA_TABLE 0 /* implicit GEMM on the matrix cores, K = (o, tap) through a gather table */
+#define LNN_DGRAD_PATH_MFMA_TAP 1   /* implicit GEMM, tap-major K over channel-permuted weights (O % 32 == 0) */
+#define LNN_DGRAD_PATH_VECTOR 2     /* C <= 4: vector-ALU kernel, all pixel classes of a 32 x 32 tile per block */
+int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* path, int32_t* tile_info);
 /* dW (+)= wgrad(X, dY)                   conv2D.py:52-54 (the reference always accumulates) */
 int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
                          float* dW, int beta);
@@ -197,6 +207,9 @@ int lnn_adam_update_multi_f32(int dev, int count, const uint64_t* n, float* cons
  * hashes of CLKernelHelper.py:210-228).  The reference draws seed = np.random.randint(2^31) on the host.
  *   uniform: out[i] = u*(high-low) + low,           u = (float)hash(i+seed) * 2^-32   (can equal high)
  *   normal : out[i] = mean + stddev * sqrt(-2 ln u0) * cos(2 pi u1),  (u0,u1) = 2-D hash of (i+seed, 1) * 2^-32
+ * Both affine maps are single precision, one fused multiply-add on (float)low, (float)high - (float)low resp.
+ * (float)mean, (float)stddev: the reference compiles its kernels with -cl-single-precision-constant
+ * (minicl/CLDevice.py:93), so the bounds it formats into the kernel text are float literals there.
  * He / Glorot initialisers are these two with derived bounds (initializer/He.py:18-33, Glorot.py:20-35). */
 int lnn_random_uniform_f32(int dev, float* out, uint64_t n, uint32_t seed, double low, double high);
 int lnn_random_normal_f32(int dev, float* out, uint64_t n, uint32_t seed, double mean, double stddev);

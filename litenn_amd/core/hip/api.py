@@ -70,6 +70,7 @@ SIGNATURES = {
     'lnn_depthwise_conv2d_wgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_dgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_wgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
+    'lnn_conv2d_dgrad_path': [ctypes.POINTER(ConvDesc), _c_int, _c_int, ctypes.POINTER(_c_int), _i32arr],
     'lnn_unfold2d_f32': [_c_int] + [_c_int] * 14 + [_ptr, _ptr, _c_int],
     'lnn_transpose_f32': [_c_int, _c_int, _i32arr, _i32arr, _ptr, _ptr, _c_int],
     'lnn_ew_fwd_f32': [_c_int, _c_int, _c_u64, _ptr, _ptr, _c_f32, _c_int],
@@ -219,6 +220,18 @@ def conv2d_fwd_bias_act(dev, desc, X, W, bias, act, slope, Y):
 
 def conv2d_dgrad(dev, desc, dY, W, dX, beta=1):
     check(lib.lnn_conv2d_dgrad_f32(dev, ctypes.byref(desc), dY, W, dX, int(beta)))
+
+
+DGRAD_PATH_MFMA_TABLE, DGRAD_PATH_MFMA_TAP, DGRAD_PATH_VECTOR = 0, 1, 2
+
+
+def conv2d_dgrad_path(desc, beta, compute_units):
+    """(path, tile_info): the kernel family conv2d_dgrad picks for this geometry on a device with that many
+    compute units, and for the vector-ALU path its tile extents (host arithmetic, needs no device)."""
+    path = _c_int(-1)
+    info = (ctypes.c_int32 * 7)()
+    check(lib.lnn_conv2d_dgrad_path(ctypes.byref(desc), int(beta), int(compute_units), ctypes.byref(path), info))
+    return path.value, dict(zip(('rows', 'cols', 'max_extent', 'min_row', 'min_col', 'max_row', 'max_col'), list(info)))
 
 
 def conv2d_wgrad(dev, desc, X, dY, dW, beta=1):

@@ -5,6 +5,7 @@
 //   forward  Y [O  x P ] = W[O x CKK]        . im2col(X)[CKK x P]     P = N*OH*OW
 //   dgrad    dX[C  x Q ] = Wt[C x O*KK]      . im2rowT(dY)[O*KK x Q]  Q = N*IH*IW
 //   wgrad    dW[O  x CKK] = dY[O x P]        . im2row(X)[P x CKK]     (split over P)
+#include <algorithm>
 #include <vector>
 
 #include "common.hpp"
@@ -915,7 +916,7 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
 
 // The vector-ALU data gradient serves C <= 4, dilation 1, stride 1 (K = 1, 3, 5) or 2 (K = 3, 4, 5, 7), when there
 // are enough tiles to occupy the chip (a small problem is quicker on the MFMA path, whose tiles are finer).
-static bool small_dgrad_applies(const DeviceCtx* ctx, const ConvGeom& g) {
+static bool small_dgrad_applies(int cus, const ConvGeom& g) {
   if (!LNN_SMALL_DGRAD || g.C > 4 || g.D != 1 || g.KH != g.KW) return false;
   const int K = g.KH;
   const bool shape = (g.S == 1 && (K == 1 || K == 3 || K == 5)) || (g.S == 2 && (K == 3 || K == 4 || K == 5 || K == 7));
@@ -923,19 +924,13 @@ static bool small_dgrad_applies(const DeviceCtx* ctx, const ConvGeom& g) {
   const long long ph = (g.IH + g.S - 1) / g.S, pw = (g.IW + g.S - 1) / g.S;
   const long long blocks = ((ph + kDsTile - 1) / kDsTile) * ((pw + kDsTile - 1) / kDsTile) * g.N;
   if ((uint64_t)g.N * g.O * g.OHW * 4 > kMaxTensorBytes) return false;
-  return blocks * 2 >= ctx->cus;
+  return blocks * 2 >= cus;
 }
 
-constexpr int kNotHere = 1;   // launch_small_dgrad: a geometry it leaves to the general path (no error)
-static int launch_small_dgrad(DeviceCtx* ctx, const ConvGeom& g, const float* dY, const float* W, float* dX, int beta) {
-  const int K = g.KH, S = g.S, n_w = g.O * K * K * 4;
-  int st = ensure_workspace(ctx, (size_t)n_w * sizeof(float));
-  if (st != LNN_OK) return st;
-  float* wc = static_cast<float*>(ctx->ws);
-  hipLaunchKernelGGL(small_dgrad_weights, dim3((n_w + 255) / 256), dim3(256), 0, ctx->stream, wc, W, g.O, g.C, K, S);
-  LNN_HIP(hipGetLastError());
-  SmallDgradArgs a;
-  a.dY = dY; a.wc = wc; a.dX = dX;
+constexpr int kNotHere = 1;   // plan_small_dgrad: a geometry it leaves to the general path (no error)
+// Tile geometry of the vector-ALU data gradient (host only; the pointers of `a` are left alone).
+static int plan_small_dgrad(const ConvGeom& g, int beta, SmallDgradArgs& a, int* grid_x) {
+  const int K = g.KH, S = g.S;
   a.N = g.N; a.O = g.O; a.C = g.C; a.OH = g.OH; a.OW = g.OW; a.IH = g.IH; a.IW = g.IW;
   int ah[4], aw[4], lo_h = 1 << 30, lo_w = 1 << 30, hi_h = -(1 << 30), hi_w = -(1 << 30), max_ph = 0, max_pw = 0;
   for (int cls = 0; cls < 4; ++cls) {
@@ -960,15 +955,34 @@ static int launch_small_dgrad(DeviceCtx* ctx, const ConvGeom& g, const float* dY
     lo_w = std::min(lo_w, aw[cls] - (nkw - 1)); hi_w = std::max(hi_w, aw[cls]);
     max_ph = std::max(max_ph, a.ph[cls]); max_pw = std::max(max_pw, a.pw[cls]);
   }
-  if (max_ph == 0 || max_pw == 0) return LNN_OK;
+  *grid_x = 0;
+  a.th = a.tw = a.tiles_x = 0;
+  a.oh_base = a.ow_base = 0;
+  a.beta = beta ? 1 : 0;
+  if (max_ph == 0 || max_pw == 0) return LNN_OK;   // nothing to compute
   for (int cls = 0; cls < S * S; ++cls) { a.dh[cls] = ah[cls] - lo_h; a.dw[cls] = aw[cls] - lo_w; }
   a.oh_base = lo_h; a.ow_base = lo_w;
   a.th = kDsTile + hi_h - lo_h; a.tw = kDsTile + hi_w - lo_w;
   const int tmax = kDsTile + (K + S - 1) / S + 1;
   if (a.th > tmax || a.tw > tmax || a.tw > 64) return kNotHere;
   a.tiles_x = (max_pw + kDsTile - 1) / kDsTile;
-  a.beta = beta ? 1 : 0;
-  const dim3 grid((unsigned)(a.tiles_x * ((max_ph + kDsTile - 1) / kDsTile)), (unsigned)g.N), block(256);
+  *grid_x = a.tiles_x * ((max_ph + kDsTile - 1) / kDsTile);
+  return LNN_OK;
+}
+
+static int launch_small_dgrad(DeviceCtx* ctx, const ConvGeom& g, const float* dY, const float* W, float* dX, int beta) {
+  SmallDgradArgs a;
+  int grid_x = 0;
+  if (plan_small_dgrad(g, beta, a, &grid_x) == kNotHere) return kNotHere;
+  if (grid_x == 0) return LNN_OK;
+  const int K = g.KH, S = g.S, n_w = g.O * K * K * 4;
+  int st = ensure_workspace(ctx, (size_t)n_w * sizeof(float));
+  if (st != LNN_OK) return st;
+  float* wc = static_cast<float*>(ctx->ws);
+  hipLaunchKernelGGL(small_dgrad_weights, dim3((n_w + 255) / 256), dim3(256), 0, ctx->stream, wc, W, g.O, g.C, K, S);
+  LNN_HIP(hipGetLastError());
+  a.dY = dY; a.wc = wc; a.dX = dX;
+  const dim3 grid((unsigned)grid_x, (unsigned)g.N), block(256);
 #define LNN_DS(S_, K_)                                                                                        \
   do {                                                                                                        \
     if (g.C == 3) hipLaunchKernelGGL((small_dgrad_kernel<S_, K_, 3>), grid, block, 0, ctx->stream, a);         \
@@ -981,6 +995,37 @@ static int launch_small_dgrad(DeviceCtx* ctx, const ConvGeom& g, const float* dY
   return LNN_OK;
 }
 
+int conv_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* path, int32_t* tile_info) {
+  ConvGeom g;
+  int st = fill_geom(d, g);
+  if (st != LNN_OK) return st;
+  if (!path || compute_units <= 0) return set_error(LNN_ERR_INVALID, "conv2d_dgrad_path: null result pointer or no compute units");
+  *path = g.O % BK == 0 ? LNN_DGRAD_PATH_MFMA_TAP : LNN_DGRAD_PATH_MFMA_TABLE;
+  if (tile_info)
+    for (int i = 0; i < 7; ++i) tile_info[i] = 0;
+  if (small_dgrad_applies(compute_units, g)) {
+    SmallDgradArgs a;
+    int grid_x = 0;
+    if (plan_small_dgrad(g, beta, a, &grid_x) != kNotHere) {
+      *path = LNN_DGRAD_PATH_VECTOR;
+      if (tile_info && grid_x > 0) {
+        const int K = g.KH, S = g.S;
+        int lo_r = 1 << 30, lo_c = 1 << 30, hi_r = -1, hi_c = -1;
+        for (int cls = 0; cls < S * S; ++cls) {
+          const int nkh = ds_nk(K, S, cls / S), nkw = ds_nk(K, S, cls % S);
+          if (nkh == 0 || nkw == 0) continue;
+          // thread (ty, tx), ty, tx < 16, reads rows dh + 2*ty - (nkh-1) ... + nkh, likewise columns
+          lo_r = std::min(lo_r, a.dh[cls] - (nkh - 1)); hi_r = std::max(hi_r, a.dh[cls] + 2 * 15 + 1);
+          lo_c = std::min(lo_c, a.dw[cls] - (nkw - 1)); hi_c = std::max(hi_c, a.dw[cls] + 2 * 15 + 1);
+        }
+        tile_info[0] = a.th; tile_info[1] = a.tw; tile_info[2] = kDsTile + (K + S - 1) / S + 1;
+        tile_info[3] = lo_r; tile_info[4] = lo_c; tile_info[5] = hi_r; tile_info[6] = hi_c;
+      }
+    }
+  }
+  return LNN_OK;
+}
+
 int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta) {
   ConvGeom full;
   int st = fill_geom(d, full);
@@ -988,7 +1033,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   if (!dY || !W || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
   const int S = full.S;
   if (S > 15) return set_error(LNN_ERR_UNSUPPORTED, "conv2d_dgrad: stride > 15");
-  if (small_dgrad_applies(ctx, full)) {
+  if (small_dgrad_applies(ctx->cus, full)) {
     st = launch_small_dgrad(ctx, full, dY, W, dX, beta);
     if (st != kNotHere) return st;
   }
@@ -1049,7 +1094,13 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   const int unit_cols = cls[0].M > 64 ? 32 : (cls[0].M > 32 ? 64 : 128);
   const long long units0 = (long long)((cls[0].M + 127) / 128) * ((cls[0].Ncols + unit_cols - 1) / unit_cols);
   if (nc > kMaxBatch || units0 >= 4ll * ctx->cus) {
-    // one after the other, each with the whole chip
+    // one after the other, each with the whole chip.  All the scratch any class needs (its permuted weights,
+    // then partial sums) is reserved before the first launch: a failed allocation then leaves dX untouched, so
+    // the caller may free memory and repeat the call.
+    size_t w_most = 0;
+    for (int i = 0; i < nc; ++i) w_most = std::max<size_t>(w_most, ((size_t)(cls[i].bytesW ? cls[i].bytesW : 4) + 255) & ~(size_t)255);
+    st = ensure_workspace(ctx, w_most + part_bytes);
+    if (st != LNN_OK) return st;
     for (int i = 0; i < nc; ++i) {
       ConvArgs& a = cls[i];
       if (tap) {
@@ -1096,10 +1147,7 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");
-  st = reserve_tables(ctx, 1);
-  if (st != LNN_OK) return st;
-  st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);
-  if (st != LNN_OK) return st;
+  a.tab = nullptr;
   const ConvGeom& g = a.g;
   a.X = X; a.W = dY; a.Out = dW;
   a.bytesX = (uint32_t)((uint64_t)g.N * g.C * g.IHW * 4);
@@ -1117,6 +1165,11 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
     if (vec && g.S == 1 && g.OW % 4 == 0 && cols_inside) return launch_by_m<PASS_WGRAD_TAP4>(ctx, a, true);
     return launch_by_m<PASS_WGRAD_TAP>(ctx, a, vec);
   }
+  // the table-driven kernel: per-column gather entries
+  st = reserve_tables(ctx, 1);
+  if (st != LNN_OK) return st;
+  st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);
+  if (st != LNN_OK) return st;
   return launch_by_m<PASS_WGRAD>(ctx, a, vec);
 }
 

@@ -42,7 +42,14 @@ int hip_fail(hipError_t e, const char* what) {
 }
 
 static int device_count_raw(int* n) {
+  // the number of devices of a process does not change once it has been read successfully
+  static int known = -1;
+  if (known > 0) {
+    *n = known;
+    return LNN_OK;
+  }
   hipError_t e = hipGetDeviceCount(n);
+  if (e == hipSuccess && *n > 0) known = *n;
   if (e == hipErrorNoDevice) {
     (void)hipGetLastError();
     *n = 0;
@@ -312,6 +319,10 @@ int lnn_depthwise_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const floa
 int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta) {
   CTX(dev);
   return launch_conv_dgrad(ctx, d, dY, W, dX, beta);
+}
+
+int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* path, int32_t* tile_info) {
+  return conv_dgrad_path(d, beta, compute_units, path, tile_info);
 }
 
 int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {

@@ -1,0 +1,69 @@
+"""Host-side plan of the data gradient (lnn_conv2d_dgrad_path: no device needed).  For every geometry the
+vector-ALU kernel accepts, the dY tile one block brings to LDS must fit the kernel's LDS plane and every window a
+thread reads must lie inside the rows / columns that were brought in; the selection between the kernel families
+must follow the documented rules, whatever the compute-unit count of the device."""
+import itertools
+
+from litenn_amd.core.hip import api
+from oracle import info_conv2d
+
+SUPPORTED = {1: (1, 3, 5), 2: (3, 4, 5, 7)}
+
+
+def _desc(N, C, H, W, O, K, s, d, padding):
+    ci = info_conv2d(H, W, K, K, s, d, padding)
+    return api.conv_desc(N, C, H, W, O, K, K, ci.OH, ci.OW, ci.PADL, ci.PADT, s, d)
+
+
+def test_vector_path_tiles_stay_inside_their_lds_plane():
+    n_vec = 0
+    for s, ks in SUPPORTED.items():
+        for K in ks:
+            pads = ['same', 'valid'] + list(range(0, K + 1)) + [(0, K, 1, 0), (K, 0, 0, 2), (1, 2, 3, 0)]
+            for padding, (H, W), C, beta in itertools.product(pads, [(70, 66), (64, 64), (33, 97), (224, 224)],
+                                                               [1, 3, 4], [0, 1]):
+                if padding == 'valid' and min(H, W) < K:
+                    continue
+                path, t = api.conv2d_dgrad_path(_desc(512, C, H, W, 8, K, s, 1, padding), beta, 256)
+                # every supported (S, K) has taps in every pixel class, so nothing falls back at this batch size
+                assert path == api.DGRAD_PATH_VECTOR, (s, K, padding, H, W, C, beta)
+                n_vec += 1
+                tag = (s, K, padding, H, W, C, beta, t)
+                assert 0 < t['rows'] <= t['max_extent'] and 0 < t['cols'] <= t['max_extent'], tag
+                assert t['cols'] <= 64, tag                          # one lane of a wavefront per tile column
+                assert t['max_extent'] == 32 + (K + s - 1) // s + 1, tag
+                assert t['min_row'] >= 0 and t['min_col'] >= 0, tag
+                assert t['max_row'] < t['rows'] and t['max_col'] < t['cols'], tag
+    assert n_vec > 1000
+
+
+def test_selection_rules():
+    big = dict(N=64, H=70, W=66, O=16)
+
+    def path(C, K, s, d=1, padding='same', N=big['N'], cus=256, beta=1, O=big['O']):
+        return api.conv2d_dgrad_path(_desc(N, C, big['H'], big['W'], O, K, s, d, padding), beta, cus)[0]
+
+    assert path(3, 7, 2, padding=3) == api.DGRAD_PATH_VECTOR
+    assert path(4, 3, 1) == api.DGRAD_PATH_VECTOR
+    assert path(5, 3, 1) == api.DGRAD_PATH_MFMA_TABLE             # more than four channels
+    assert path(3, 3, 1, d=2) == api.DGRAD_PATH_MFMA_TABLE        # dilation
+    assert path(3, 5, 3, padding=2) == api.DGRAD_PATH_MFMA_TABLE  # stride 3
+    assert path(3, 7, 1) == api.DGRAD_PATH_MFMA_TABLE             # 7 x 7 at stride 1
+    assert path(3, 3, 1, O=32) == api.DGRAD_PATH_VECTOR           # C decides, not O
+    assert path(8, 3, 1, O=32) == api.DGRAD_PATH_MFMA_TAP
+    # too few tiles for the chip: 3 x 3 tiles of 32 x 32 per 70 x 66 image at stride 1
+    assert path(3, 3, 1, N=14, cus=256) == api.DGRAD_PATH_MFMA_TABLE       # 126 blocks < 128
+    assert path(3, 3, 1, N=15, cus=256) == api.DGRAD_PATH_VECTOR           # 135 blocks
+    assert path(3, 3, 1, N=14, cus=128) == api.DGRAD_PATH_VECTOR           # the same problem on a smaller part
+    assert path(3, 3, 1, N=1, cus=304) == api.DGRAD_PATH_MFMA_TABLE
+
+
+def test_bad_arguments():
+    import pytest
+    d = _desc(4, 3, 16, 16, 4, 3, 1, 1, 'same')
+    with pytest.raises(api.HipException) as e:
+        api.conv2d_dgrad_path(d, 0, 0)
+    assert e.value.code == api.ERR_INVALID
+    bad = api.conv_desc(1, 1, 4, 4, 1, 3, 3, 4, 4, 1, 1, 0, 1)
+    with pytest.raises(api.HipException):
+        api.conv2d_dgrad_path(bad, 0, 256)
