@@ -133,6 +133,20 @@ int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units,
 int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
                          float* dW, int beta);
 
+/* The same computation as lnn_conv2d_wgrad_f32, bit for bit, without any device allocation.  It has no counterpart
+ * in the reference (whose buffers all come from clCreateBuffer at run time); it is for callers that cannot call
+ * hipMalloc: code under HIP graph capture, tight serving or training loops, harnesses that forbid allocation.
+ * The split-K partial sums (and the gather table of geometries whose channel count does not fill the pixel-major
+ * tiles) live in a fixed device array of LNN_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until
+ * the process ends.  A problem that needs more returns LNN_ERR_UNSUPPORTED and launches nothing; on a 256-CU
+ * device the partial sums never exceed 32 MiB, so only the added table of an unusually shaped problem can.
+ * The one-time set-up of a device (stream, address of the array) happens in the first call of ANY entry point on
+ * that device; after it this function calls no hipMalloc / hipFree or other allocating routine.  All calls on one
+ * GPU share the array: calls that overlap in time on one GPU (from two threads) race. */
+#define LNN_NOALLOC_SCRATCH_BYTES (32u << 20)
+int lnn_conv2d_wgrad_noalloc_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
+                                 float* dW, int beta);
+
 /* ---- depthwise convolution (one KH x KW filter per channel; K is [C,KH,KW], desc.O must equal desc.C).
  * Y (+)= depthwise(X, K)                 depthwise_conv2D.py:74-96  (O_depthwise_krn)
  * dX (+)= its data gradient              depthwise_conv2D.py:98-124 (dI_depthwise_krn; the reference always accumulates)

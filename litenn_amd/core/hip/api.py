@@ -70,6 +70,7 @@ SIGNATURES = {
     'lnn_depthwise_conv2d_wgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_dgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_wgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
+    'lnn_conv2d_wgrad_noalloc_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_dgrad_path': [ctypes.POINTER(ConvDesc), _c_int, _c_int, ctypes.POINTER(_c_int), _i32arr],
     'lnn_unfold2d_f32': [_c_int] + [_c_int] * 14 + [_ptr, _ptr, _c_int],
     'lnn_transpose_f32': [_c_int, _c_int, _i32arr, _i32arr, _ptr, _ptr, _c_int],
@@ -220,6 +221,15 @@ def conv2d_fwd_bias_act(dev, desc, X, W, bias, act, slope, Y):
 
 def conv2d_dgrad(dev, desc, dY, W, dX, beta=1):
     check(lib.lnn_conv2d_dgrad_f32(dev, ctypes.byref(desc), dY, W, dX, int(beta)))
+
+
+NOALLOC_SCRATCH_BYTES = 32 << 20
+
+
+def conv2d_wgrad_noalloc(dev, desc, X, dY, dW, beta=1):
+    """conv2d_wgrad without device allocation: scratch is a fixed array inside the library (NOALLOC_SCRATCH_BYTES);
+    problems that need more raise ERR_UNSUPPORTED."""
+    check(lib.lnn_conv2d_wgrad_noalloc_f32(dev, ctypes.byref(desc), X, dY, dW, int(beta)))
 
 
 DGRAD_PATH_MFMA_TABLE, DGRAD_PATH_MFMA_TAP, DGRAD_PATH_VECTOR = 0, 1, 2

@@ -23,6 +23,11 @@ struct DeviceCtx {
   size_t ws_bytes = 0;
   // gather tables, one per (geometry, kind)
   std::map<std::array<int, 16>, KEntry*> tables;
+  // this device's copy of the library's fixed scratch array (device address, looked up once per device)
+  void* static_ws = nullptr;
+  // true while an allocation-free entry point runs: ws / ws_bytes then describe the fixed array, requests that do
+  // not fit fail instead of allocating, and gather tables are carved from its tail instead of being cached
+  bool no_alloc = false;
 };
 
 int set_error(int code, const std::string& msg);

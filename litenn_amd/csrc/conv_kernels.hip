@@ -578,7 +578,7 @@ static int fill_geom(const lnn_conv2d_desc* d, ConvGeom& g) {
 // Bound the table cache: before a call that may add up to n tables, drop everything once the work queued so
 // far is done.  Never in the middle of a call: its earlier tables must stay valid until it has launched.
 static int reserve_tables(DeviceCtx* ctx, size_t n) {
-  if (ctx->tables.size() + n <= 256) return LNN_OK;
+  if (ctx->no_alloc || ctx->tables.size() + n <= 256) return LNN_OK;
   LNN_HIP(hipStreamSynchronize(ctx->stream));
   for (auto& kv : ctx->tables) (void)hipFree(kv.second);
   ctx->tables.clear();
@@ -593,6 +593,18 @@ static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const PixelCla
   const int Kpad = mode == 2 ? K + 2 : ((K + BK - 1) / BK) * BK + BK;
   const std::array<int, 16> key = {mode, g.C,  g.O,  g.KH, g.KW,   g.D,    g.IH,  g.IW,
                                    g.OH, g.OW, g.S, g.PADT, g.PADL, pc.rh, pc.rw, 0};
+  if (ctx->no_alloc) {
+    // from the tail of the fixed scratch array, built anew by every call (the next call reuses the memory)
+    const size_t tb = ((size_t)Kpad * sizeof(KEntry) + 255) & ~(size_t)255;
+    if (tb > ctx->ws_bytes)
+      return set_error(LNN_ERR_UNSUPPORTED, "conv2d: the gather table does not fit the allocation-free entry point's scratch");
+    ctx->ws_bytes -= tb;
+    KEntry* t = reinterpret_cast<KEntry*>(static_cast<char*>(ctx->ws) + ctx->ws_bytes);
+    hipLaunchKernelGGL(build_ktable, dim3((Kpad + 255) / 256), dim3(256), 0, ctx->stream, t, K, Kpad, mode, g, pc);
+    LNN_HIP(hipGetLastError());
+    *out = t;
+    return LNN_OK;
+  }
   auto it = ctx->tables.find(key);
   if (it != ctx->tables.end()) {
     *out = it->second;

@@ -23,6 +23,13 @@ int launch_update_multi(DeviceCtx*, int, int, const uint64_t*, float* const*, co
 int launch_bias_act_bwd(DeviceCtx*, int, int, int, const float*, const float*, int, float, float*, float*, int);
 int launch_random_normal(DeviceCtx*, float*, uint64_t, uint32_t, double, double);
 
+// Scratch of the allocation-free entry point (lnn_conv2d_wgrad_noalloc_f32): split-K partial sums and, for
+// geometries that need one, the gather table.  Every GPU the library runs on holds its own copy of this array
+// from the time the code object is loaded until the process ends.  In host code the name `scratch` is only a
+// handle for hipGetSymbolAddress; the device address kept in DeviceCtx::static_ws is what kernels receive.
+constexpr size_t kStaticScratchBytes = LNN_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 static thread_local std::string g_error;
 constexpr int kMaxDevices = 64;
 static DeviceCtx g_ctx[kMaxDevices];
@@ -95,6 +102,17 @@ DeviceCtx* get_ctx(int dev, int* status) {
         *status = hip_fail(e, "hipStreamCreateWithFlags");
         return nullptr;
       }
+      // device `dev` is current here: its copy of the scratch array
+      void* sp = nullptr;
+      e = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || sp == nullptr) {
+        (void)hipStreamDestroy(c->stream);
+        c->stream = nullptr;
+        *status = e != hipSuccess ? hip_fail(e, "hipGetSymbolAddress(scratch)")
+                                  : set_error(LNN_ERR_HIP, "hipGetSymbolAddress(scratch) returned a null address");
+        return nullptr;
+      }
+      c->static_ws = sp;
       c->index = dev;
       c->cus = prop.multiProcessorCount;
       c->ready = true;
@@ -106,6 +124,9 @@ DeviceCtx* get_ctx(int dev, int* status) {
 
 int ensure_workspace(DeviceCtx* ctx, size_t bytes) {
   if (bytes <= ctx->ws_bytes) return LNN_OK;
+  if (ctx->no_alloc)
+    return set_error(LNN_ERR_UNSUPPORTED, "this problem needs " + std::to_string(bytes) + " bytes of scratch; the allocation-free "
+                     "entry point has " + std::to_string(ctx->ws_bytes) + " (use the allocating entry point)");
   // earlier launches may still read the old buffer
   LNN_HIP(hipStreamSynchronize(ctx->stream));
   if (ctx->ws) {
@@ -327,6 +348,31 @@ int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units,
 
 int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
   CTX(dev);
+  return launch_conv_wgrad(ctx, d, X, dY, dW, beta);
+}
+
+namespace {
+// For the duration of one call the device's scratch is the fixed array (single-threaded callers per device).
+struct FixedScratch {
+  DeviceCtx* c;
+  void* ws;
+  size_t bytes;
+  explicit FixedScratch(DeviceCtx* ctx) : c(ctx), ws(ctx->ws), bytes(ctx->ws_bytes) {
+    c->ws = c->static_ws;
+    c->ws_bytes = kStaticScratchBytes;
+    c->no_alloc = true;
+  }
+  ~FixedScratch() {
+    c->ws = ws;
+    c->ws_bytes = bytes;
+    c->no_alloc = false;
+  }
+};
+}  // namespace
+
+int lnn_conv2d_wgrad_noalloc_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
+  CTX(dev);
+  FixedScratch fixed(ctx);
   return launch_conv_wgrad(ctx, d, X, dY, dW, beta);
 }
 
