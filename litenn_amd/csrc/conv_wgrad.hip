@@ -1,0 +1,39 @@
+// Convolution weight gradient (split over the output pixels, deterministic slice reduction).
+#include "conv_common.hpp"
+
+namespace lnn {
+
+int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
+  ConvArgs a;
+  a.ws_used = 0;
+  a.post = PostOp{nullptr, 0, 0.0f};
+  int st = fill_geom(d, a.g);
+  if (st != LNN_OK) return st;
+  if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");
+  a.tab = nullptr;
+  const ConvGeom& g = a.g;
+  a.X = X; a.W = dY; a.Out = dW;
+  a.bytesX = (uint32_t)((uint64_t)g.N * g.C * g.IHW * 4);
+  a.bytesW = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
+  a.bytesOut = (uint32_t)((uint64_t)g.O * g.C * g.KK * 4);
+  a.M = g.O; a.Ncols = g.C * g.KK; a.K = g.N * g.OHW;
+  a.beta = beta ? 1 : 0;
+  // pixel-major loaders when the channels fill whole units of the tile shape chosen for O
+  const int unit = g.O > 64 ? 32 : (g.O > 32 ? 64 : 128);
+  // ... and a K step of pixels never wraps around an image more than once
+  const bool vec = g.OHW % 4 == 0 && aligned16(dY);
+  if (g.C % unit == 0 && BK / g.OW + 1 <= g.OH) {
+    // every tap of every output pixel reads a column inside the image: the gather can move four pixels at a time
+    const bool cols_inside = g.PADL == 0 && g.OW - 1 + (g.KW - 1) * g.D <= g.IW - 1;
+    if (vec && g.S == 1 && g.OW % 4 == 0 && cols_inside) return launch_by_m<PASS_WGRAD_TAP4>(ctx, a, true);
+    return launch_by_m<PASS_WGRAD_TAP>(ctx, a, vec);
+  }
+  // the table-driven kernel: per-column gather entries
+  st = reserve_tables(ctx, 1);
+  if (st != LNN_OK) return st;
+  st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);
+  if (st != LNN_OK) return st;
+  return launch_by_m<PASS_WGRAD>(ctx, a, vec);
+}
+
+}  // namespace lnn
