@@ -29,14 +29,21 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_MFMA_TFLOPS = 157.3   # 256 CU x 2.4 GHz x 256 flop/clk/CU
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch from hardware counters (FETCH_SIZE + WRITE_SIZE, each scaled by its reading for a plain
-# copy of known size), measured separately under rocprofv3 --pmc; keyed by workload and pass.  A pass that has
-# not been measured reports null.
-MEASURED_TRAFFIC_BYTES = {
-    'cfg3_vgg3x3': {'fwd': 316.5e6 + 4.5e6, 'dX': 384.6e6 + 4.5e6, 'dW': 236.3e6 + 40.5e6},   # + weight permutation / slice reduction
-    'cfg2_matmul': {'fwd': 1208.2e6, 'dA': 1275.5e6, 'dB': 1275.3e6},
-    'cfgD_depthwise': {'fwd': 206.1e6, 'dX': 309.8e6, 'dK': 205.7e6 + 0.2e6},
-}
+def measured_traffic():
+    """HBM bytes per launch from hardware counters (FETCH_SIZE + WRITE_SIZE, each scaled by its reading for a plain
+    copy of known size), measured separately under rocprofv3 --pmc: the `traffic_bytes <workload> <pass> <bytes>`
+    lines of the committed summaries profiles/*_hbm_traffic_pmc.txt.  A pass that has not been measured reports null."""
+    import glob
+    table = {}
+    for path in sorted(glob.glob(os.path.join(ROOT, 'profiles', '*_hbm_traffic_pmc.txt'))):
+        for line in open(path):
+            f = line.split()
+            if len(f) == 4 and f[0] == 'traffic_bytes':
+                table.setdefault(f[1], {})[f[2]] = float(f[3])
+    return table
+
+
+MEASURED_TRAFFIC_BYTES = measured_traffic()
 
 CONV_CONFIGS = {
     # name: (x shape, w shape, stride, dilation, padding, seed)
@@ -106,6 +113,7 @@ def rel_err(got, ref):
 
 
 SETTLE_S = 0.25
+CPU_OPENCL = 'not probed'
 
 
 def settle(step, sync):
@@ -119,6 +127,60 @@ def settle(step, sync):
         sync()
 
 
+def timed_steps(step, sync, steps, warmup):
+    """The measurement protocol of every workload: (cold) `warmup` steps then `steps` timed steps straight after
+    start-up, as a caller who does nothing special sees them; then the same again after settle().  Returns
+    (ms per step settled, ms per step cold)."""
+    out = []
+    for settled in (False, True):
+        if settled:
+            settle(step, sync)
+        for _ in range(warmup):
+            step()
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        sync()
+        out.append((time.perf_counter() - t0) * 1e3 / steps)
+    return out[1], out[0]
+
+
+def probe_cpu_opencl():
+    """Looks for a CPU OpenCL device (PoCL or any other) through the ICD loader, the way the reference binds
+    OpenCL (find_library('OpenCL'), clGetPlatformIDs, clGetDeviceIDs; minicl/api/OpenCL/OpenCL.py:16-23, 214-310).
+    Runs in a child process so that a misbehaving ICD cannot disturb the measurement.  Returns a sentence."""
+    import subprocess
+    code = r"""
+import ctypes, ctypes.util
+name = ctypes.util.find_library('OpenCL')
+if not name:
+    print('no OpenCL ICD loader on this host'); raise SystemExit
+cl = ctypes.CDLL(name)
+n = ctypes.c_uint(0)
+if cl.clGetPlatformIDs(0, None, ctypes.byref(n)) != 0 or n.value == 0:
+    print('no CPU OpenCL device on this host (the ICD loader lists no platform)'); raise SystemExit
+plats = (ctypes.c_void_p * n.value)()
+cl.clGetPlatformIDs(n.value, plats, None)
+found = []
+for p in plats:
+    buf = ctypes.create_string_buffer(256)
+    cl.clGetPlatformInfo(ctypes.c_void_p(p), 0x0902, 256, buf, None)
+    m = ctypes.c_uint(0)
+    rc = cl.clGetDeviceIDs(ctypes.c_void_p(p), ctypes.c_ulong(2), 0, None, ctypes.byref(m))   # CL_DEVICE_TYPE_CPU
+    if rc == 0 and m.value > 0:
+        found.append(buf.value.decode())
+print('CPU OpenCL device present on platform(s): ' + ', '.join(found) if found else
+      'no CPU OpenCL device on this host (%d platform(s) listed by the ICD loader, none with a CPU device)' % n.value)
+"""
+    try:
+        r = subprocess.run([sys.executable, '-c', code], capture_output=True, text=True, timeout=60)
+        lines = [l for l in r.stdout.strip().splitlines() if l.strip()]
+        return lines[-1] if lines else f'no CPU OpenCL device on this host (probe ended with status {r.returncode})'
+    except Exception as e:   # noqa: BLE001
+        return f'no CPU OpenCL device on this host (probe failed: {type(e).__name__})'
+
+
 def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
     xs, ws, s, d, padding, seed = CONV_CONFIGS[name]
     x, w, dy, ci = conv_tensors(xs, ws, s, d, padding, seed)
@@ -130,25 +192,33 @@ def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
     bytes_pass = {'fwd': 4.0 * (nx + nw + ny), 'dX': 4.0 * (ny + nw + 2 * nx), 'dW': 4.0 * (nx + ny + 2 * nw)}
     X, W, dY = Dev(api, x), Dev(api, w), Dev(api, dy)
     Y, dX, dW = Dev(api, shape=dy.shape), Dev(api, shape=xs), Dev(api, shape=ws)
-    passes = {
-        'fwd': lambda: api.conv2d_fwd(0, desc, X.ptr, W.ptr, Y.ptr, 0),
-        'dX': lambda: api.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, 1),
-        'dW': lambda: api.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW.ptr, 1),
-    }
+    # As a training step runs it: the weights change once per step, so the copy in the kernels' layout that forward
+    # and data gradient share (where the geometry's kernels read one) is made once per step, inside the forward pass.
+    fwd_pw, dx_pw = api.conv2d_weights_plan(desc, api.PASS_FWD), api.conv2d_weights_plan(desc, api.PASS_DGRAD)
+    in_place = KH * KW == 1                      # a 1x1 kernel already has the layout
+    Wp = W if in_place or not (fwd_pw or dx_pw) else Dev(api, shape=(O, KH * KW, C))
+
+    def p_fwd():
+        if (fwd_pw or dx_pw) and not in_place:
+            api.conv2d_permute_weights(0, desc, W.ptr, api.W_OIHW, Wp.ptr)
+        if fwd_pw:
+            api.conv2d_fwd_pw(0, desc, X.ptr, Wp.ptr, None, api.ACT_NONE, 0.0, Y.ptr, 0)
+        else:
+            api.conv2d_fwd(0, desc, X.ptr, W.ptr, Y.ptr, 0)
+
+    def p_dx():
+        if dx_pw:
+            api.conv2d_dgrad_pw(0, desc, dY.ptr, Wp.ptr, dX.ptr, 1)
+        else:
+            api.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, 1)
+
+    passes = {'fwd': p_fwd, 'dX': p_dx, 'dW': lambda: api.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW.ptr, 1)}
 
     def step():
         for fn in passes.values():
             fn()
 
-    settle(step, lambda: api.synchronize(0))
-    for _ in range(warmup):
-        step()
-    api.synchronize(0)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    api.synchronize(0)
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    wall_ms, cold_ms = timed_steps(step, lambda: api.synchronize(0), steps, warmup)
 
     per_pass = {}
     for k, fn in passes.items():
@@ -175,7 +245,8 @@ def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
     got = (Y.get(), dX.get(), dW.get())
     result = {
         'metric': 'conv2D fwd+bwd fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
-        'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
+        'value_cold': 3 * flops / cold_ms / 1e9,
+        'ms_per_step_cold': cold_ms, 'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
         'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
         'config': {'workload': f'{name}: x{list(xs)} w{list(ws)} stride {s} dilation {d} padding {padding!r}, '
                                'step = fwd + dX(+=) + dW(+=)'},
@@ -201,10 +272,11 @@ def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
             'value': 3 * flops / cpu_s / 1e12, 'unit': 'TFLOP/s', 'cores': cores, 'kind': 'port',
             'ms_per_step': cpu_s * 1e3,
             'sample': f'the full {name} step (fwd + dX + dW), median of {cpu_steps} after 1 warm-up, '
-                      'C restatement of unfold -> register-tiled GeMM -> transpose incl. zero fills, OpenMP'}
+                      'C restatement of unfold -> register-tiled GeMM -> transpose incl. zero fills, OpenMP',
+            'cpu_opencl': CPU_OPENCL}
         result['parity'] = {'checked_against': 'cpu_baseline outputs (fp32 reference data flow)',
                             'max_rel_err': max(rel_err(g, r) for g, r in zip(got, ref)), 'tolerance': 1e-4}
-    for a in (X, W, dY, Y, dX, dW):
+    for a in (X, W, dY, Y, dX, dW) + (() if Wp is W else (Wp,)):
         a.free()
     return result
 
@@ -225,15 +297,7 @@ def bench_matmul(api, steps, warmup, n=4096, cpu=True):
         for fn in passes.values():
             fn()
 
-    settle(step, lambda: api.synchronize(0))
-    for _ in range(warmup):
-        step()
-    api.synchronize(0)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    api.synchronize(0)
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    wall_ms, cold_ms = timed_steps(step, lambda: api.synchronize(0), steps, warmup)
     per_pass = {}
     for k, fn in passes.items():
         ms = time_events(api, fn, max(steps, 5))
@@ -243,12 +307,12 @@ def bench_matmul(api, steps, warmup, n=4096, cpu=True):
     dB.zero()
     step()
     res = {'metric': 'matmul fwd+dA+dB fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
-           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
+           'ms_per_step_cold': cold_ms, 'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
            'config': {'workload': f'cfg2_matmul: [{n}x{n}] @ [{n}x{n}], step = C + dA(+=) + dB(+=)'},
            'roofline': {'bound': 'mfma', 'kernel': dom, 'achieved': per_pass[dom]['tflops'],
                         'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s', 'frac': per_pass[dom]['frac_mfma'],
-                        'traffic': MEASURED_TRAFFIC_BYTES['cfg2_matmul'].get(dom) if n == 4096 else None},
+                        'traffic': MEASURED_TRAFFIC_BYTES.get('cfg2_matmul', {}).get(dom) if n == 4096 else None},
            'passes': per_pass}
     if cpu:
         from oracle import refpath
@@ -271,8 +335,7 @@ def bench_matmul(api, steps, warmup, n=4096, cpu=True):
 
 def bench_conv_transpose(api, steps, warmup, cpu=True):
     """Decoder layer: conv2DTranspose 256 -> 128, 5x5, stride 2, 'same', 16x16 -> 32x32, batch 16.  The three
-    passes run on the convolution kernels with the roles swapped (forward = dgrad, dI = forward, dK = wgrad)
-    on the kernel with its channel axes swapped; the swaps are part of the timed passes."""
+    passes run on the convolution kernels with the roles swapped (forward = dgrad, dI = forward, dK = wgrad)."""
     N, IC, IH, IW, OC, KS, S = 16, 256, 16, 16, 128, 5, 2
     ci = conv_info((N, IC, IH, IW), (OC, IC, KS, KS), S, 1, 'same')
     rs = np.random.RandomState(0)
@@ -281,24 +344,23 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
     dy = rs.normal(0, 1, (N, OC, ci.OH_T, ci.OW_T)).astype(np.float32)
     desc = api.conv_desc(N, OC, ci.OH_T, ci.OW_T, IC, KS, KS, IH, IW, ci.PADL, ci.PADT, S, 1)
     X, K, dY = Dev(api, x), Dev(api, k), Dev(api, dy)
-    Kt, dKt = Dev(api, shape=(IC, OC, KS, KS)), Dev(api, shape=(IC, OC, KS, KS))
     Y, dI, dK = Dev(api, shape=dy.shape), Dev(api, shape=x.shape), Dev(api, shape=k.shape)
     flops = 2.0 * N * IC * IH * IW * OC * KS * KS
 
-    def swap(src, dst, shape, beta):
-        api.transpose(0, shape, (1, 0, 2, 3), src, dst, beta)
+    # The kernel is stored (OC, IC, KH, KW): relative to the borrowed convolution (OC channels in, IC out) its channel
+    # axes are swapped.  The copy in the kernels' layout is made straight from that storage, once per step (the
+    # weights change once per step), and the kernel gradient is written straight into that storage.
+    Wp = Dev(api, shape=(IC, KS * KS, OC))
 
     def p_fwd():
-        swap(K.ptr, Kt.ptr, k.shape, 0)
-        api.conv2d_dgrad(0, desc, X.ptr, Kt.ptr, Y.ptr, 0)
+        api.conv2d_permute_weights(0, desc, K.ptr, api.W_IOHW, Wp.ptr)
+        api.conv2d_dgrad_pw(0, desc, X.ptr, Wp.ptr, Y.ptr, 0)
 
     def p_di():
-        swap(K.ptr, Kt.ptr, k.shape, 0)
-        api.conv2d_fwd(0, desc, dY.ptr, Kt.ptr, dI.ptr, 1)
+        api.conv2d_fwd_pw(0, desc, dY.ptr, Wp.ptr, None, api.ACT_NONE, 0.0, dI.ptr, 1)
 
     def p_dk():
-        api.conv2d_wgrad(0, desc, dY.ptr, X.ptr, dKt.ptr, 0)
-        swap(dKt.ptr, dK.ptr, (IC, OC, KS, KS), 1)
+        api.conv2d_wgrad_iohw(0, desc, dY.ptr, X.ptr, dK.ptr, 1)
 
     passes = {'fwd': p_fwd, 'dI': p_di, 'dK': p_dk}
 
@@ -306,15 +368,7 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
         for fn in passes.values():
             fn()
 
-    settle(step, lambda: api.synchronize(0))
-    for _ in range(warmup):
-        step()
-    api.synchronize(0)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    api.synchronize(0)
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    wall_ms, cold_ms = timed_steps(step, lambda: api.synchronize(0), steps, warmup)
     per_pass = {}
     for name, fn in passes.items():
         ms = time_events(api, fn, max(steps, 5))
@@ -324,7 +378,7 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
     dK.zero()
     step()
     res = {'metric': 'conv2DTranspose fwd+bwd fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
-           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
+           'ms_per_step_cold': cold_ms, 'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
            'config': {'workload': f'cfgT_decoder: conv2DTranspose x[{N}, {IC}, {IH}, {IW}] k[{OC}, {IC}, {KS}, {KS}] '
                                   f"stride {S} 'same', step = fwd + dI(+=) + dK(+=)"},
@@ -342,7 +396,7 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
         got_y, got_di = Y.get()[:2], dI.get()[:2]
         res['parity'] = {'checked_against': 'fp64 oracle on images 0-1 (Y, dI)',
                          'max_rel_err': max(rel_err(got_y, ry), rel_err(got_di, rdi)), 'tolerance': 1e-4}
-    for t in (X, K, dY, Kt, dKt, Y, dI, dK):
+    for t in (X, K, dY, Wp, Y, dI, dK):
         t.free()
     return res
 
@@ -371,15 +425,7 @@ def bench_depthwise(api, steps, warmup, cpu=True):
         for fn in passes.values():
             fn()
 
-    settle(step, lambda: api.synchronize(0))
-    for _ in range(warmup):
-        step()
-    api.synchronize(0)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    api.synchronize(0)
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    wall_ms, cold_ms = timed_steps(step, lambda: api.synchronize(0), steps, warmup)
     per_pass = {}
     for name, fn in passes.items():
         ms = time_events(api, fn, max(steps, 5))
@@ -391,14 +437,14 @@ def bench_depthwise(api, steps, warmup, cpu=True):
     step()
     total_bytes = sum(bytes_pass.values())
     res = {'metric': 'depthwise_conv2D fwd+bwd algorithmic GB/s', 'value': total_bytes / wall_ms / 1e6, 'unit': 'GB/s',
-           'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
+           'ms_per_step_cold': cold_ms, 'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
            'config': {'workload': f"cfgD_depthwise: x[{N}, {C}, {H}, {H}] k[{C}, {KS}, {KS}] stride 1 'same', "
                                   'step = fwd + dX(+=) + dK(+=)'},
            'images_per_s': N / wall_ms * 1e3,
            'roofline': {'bound': 'hbm', 'kernel': dom, 'achieved': per_pass[dom]['alg_gbs'], 'peak': PEAK_HBM_GBS,
                         'unit': 'GB/s', 'frac': per_pass[dom]['frac_hbm'],
-                        'traffic': MEASURED_TRAFFIC_BYTES['cfgD_depthwise'].get(dom)},
+                        'traffic': MEASURED_TRAFFIC_BYTES.get('cfgD_depthwise', {}).get(dom)},
            'passes': per_pass}
     if cpu:
         from oracle import depthwise_all
@@ -445,30 +491,26 @@ def bench_encoder(steps, warmup):
     opt = nn.optimizer.SGD(enc.trainables(), lr=1e-3)
     x_t = nn.Tensor_from_value(x_n)
 
+    last = {}
+
     def step():
         opt.zero_grad()
         loss = nn.square(enc(x_t)).mean()
         loss.backward()
         opt.step()
-        return loss
+        last['loss'] = loss
 
-    settle(step, nn.devices.wait)
-    for _ in range(warmup):
-        step()
-    nn.devices.wait()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        loss = step()
-    nn.devices.wait()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    wall_ms, cold_ms = timed_steps(step, nn.devices.wait, steps, warmup)
     flops = 61.66e9
     res = {'metric': 'encoder training step images/s', 'value': 16 / wall_ms * 1e3, 'unit': 'images/s', 'n_gpus': 1,
-           'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True, 'scaling': 'weak',
+           'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'ms_per_step_cold': cold_ms,
+           'value_cold': 16 / cold_ms * 1e3, 'higher_is_better': True, 'scaling': 'weak',
            'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
            'config': {'workload': 'cfg5_encoder: 16x3x128x128, 3->64->128->256->512, 5x5 s2 p2, leaky_relu(0.1), '
                                   'loss mean(square), SGD lr 1e-3; forward + backward + update'},
-           'conv_tflops': flops / wall_ms / 1e9, 'final_loss': float(loss.np()[0])}
-    del loss, x_t, opt, enc, layers
+           'conv_tflops': flops / wall_ms / 1e9, 'final_loss': float(last['loss'].np()[0])}
+    last.clear()
+    del x_t, opt, enc, layers
     return res
 
 
@@ -488,6 +530,9 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)')
+    global CPU_OPENCL
+    if not args.no_cpu:
+        CPU_OPENCL = probe_cpu_opencl()          # before this process touches the GPU
     from litenn_amd.core.hip import api
     if api.device_count() < 1:
         sys.exit('bench.py needs an MI355X: no HIP device is visible')

@@ -133,6 +133,35 @@ int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units,
 int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
                          float* dW, int beta);
 
+/* ---- weights kept in the kernels' own layout.  The kernels for channel counts that are multiples of 32 read the
+ * weights as Wp[o][kh*KW + kw][c]; lnn_conv2d_fwd_f32 / lnn_conv2d_dgrad_f32 make that copy in scratch on every
+ * call.  A caller that knows when its weights change (once per optimizer step) makes the copy once with
+ * lnn_conv2d_permute_weights_f32 and hands it to the *_pw entry points: forward and data gradient then share it.
+ * The reference has the same need and no such cache: conv2D_dI_gradfn transposes the kernel to (O, KH, KW, C) on
+ * every backward pass (conv2D.py:48), and conv2DTranspose swaps the kernel's channel axes in every pass
+ * (conv2DTranspose.py:33-47).  w_layout LNN_W_IOHW reads weights stored [C][O][KH][KW] - how a transposed
+ * convolution, whose passes are this convolution's passes with the roles swapped, keeps its kernel - so that no
+ * swapped copy is needed; lnn_conv2d_wgrad_iohw_f32 writes the weight gradient in that layout.
+ * lnn_conv2d_weights_plan (host arithmetic, no device needed) says for pass LNN_PASS_FWD / LNN_PASS_DGRAD whether
+ * the geometry's kernels read Wp (only then may the *_pw entry point be used), and for LNN_PASS_WGRAD whether
+ * lnn_conv2d_wgrad_iohw_f32 serves it.  Wp holds O*C*KH*KW floats and must be 16-byte aligned; for a 1x1 kernel
+ * stored OIHW the weights themselves are a valid Wp. */
+#define LNN_W_OIHW 0
+#define LNN_W_IOHW 1
+#define LNN_PASS_FWD 0
+#define LNN_PASS_DGRAD 1
+#define LNN_PASS_WGRAD 2
+int lnn_conv2d_weights_plan(const lnn_conv2d_desc* d, int pass, int* yes);
+int lnn_conv2d_permute_weights_f32(int dev, const lnn_conv2d_desc* d, const float* W, int w_layout, float* Wp);
+/* Y (+)= act(conv(X, W) + bias)   with W given as Wp; bias may be NULL; bias / act need beta == 0 */
+int lnn_conv2d_fwd_pw_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* Wp, const float* bias,
+                          int act, float slope, float* Y, int beta);
+/* dX (+)= dgrad(dY, W)            with W given as Wp */
+int lnn_conv2d_dgrad_pw_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* Wp, float* dX, int beta);
+/* dW[c][o][kh][kw] (+)= wgrad(X, dY)[o][c][kh][kw] */
+int lnn_conv2d_wgrad_iohw_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW,
+                              int beta);
+
 /* The same computation as lnn_conv2d_wgrad_f32, bit for bit, without any device allocation.  It has no counterpart
  * in the reference (whose buffers all come from clCreateBuffer at run time); it is for callers that cannot call
  * hipMalloc: code under HIP graph capture, tight serving or training loops, harnesses that forbid allocation.

@@ -12,12 +12,14 @@ class HipBuffer:
      size        bytes
      init_func   callable(HipBuffer) run right after physical allocation
     """
-    __slots__ = ['device', 'size', 'init_func', '_ptr', '__weakref__']
+    __slots__ = ['device', 'size', 'init_func', '_ptr', '_version', '_derived', '__weakref__']
     _object_count = 0
 
     def __init__(self, device, size, init_func=None):
         HipBuffer._object_count += 1
         self._ptr = None
+        self._version = 0      # grows whenever the contents may have changed (any access that is not read-only)
+        self._derived = None   # {key: (version, HipBuffer)}: copies in another layout, valid for that version only
         if size <= 0:
             raise ValueError(f'Create HipBuffer with {size} size.')
         self.device = device
@@ -31,16 +33,35 @@ class HipBuffer:
     def has_ptr(self):
         return self._ptr is not None
 
-    def get_ptr(self, skip_init=False):
+    def get_ptr(self, skip_init=False, readonly=False):
         """Device address.  skip_init=True is for a caller about to overwrite
-        every element: the initialiser is not run on first allocation."""
+        every element: the initialiser is not run on first allocation.
+        readonly=True is a promise not to write through the pointer; every other access counts as a change of
+        the contents and invalidates copies derived from them (see derived())."""
         if self._ptr is None:
             self._ptr = self.device._mem_alloc(self.size)
             if self.init_func is not None and not skip_init:
                 self.init_func(self)
+        if not readonly:
+            self._version += 1
         return self._ptr
 
+    def derived(self, key, size, make):
+        """A buffer computed from this one's current contents (the weights in a kernel's own layout), kept until
+        the contents change: make(src_ptr, dst_ptr) fills it.  Returns the derived HipBuffer."""
+        src = self.get_ptr(readonly=True)
+        if self._derived is None:
+            self._derived = {}
+        entry = self._derived.get(key)
+        if entry is not None and entry[0] == self._version:
+            return entry[1]
+        buf = entry[1] if entry is not None else HipBuffer(self.device, size)
+        make(src, buf.get_ptr(skip_init=True))
+        self._derived[key] = (self._version, buf)
+        return buf
+
     def free_ptr(self):
+        self._derived = None
         if self._ptr is not None:
             self.device._mem_free(self._ptr, self.size)
             self._ptr = None
@@ -57,7 +78,7 @@ class HipBuffer:
             if ShallowMode.active():
                 return
             if self.device is value.device:
-                api.memcpy_d2d(self.device.index, self.get_ptr(skip_init=True), value.get_ptr(), self.size)
+                api.memcpy_d2d(self.device.index, self.get_ptr(skip_init=True), value.get_ptr(readonly=True), self.size)
             else:
                 self.set(value.np())
             return
@@ -92,7 +113,7 @@ class HipBuffer:
         if out.nbytes != self.size:
             raise ValueError(f'Unable to represent HipBuffer with size {self.size} as shape {shape} with dtype {dtype}')
         if not ShallowMode.active():
-            api.memcpy_d2h(self.device.index, out, self.get_ptr())
+            api.memcpy_d2h(self.device.index, out, self.get_ptr(readonly=True))
         return out
 
     def __str__(self):

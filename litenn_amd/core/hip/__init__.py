@@ -10,7 +10,9 @@ def launch(fn, *args):
     """Run `fn(device_index, *per_device_args)` on every current device, taking
     from each HipDevicesBuffers argument that device's pointer (the fan-out of
     CLKernel.run, CLKernel.py:58-62).  A (tensor, 'w') tuple marks an output
-    that will be completely overwritten, so its initialiser is skipped.
+    that will be completely overwritten, so its initialiser is skipped; a
+    (tensor, 'r') tuple one that is only read (a plain tensor argument counts
+    as possibly written, which invalidates layout copies derived from it).
     Nothing runs in shallow mode.
 
     The library allocates on its own for some calls (scratch for partial sums, gather tables); when that runs
@@ -24,6 +26,8 @@ def launch(fn, *args):
         for a in args:
             if isinstance(a, tuple) and len(a) == 2 and a[1] == 'w' and isinstance(a[0], HipDevicesBuffers):
                 resolved.append(a[0]._get_buffers()[i].get_ptr(skip_init=True))
+            elif isinstance(a, tuple) and len(a) == 2 and a[1] == 'r' and isinstance(a[0], HipDevicesBuffers):
+                resolved.append(a[0]._get_buffers()[i].get_ptr(readonly=True))
             elif isinstance(a, HipDevicesBuffers):
                 resolved.append(a._get_buffers()[i].get_ptr())
             else:
@@ -35,3 +39,30 @@ def launch(fn, *args):
             except api.HipException as e:
                 if e.code != api.ERR_OOM or not device._release_largest_pooled():
                     raise
+
+
+class _BufferList(HipDevicesBuffers):
+    """Per-device buffers that already exist, in the shape launch() takes."""
+
+    def __init__(self, buffers):
+        self._buffers = buffers
+
+
+def permuted_weights(kernel_t, desc, w_layout=api.W_OIHW):
+    """The convolution weights of kernel_t in the layout the tap-major kernels read, Wp[o][tap][c], as a launch()
+    argument (pass it as (result, 'r')).  One copy per device, made on first use and again only after kernel_t's
+    contents may have changed (an optimizer step, set(), fill(), any launch that took it as a plain argument):
+    forward and data gradient of a training step, and every pass of an inference loop, share it.
+    w_layout W_IOHW: kernel_t is stored (C, O, KH, KW) relative to desc, as a transposed convolution keeps it.
+    A 1x1 kernel stored OIHW already has the layout and is returned itself."""
+    if w_layout == api.W_OIHW and desc.KH * desc.KW == 1:
+        return kernel_t
+    if ShallowMode.active():
+        return kernel_t
+    key = ('wp', int(w_layout), desc.O, desc.C, desc.KH, desc.KW)
+    size = desc.O * desc.C * desc.KH * desc.KW * 4
+    out = []
+    for buf in kernel_t._get_buffers():
+        dev = buf.device.index
+        out.append(buf.derived(key, size, lambda src, dst, dev=dev: api.conv2d_permute_weights(dev, desc, src, w_layout, dst)))
+    return _BufferList(out)

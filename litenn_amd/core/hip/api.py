@@ -70,6 +70,11 @@ SIGNATURES = {
     'lnn_depthwise_conv2d_wgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_dgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_wgrad_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
+    'lnn_conv2d_weights_plan': [ctypes.POINTER(ConvDesc), _c_int, ctypes.POINTER(_c_int)],
+    'lnn_conv2d_permute_weights_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _c_int, _ptr],
+    'lnn_conv2d_fwd_pw_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int, ctypes.c_float, _ptr, _c_int],
+    'lnn_conv2d_dgrad_pw_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
+    'lnn_conv2d_wgrad_iohw_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_wgrad_noalloc_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_dgrad_path': [ctypes.POINTER(ConvDesc), _c_int, _c_int, ctypes.POINTER(_c_int), _i32arr],
     'lnn_unfold2d_f32': [_c_int] + [_c_int] * 14 + [_ptr, _ptr, _c_int],
@@ -221,6 +226,34 @@ def conv2d_fwd_bias_act(dev, desc, X, W, bias, act, slope, Y):
 
 def conv2d_dgrad(dev, desc, dY, W, dX, beta=1):
     check(lib.lnn_conv2d_dgrad_f32(dev, ctypes.byref(desc), dY, W, dX, int(beta)))
+
+
+W_OIHW, W_IOHW = 0, 1
+PASS_FWD, PASS_DGRAD, PASS_WGRAD = 0, 1, 2
+
+
+def conv2d_weights_plan(desc, which):
+    """True if the geometry's forward / data-gradient kernels read the permuted weights Wp[o][tap][c] (so the
+    *_pw entry points apply), resp. if conv2d_wgrad_iohw serves its weight gradient.  Host arithmetic only."""
+    yes = _c_int(0)
+    check(lib.lnn_conv2d_weights_plan(ctypes.byref(desc), int(which), ctypes.byref(yes)))
+    return bool(yes.value)
+
+
+def conv2d_permute_weights(dev, desc, W, w_layout, Wp):
+    check(lib.lnn_conv2d_permute_weights_f32(dev, ctypes.byref(desc), W, int(w_layout), Wp))
+
+
+def conv2d_fwd_pw(dev, desc, X, Wp, bias, act, slope, Y, beta=0):
+    check(lib.lnn_conv2d_fwd_pw_f32(dev, ctypes.byref(desc), X, Wp, bias, int(act), float(slope), Y, int(beta)))
+
+
+def conv2d_dgrad_pw(dev, desc, dY, Wp, dX, beta=1):
+    check(lib.lnn_conv2d_dgrad_pw_f32(dev, ctypes.byref(desc), dY, Wp, dX, int(beta)))
+
+
+def conv2d_wgrad_iohw(dev, desc, X, dY, dW, beta=1):
+    check(lib.lnn_conv2d_wgrad_iohw_f32(dev, ctypes.byref(desc), X, dY, dW, int(beta)))
 
 
 NOALLOC_SCRATCH_BYTES = 32 << 20

@@ -1,7 +1,7 @@
 import litenn_amd as nn
 import litenn_amd.core as nc
 from ..backward import at_end_of_sweep, current_sweep
-from ..hip import api, launch, ShallowMode
+from ..hip import api, launch, permuted_weights, ShallowMode
 
 
 def conv2D(input_t, kernel_t, stride=1, dilation=1, padding='same'):
@@ -21,7 +21,11 @@ def conv2D(input_t, kernel_t, stride=1, dilation=1, padding='same'):
     output_t._set_op_name('conv2D')
     output_t._assign_gradfn(input_t, lambda O_t, dO_t: conv2D_dI_gradfn(op, input_t, kernel_t, dO_t))
     output_t._assign_gradfn(kernel_t, lambda O_t, dO_t: conv2D_dK_gradfn(op, input_t, kernel_t, dO_t))
-    launch(lambda dev, x, w, y: api.conv2d_fwd(dev, op.desc, x, w, y, 0), input_t, kernel_t, (output_t, 'w'))
+    if op.fwd_pw:
+        launch(lambda dev, x, wp, y: api.conv2d_fwd_pw(dev, op.desc, x, wp, None, api.ACT_NONE, 0.0, y, 0),
+               (input_t, 'r'), (permuted_weights(kernel_t, op.desc), 'r'), (output_t, 'w'))
+    else:
+        launch(lambda dev, x, w, y: api.conv2d_fwd(dev, op.desc, x, w, y, 0), (input_t, 'r'), (kernel_t, 'r'), (output_t, 'w'))
     return output_t
 
 
@@ -53,12 +57,17 @@ def conv2D_bias_act(input_t, kernel_t, bias_t=None, stride=1, dilation=1, paddin
         output_t._assign_gradfn(bias_t, lambda O_t, dO_t: epi.bias(O_t, dO_t, bias_t))
     output_t._assign_gradfn(input_t, lambda O_t, dO_t: conv2D_dI_gradfn(op, input_t, kernel_t, epi.pre(O_t, dO_t)))
     output_t._assign_gradfn(kernel_t, lambda O_t, dO_t: conv2D_dK_gradfn(op, input_t, kernel_t, epi.pre(O_t, dO_t)))
-    if bias_t is None:
-        launch(lambda dev, x, w, y: api.conv2d_fwd_bias_act(dev, op.desc, x, w, None, act, alpha, y),
-               input_t, kernel_t, (output_t, 'w'))
-    else:
-        launch(lambda dev, x, w, b, y: api.conv2d_fwd_bias_act(dev, op.desc, x, w, b, act, alpha, y),
-               input_t, kernel_t, bias_t, (output_t, 'w'))
+    args = [(input_t, 'r'), (permuted_weights(kernel_t, op.desc), 'r') if op.fwd_pw else (kernel_t, 'r')]
+    if bias_t is not None:
+        args.append((bias_t, 'r'))
+
+    def run(dev, x, w, *rest):
+        b, y = (rest[0], rest[1]) if bias_t is not None else (None, rest[0])
+        if op.fwd_pw:
+            api.conv2d_fwd_pw(dev, op.desc, x, w, b, act, alpha, y, 0)
+        else:
+            api.conv2d_fwd_bias_act(dev, op.desc, x, w, b, act, alpha, y)
+    launch(run, *args, (output_t, 'w'))
     return output_t
 
 
@@ -128,13 +137,17 @@ class _EpilogueGrad:
 def conv2D_dI_gradfn(op, input_t, kernel_t, dO_t):
     """input.grad += dgrad(dO, kernel)   (conv2D.py:46-50)."""
     grad_t, beta = nc.op.accumulate_target(input_t.get_grad())
-    launch(lambda dev, dy, w, dx: api.conv2d_dgrad(dev, op.desc, dy, w, dx, beta), dO_t, kernel_t, grad_t)
+    if op.dgrad_pw:
+        launch(lambda dev, dy, wp, dx: api.conv2d_dgrad_pw(dev, op.desc, dy, wp, dx, beta),
+               (dO_t, 'r'), (permuted_weights(kernel_t, op.desc), 'r'), grad_t)
+    else:
+        launch(lambda dev, dy, w, dx: api.conv2d_dgrad(dev, op.desc, dy, w, dx, beta), (dO_t, 'r'), (kernel_t, 'r'), grad_t)
 
 
 def conv2D_dK_gradfn(op, input_t, kernel_t, dO_t):
     """kernel.grad += wgrad(input, dO)   (conv2D.py:52-54)."""
     grad_t, beta = nc.op.accumulate_target(kernel_t.get_grad())
-    launch(lambda dev, x, dy, dw: api.conv2d_wgrad(dev, op.desc, x, dy, dw, beta), input_t, dO_t, grad_t)
+    launch(lambda dev, x, dy, dw: api.conv2d_wgrad(dev, op.desc, x, dy, dw, beta), (input_t, 'r'), (dO_t, 'r'), grad_t)
 
 
 class _Conv2DOp:
@@ -155,3 +168,7 @@ class _Conv2DOp:
         self.info = ci
         self.output_shape = nc.TensorShape((N, KO, ci.OH, ci.OW))
         self.desc = api.conv_desc(N, IC, IH, IW, KO, KH, KW, ci.OH, ci.OW, ci.PADL, ci.PADT, stride, dilation)
+        # whether this geometry's forward / data-gradient kernels read the weights in their permuted layout, of
+        # which one cached copy then serves both passes until the weights change
+        self.fwd_pw = api.conv2d_weights_plan(self.desc, api.PASS_FWD)
+        self.dgrad_pw = api.conv2d_weights_plan(self.desc, api.PASS_DGRAD)

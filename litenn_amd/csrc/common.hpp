@@ -46,13 +46,18 @@ constexpr uint64_t kMaxTensorBytes = 0x7fffffffull;   // raw buffer descriptors 
 // launchers implemented in the kernel translation units
 int launch_gemm(DeviceCtx* ctx, int ta, int tb, int batch, int M, int N, int K, const float* A, int lda,
                 long long sA, const float* B, int ldb, long long sB, float* C, int ldc, long long sC, int beta);
+// Wp: the weights in the permuted layout (made by launch_permute_weights), or null; W may be null when Wp is given
 int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta,
-                    const float* bias, int act, float slope);
+                    const float* bias, int act, float slope, const float* Wp = nullptr);
+int conv_weights_plan(const lnn_conv2d_desc* d, int pass, int* yes);
+int launch_permute_weights(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* W, int w_layout, float* Wp);
 int launch_dw_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* K, float* Y, int beta);
 int launch_dw_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* K, float* dX, int beta);
 int launch_dw_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dK, int beta);
-int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta);
+int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta,
+                      const float* Wp = nullptr);
 int conv_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* path, int32_t* tile_info);
-int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta);
+int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta,
+                      int w_iohw = 0);
 
 }  // namespace lnn

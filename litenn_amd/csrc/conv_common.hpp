@@ -56,6 +56,7 @@ struct ConvArgs {
   int chunk_units;   // tap-major wgrad: units per workgroup
   // dgrad: g describes one pixel class (g.IH, g.IW = class grid); the plane it is cut from:
   int full_IW, full_IHW, cls_org, cls_s;
+  int w_iohw;        // wgrad: dW is stored [C][O][KH][KW]
 };
 
 // One class of input pixels of a strided dgrad: pixels (h0 + S*i, w0 + S*j),
@@ -188,18 +189,23 @@ __global__ __launch_bounds__(256) void reduce_partials_batch(ReduceBatch b) {
 
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
 // PASS_WGRAD_TAP4: PASS_WGRAD_TAP with 128-bit transfers of the pixel gather too (stride 1, OW % 4 == 0, no padded columns)
-enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5, PASS_WGRAD_TAP4 = 6 };
+// PASS_DGRAD_TAPW: tap-major dgrad that reads the weights in the forward pass's permuted layout (C % 4 == 0)
+enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5, PASS_WGRAD_TAP4 = 6,
+       PASS_DGRAD_TAPW = 7 };
 constexpr bool wgrad_tap(int pass) { return pass == PASS_WGRAD_TAP || pass == PASS_WGRAD_TAP4; }
+constexpr bool dgrad_tap(int pass) { return pass == PASS_DGRAD_TAP || pass == PASS_DGRAD_TAPW; }
 
 // Wp[a][tap][b] = W[..] so that the tap-major K index tap*CH + ch is contiguous:
-//   mode 0 (forward): Wp[o][tap][c] = W[o][c][tap]
-//   mode 1 (dgrad):   Wp[c][t][o] = W[o][c][tap_t], t over the taps of the pixel class
+//   mode 0 (forward, and the data gradient when C % 4 == 0): Wp[o][tap][c] = W[o][c][tap]
+//   mode 2: the same from weights stored with their channel axes swapped, W[c][o][tap] (a transposed
+//           convolution keeps its kernel that way)
+//   mode 1 (dgrad, other C): Wp[c][t][o] = W[o][c][tap_t], t over the taps of the pixel class
 __device__ __forceinline__ void permute_one(float* wp, const float* w, int O, int C, int KK, int mode, const ConvGeom& g,
                                             const PixelClass& pc, int i) {
-  if (mode == 0) {
+  if (mode == 0 || mode == 2) {
     if (i >= O * C * KK) return;
     const int b = i % C, tap = (i / C) % KK, a = i / (C * KK);
-    wp[i] = w[((size_t)a * C + b) * KK + tap];
+    wp[i] = mode == 0 ? w[((size_t)a * C + b) * KK + tap] : w[((size_t)b * O + a) * KK + tap];
   } else {
     const int nt = pc.nkh * pc.nkw;
     if (i >= O * C * nt) return;
@@ -225,7 +231,7 @@ template <int PASS, int WM, int NTMAX, bool FLAG>
 struct ConvCfg {
   static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
   // the tap-major passes send both operands straight into unpadded LDS tiles, three stages deep
-  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || PASS == PASS_DGRAD_TAP || wgrad_tap(PASS);
+  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || dgrad_tap(PASS) || wgrad_tap(PASS);
   // A side is K-contiguous in LDS for all passes.
   static constexpr int SA = DIRECT ? BM * BK : LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
@@ -281,6 +287,14 @@ struct ConvProblem<PASS_DGRAD_TAP, FLAG, ST> : ConvProblemBase {
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
 template <bool FLAG, int ST>
+struct ConvProblem<PASS_DGRAD_TAPW, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
+  template <int R> using LA = ConvDgradATapMC<R>;        // the forward pass's permuted weights [O][KK*C]
+  template <int R> using LB = ConvDgradBTap<R, LNN_FD_B_DIRECT != 0>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, tab, row0, kbeg); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
+};
+template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = ConvWgradA<R, FLAG>;
@@ -319,12 +333,13 @@ __host__ __device__ inline OutMap final_map(const ConvArgs& a) {
   OutMap om = plain_map(a.Ncols);
   if (PASS == PASS_FWD || PASS == PASS_FWD_TAP) {
     om.nchw = 1; om.ld = a.g.OHW; om.mtot = a.g.O; om.dHW = a.g.dOHW;
-  } else if (PASS == PASS_DGRAD || PASS == PASS_DGRAD_TAP) {
+  } else if (PASS == PASS_DGRAD || dgrad_tap(PASS)) {
     om.nchw = 3; om.ld = a.full_IHW; om.mtot = a.g.C; om.dHW = a.g.dIHW;
     om.dCW = a.g.dIW; om.s = a.cls_s; om.iw = a.full_IW; om.org = a.cls_org;
   } else if (wgrad_tap(PASS)) {
-    // GEMM column tap*C + c lands in dW[o][c][tap]
+    // GEMM column tap*C + c lands in dW[o][c][tap], or in dW[c][o][tap] for a gradient kept with swapped channel axes
     om.nchw = 2; om.ld = a.Ncols; om.mtot = a.g.KK; om.dHW = a.dC;
+    if (a.w_iohw) { om.ld = a.g.KK; om.mtot = a.g.O * a.g.KK; }
   }
   return om;
 }
@@ -647,7 +662,7 @@ static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_
   // kernels, whose time follows the multiply-adds, each gets workgroups in proportion to its work instead
   // (256 -> 512 channels at 16 x 16: 77 -> 63 us).
   std::vector<long long> share(n, equal);
-  if (LNN_CLASS_SHARES && PASS == PASS_DGRAD_TAP && n <= kMaxBatch) {
+  if (LNN_CLASS_SHARES && dgrad_tap(PASS) && n <= kMaxBatch) {
     std::vector<long long> prop(n, equal);
     long long total = 0, given = 0;
     for (int i = 0; i < n; ++i) total += (long long)cls[i].K * cls[i].Ncols;
@@ -738,6 +753,13 @@ static int launch_by_m(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   if (a.M > 64) return launch_pass<PASS, 4, 4>(ctx, a, flag);
   if (a.M > 32) return launch_pass<PASS, 2, 2>(ctx, a, flag);
   return launch_pass<PASS, 1, 1>(ctx, a, flag);
+}
+
+// The weight gradient runs on the pixel-major loaders (tap-major columns) when the channels fill whole units of
+// the tile shape chosen for O and a K step of pixels never wraps around an image more than once.
+static bool wgrad_is_pixel_major(const ConvGeom& g) {
+  const int unit = g.O > 64 ? 32 : (g.O > 32 ? 64 : 128);
+  return g.C % unit == 0 && BK / g.OW + 1 <= g.OH;
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }

@@ -276,14 +276,22 @@ int conv_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* 
   return LNN_OK;
 }
 
-int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta) {
+// Whether the data gradient of this geometry reads the weights in the forward pass's permuted layout
+// Wp[o][tap][c] (shared with the forward pass, made once per weight update by the caller or per call here).
+bool dgrad_reads_permuted(const ConvGeom& g) { return g.O % BK == 0 && g.C % 4 == 0 && g.C > 4; }
+
+int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta,
+                      const float* Wp) {
   ConvGeom full;
   int st = fill_geom(d, full);
   if (st != LNN_OK) return st;
-  if (!dY || !W || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
+  const bool tapw = dgrad_reads_permuted(full);
+  if (Wp && !tapw) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: this geometry does not read permuted weights");
+  if (Wp && !aligned16(Wp)) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: permuted weights must be 16-byte aligned");
+  if (!dY || (!W && !Wp) || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
   const int S = full.S;
   if (S > 15) return set_error(LNN_ERR_UNSUPPORTED, "conv2d_dgrad: stride > 15");
-  if (small_dgrad_applies(ctx->cus, full)) {
+  if (!tapw && small_dgrad_applies(ctx->cus, full)) {
     st = launch_small_dgrad(ctx, full, dY, W, dX, beta);
     if (st != kNotHere) return st;
   }
@@ -309,6 +317,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
       if (nt == 0 && beta) continue;                        // nothing to add; without beta the class is zero-filled
       ConvArgs a;
       a.ws_used = 0;
+      a.w_iohw = 0;
       a.post = PostOp{nullptr, 0, 0.0f};
       a.g = full;
       ConvGeom& g = a.g;
@@ -320,14 +329,14 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
       a.tab = nullptr;
       a.X = dY; a.W = W; a.Out = dX;
       a.bytesX = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
-      a.bytesW = (uint32_t)((uint64_t)g.O * g.C * (tap ? nt : g.KK) * 4);
+      a.bytesW = (uint32_t)((uint64_t)g.O * g.C * (tap && !tapw ? nt : g.KK) * 4);
       a.bytesOut = (uint32_t)((uint64_t)g.N * g.C * full.IHW * 4);
       a.M = g.C; a.Ncols = g.N * g.IHW; a.K = g.O * nt;
       a.beta = beta ? 1 : 0;
       a.dC = make_fastdiv(1);
       st = get_table(ctx, full, tap ? 2 : 1, pc, &a.tab);
       if (st != LNN_OK) return st;
-      if (tap) {
+      if (tap && !tapw) {
         w_off.push_back(w_bytes);
         w_bytes += ((size_t)(a.bytesW ? a.bytesW : 4) + 255) & ~(size_t)255;
       }
@@ -343,7 +352,31 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   // sharing it; neither do more classes than one launch holds (stride > 2).
   const int unit_cols = cls[0].M > 64 ? 32 : (cls[0].M > 32 ? 64 : 128);
   const long long units0 = (long long)((cls[0].M + 127) / 128) * ((cls[0].Ncols + unit_cols - 1) / unit_cols);
-  if (nc > kMaxBatch || units0 >= 4ll * ctx->cus) {
+  const bool one_by_one = nc > kMaxBatch || units0 >= 4ll * ctx->cus;
+  if (tapw) {
+    // every class reads the same copy of the weights, Wp[o][tap][c]: the caller's, the weights themselves (a 1x1
+    // kernel already has that layout), or one made here at the front of the scratch buffer
+    const float* wsrc = Wp ? Wp : (full.KK == 1 && aligned16(W) ? W : nullptr);
+    if (!wsrc) w_bytes = ((size_t)full.O * full.C * full.KK * sizeof(float) + 255) & ~(size_t)255;
+    st = ensure_workspace(ctx, w_bytes + part_bytes);
+    if (st != LNN_OK) return st;
+    if (!wsrc) {
+      size_t used = 0;
+      st = permuted_weights(ctx, full, W, 0, PixelClass{}, &wsrc, &used);
+      if (st != LNN_OK) return st;
+    }
+    for (int i = 0; i < nc; ++i) {
+      cls[i].W = wsrc;
+      cls[i].ws_used = w_bytes;
+    }
+    if (!one_by_one) return launch_classes_by_m<PASS_DGRAD_TAPW>(ctx, cls, w_bytes);
+    for (int i = 0; i < nc; ++i) {
+      st = launch_by_m<PASS_DGRAD_TAPW>(ctx, cls[i], true);
+      if (st != LNN_OK) return st;
+    }
+    return LNN_OK;
+  }
+  if (one_by_one) {
     // one after the other, each with the whole chip.  All the scratch any class needs (its permuted weights,
     // then partial sums) is reserved before the first launch: a failed allocation then leaves dX untouched, so
     // the caller may free memory and repeat the call.

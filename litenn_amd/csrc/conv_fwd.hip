@@ -3,15 +3,47 @@
 
 namespace lnn {
 
+// Which passes of a geometry read (forward, data gradient) the weights in the permuted layout Wp[o][tap][c], or can
+// write (weight gradient) a gradient whose channel axes are swapped.  Host arithmetic only.
+int conv_weights_plan(const lnn_conv2d_desc* d, int pass, int* yes) {
+  ConvGeom g;
+  int st = fill_geom(d, g);
+  if (st != LNN_OK) return st;
+  if (!yes) return set_error(LNN_ERR_INVALID, "conv2d_weights_plan: null result pointer");
+  if (pass == LNN_PASS_FWD) *yes = g.C % BK == 0;
+  else if (pass == LNN_PASS_DGRAD) *yes = g.O % BK == 0 && g.C % 4 == 0 && g.C > 4;
+  else if (pass == LNN_PASS_WGRAD) *yes = wgrad_is_pixel_major(g);
+  else return set_error(LNN_ERR_INVALID, "conv2d_weights_plan: unknown pass");
+  return LNN_OK;
+}
+
+// Wp[o][kh*KW + kw][c] = W[o][c][kh][kw] (w_layout LNN_W_OIHW) or W[c][o][kh][kw] (LNN_W_IOHW)
+int launch_permute_weights(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* W, int w_layout, float* Wp) {
+  ConvGeom g;
+  int st = fill_geom(d, g);
+  if (st != LNN_OK) return st;
+  if (!W || !Wp) return set_error(LNN_ERR_INVALID, "conv2d_permute_weights: null pointer");
+  if (w_layout != LNN_W_OIHW && w_layout != LNN_W_IOHW) return set_error(LNN_ERR_INVALID, "conv2d_permute_weights: unknown layout");
+  if (!aligned16(Wp)) return set_error(LNN_ERR_INVALID, "conv2d_permute_weights: the destination must be 16-byte aligned");
+  const int n = g.O * g.C * g.KK;
+  hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, Wp, W, g.O, g.C, g.KK,
+                     w_layout == LNN_W_OIHW ? 0 : 2, g, PixelClass{});
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
 int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta,
-                    const float* bias, int act, float slope) {
+                    const float* bias, int act, float slope, const float* Wp) {
   ConvArgs a;
   a.ws_used = 0;
+  a.w_iohw = 0;
   a.post = PostOp{bias, act, slope};
   if (beta && a.post.any()) return set_error(LNN_ERR_INVALID, "conv2d_fwd: bias / activation cannot be combined with accumulation");
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
-  if (!X || !W || !Y) return set_error(LNN_ERR_INVALID, "conv2d_fwd: null pointer");
+  if (Wp && a.g.C % BK != 0) return set_error(LNN_ERR_INVALID, "conv2d_fwd: this geometry does not read permuted weights");
+  if (Wp && !aligned16(Wp)) return set_error(LNN_ERR_INVALID, "conv2d_fwd: permuted weights must be 16-byte aligned");
+  if (!X || (!W && !Wp) || !Y) return set_error(LNN_ERR_INVALID, "conv2d_fwd: null pointer");
   st = reserve_tables(ctx, 1);
   if (st != LNN_OK) return st;
   a.tab = nullptr;
@@ -22,6 +54,10 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   a.bytesOut = (uint32_t)((uint64_t)g.N * g.O * g.OHW * 4);
   a.M = g.O; a.Ncols = g.N * g.OHW; a.K = g.C * g.KK;
   a.beta = beta ? 1 : 0;
+  if (Wp) {
+    a.W = Wp;
+    return launch_by_m<PASS_FWD_TAP>(ctx, a, true);
+  }
   if (g.C % BK == 0 && (g.KK > 1 || aligned16(W))) {
     if (g.KK > 1) {   // a 1x1 kernel already is [O][tap][C]
       st = permuted_weights(ctx, g, W, 0, PixelClass{}, &a.W, &a.ws_used);

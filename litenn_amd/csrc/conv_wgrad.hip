@@ -3,8 +3,10 @@
 
 namespace lnn {
 
-int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
+int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta,
+                      int w_iohw) {
   ConvArgs a;
+  a.w_iohw = w_iohw ? 1 : 0;
   a.ws_used = 0;
   a.post = PostOp{nullptr, 0, 0.0f};
   int st = fill_geom(d, a.g);
@@ -18,16 +20,14 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   a.bytesOut = (uint32_t)((uint64_t)g.O * g.C * g.KK * 4);
   a.M = g.O; a.Ncols = g.C * g.KK; a.K = g.N * g.OHW;
   a.beta = beta ? 1 : 0;
-  // pixel-major loaders when the channels fill whole units of the tile shape chosen for O
-  const int unit = g.O > 64 ? 32 : (g.O > 32 ? 64 : 128);
-  // ... and a K step of pixels never wraps around an image more than once
   const bool vec = g.OHW % 4 == 0 && aligned16(dY);
-  if (g.C % unit == 0 && BK / g.OW + 1 <= g.OH) {
+  if (wgrad_is_pixel_major(g)) {
     // every tap of every output pixel reads a column inside the image: the gather can move four pixels at a time
     const bool cols_inside = g.PADL == 0 && g.OW - 1 + (g.KW - 1) * g.D <= g.IW - 1;
     if (vec && g.S == 1 && g.OW % 4 == 0 && cols_inside) return launch_by_m<PASS_WGRAD_TAP4>(ctx, a, true);
     return launch_by_m<PASS_WGRAD_TAP>(ctx, a, vec);
   }
+  if (w_iohw) return set_error(LNN_ERR_UNSUPPORTED, "conv2d_wgrad: this geometry cannot write a gradient with swapped channel axes");
   // the table-driven kernel: per-column gather entries
   st = reserve_tables(ctx, 1);
   if (st != LNN_OK) return st;

@@ -342,6 +342,32 @@ int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, con
   return launch_conv_dgrad(ctx, d, dY, W, dX, beta);
 }
 
+int lnn_conv2d_weights_plan(const lnn_conv2d_desc* d, int pass, int* yes) { return conv_weights_plan(d, pass, yes); }
+
+int lnn_conv2d_permute_weights_f32(int dev, const lnn_conv2d_desc* d, const float* W, int w_layout, float* Wp) {
+  CTX(dev);
+  return launch_permute_weights(ctx, d, W, w_layout, Wp);
+}
+
+int lnn_conv2d_fwd_pw_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* Wp, const float* bias, int act,
+                          float slope, float* Y, int beta) {
+  CTX(dev);
+  if (!Wp) return set_error(LNN_ERR_INVALID, "conv2d_fwd_pw: null pointer");
+  if (act != LNN_ACT_NONE && act != LNN_ACT_LEAKY_RELU) return set_error(LNN_ERR_INVALID, "conv2d_fwd_pw: unknown activation");
+  return launch_conv_fwd(ctx, d, X, nullptr, Y, beta, bias, act, slope, Wp);
+}
+
+int lnn_conv2d_dgrad_pw_f32(int dev, const lnn_conv2d_desc* d, const float* dY, const float* Wp, float* dX, int beta) {
+  CTX(dev);
+  if (!Wp) return set_error(LNN_ERR_INVALID, "conv2d_dgrad_pw: null pointer");
+  return launch_conv_dgrad(ctx, d, dY, nullptr, dX, beta, Wp);
+}
+
+int lnn_conv2d_wgrad_iohw_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
+  CTX(dev);
+  return launch_conv_wgrad(ctx, d, X, dY, dW, beta, 1);
+}
+
 int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* path, int32_t* tile_info) {
   return conv_dgrad_path(d, beta, compute_units, path, tile_info);
 }

@@ -557,6 +557,58 @@ struct ConvDgradBTap {
   }
 };
 
+// dgrad weight operand read from the weights in the layout the tap-major forward pass reads,
+// Wp[o][tap][c] (tap = kh*KW + kw): element (row c, k = (tap, o)) sits at o*ld + tap*C + c with ld = KK*C, so for
+// one tap the 32 output channels of a K step are 32 rows of C contiguous floats: a K-major stored matrix, moved
+// with 128-bit transfers into the group's [BK][R] slab exactly as DirectMC moves one (C % 4 == 0, 16-byte
+// aligned Wp).  The K advance (next 32 output channels, then the class's next tap, whose index the per-tap table
+// carries in .w) rides in the scalar offset.  Forward and data gradient thus share one permuted copy of the
+// weights, whatever the stride and the pixel class.
+template <int R>
+struct ConvDgradATapMC {
+  static constexpr bool KC = false, DIRECT = true;
+  static constexpr int LAYOUT = LAY_MC_SPLIT;
+  static constexpr int NI = BK * R / 256, E = (NI + 3) / 4;
+  static constexpr int NLD = NI % 4 == 0 ? E : -1;
+  static_assert(R % 8 == 0, "whole 256-float transfers");
+  rsrc_t rs;
+  ktab_t tab;           // one entry per tap of the pixel class: .w = kh*KW + kw
+  uint32_t voff[E];
+  int ld, O, C;
+  int o0, tap, cw, nw;  // K position of the next transfer; tap index of the current tap and of the one after it
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int row0, int kbeg) {
+    rs = r;
+    tab = as_ktab(tab_);
+    ld = g.KK * g.C; O = g.O; C = g.C;
+    tap = kbeg / g.O;
+    o0 = kbeg - tap * g.O;
+    cw = (tab + tap)->w;
+    nw = (tab + tap + 1)->w;
+    const int wave = gwave(), lane = threadIdx.x & 63;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int f = (wave + 4 * e) * 256 + lane * 4, k = f / R, n = f - k * R;
+      voff[e] = (k < BK && row0 + n < g.C) ? (uint32_t)(k * ld + row0 + n) * 4u : OOB;
+    }
+  }
+  __device__ __forceinline__ void issue(int, float* lds, int, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+    const uint32_t soff = (uint32_t)(o0 * ld + cw * C) * 4u;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int q = wave + 4 * e;
+      if (NI % 4 == 0 || q < NI) buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff);
+    }
+    o0 += BK;
+    if (o0 >= O) {   // wave-uniform: next tap of the class
+      o0 = 0;
+      ++tap;
+      cw = nw;
+      nw = (tab + tap + 1)->w;
+    }
+  }
+};
+
 // dgrad gather of dY.  A strided convolution is handled as S*S independent
 // stride-1 problems, one per class of input pixels with equal
 // ((ih + PT) mod S, (iw + PL) mod S): inside a class only the taps with

@@ -12,7 +12,7 @@ from oracle import (conv2d_fwd, conv2d_dx, conv2d_dw, unfold_index_map, unfold_T
 from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
-         'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
+         'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'conv2d_permute_weights', 'conv2d_fwd_pw', 'conv2d_dgrad_pw', 'conv2d_wgrad_iohw', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
          'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal', 'bias_act_bwd', 'sgd_update_multi', 'adam_update_multi']
 
 
@@ -116,6 +116,47 @@ class FakeHip:
         self.launches += 1
         xs, ws, ys, pad = self._geom(d)
         self._put(self.f(dW, ws), conv2d_dw(self.f(X, xs), self.f(dY, ys), ws, d.stride, d.dilation, pad), beta)
+
+    # the weights in the kernels' permuted layout Wp[o][tap][c]
+    def conv2d_permute_weights(self, dev, d, W, w_layout, Wp):
+        self.launches += 1
+        kk = d.KH * d.KW
+        if w_layout == real_api.W_OIHW:
+            w = self.f(W, (d.O, d.C, kk))
+        else:
+            w = self.f(W, (d.C, d.O, kk)).transpose(1, 0, 2)
+        self.f(Wp, (d.O, kk, d.C))[...] = w.transpose(0, 2, 1)
+
+    def _from_wp(self, d, Wp):
+        assert real_api.conv2d_weights_plan(d, real_api.PASS_FWD) or real_api.conv2d_weights_plan(d, real_api.PASS_DGRAD)
+        return np.ascontiguousarray(self.f(Wp, (d.O, d.KH * d.KW, d.C)).transpose(0, 2, 1)).reshape(d.O, d.C, d.KH, d.KW)
+
+    def conv2d_fwd_pw(self, dev, d, X, Wp, bias, act, slope, Y, beta=0):
+        self.launches += 1
+        assert real_api.conv2d_weights_plan(d, real_api.PASS_FWD), 'forward of this geometry does not read permuted weights'
+        xs, ws, ys, pad = self._geom(d)
+        r = conv2d_fwd(self.f(X, xs), self._from_wp(d, Wp), d.stride, d.dilation, pad)
+        if bias is not None or act:
+            assert not beta
+            r = r.astype(np.float32)
+            if bias is not None:
+                r = r + self.f(bias, (d.O,)).reshape(1, -1, 1, 1)
+            if act == 1:
+                r = np.where(r >= 0, r, np.float32(slope) * r)
+        self._put(self.f(Y, ys), r, beta)
+
+    def conv2d_dgrad_pw(self, dev, d, dY, Wp, dX, beta=1):
+        self.launches += 1
+        assert real_api.conv2d_weights_plan(d, real_api.PASS_DGRAD), 'dgrad of this geometry does not read permuted weights'
+        xs, ws, ys, pad = self._geom(d)
+        self._put(self.f(dX, xs), conv2d_dx(self.f(dY, ys), self._from_wp(d, Wp), xs, d.stride, d.dilation, pad), beta)
+
+    def conv2d_wgrad_iohw(self, dev, d, X, dY, dW, beta=1):
+        self.launches += 1
+        assert real_api.conv2d_weights_plan(d, real_api.PASS_WGRAD), 'wgrad of this geometry cannot write swapped axes'
+        xs, ws, ys, pad = self._geom(d)
+        dw = conv2d_dw(self.f(X, xs), self.f(dY, ys), ws, d.stride, d.dilation, pad)
+        self._put(self.f(dW, (d.C, d.O, d.KH, d.KW)), dw.transpose(1, 0, 2, 3), beta)
 
     def depthwise_conv2d_fwd(self, dev, d, X, K, Y, beta=0):
         self.launches += 1

@@ -69,6 +69,73 @@ def test_conv2d_transpose_reference_style(nn_backend):
     assert n_cases > 250
 
 
+def test_conv2d_transpose_wide_channels(nn_backend):
+    """Channel counts for which the borrowed convolution passes read the kernel in their own permuted layout: the
+    copy is made straight from the kernel as stored, and the kernel gradient is written straight into its layout."""
+    nn = nn_backend
+    rs = np.random.RandomState(4)
+    for n, ic, oc, hw, ks, stride, padding in [(2, 32, 8, 6, 3, 2, 'same'), (1, 32, 32, 5, 5, 2, 'same'),
+                                                (2, 64, 32, 4, 3, 1, 'valid'), (1, 32, 36, 7, 4, 2, 'valid'),
+                                                (2, 96, 64, 3, 1, 1, 'same')]:
+        input_n = rs.randint(-3, 4, size=(n, ic, hw, hw)).astype(np.float32)
+        kernel_n = rs.randint(-3, 4, size=(oc, ic, ks, ks)).astype(np.float32)
+        input_t, kernel_t = nn.Tensor_from_value(input_n), nn.Tensor_from_value(kernel_n)
+        out_t = nn.conv2DTranspose(input_t, kernel_t, stride=stride, padding=padding)
+        grad_n = rs.randint(-3, 4, size=tuple(out_t.shape)).astype(np.float32)
+        y, dI, dK = conv2d_transpose_all(input_n, kernel_n, grad_n, stride, 1, padding)
+        assert np.array_equal(out_t.np(), y), (n, ic, oc, hw, ks, stride, padding)
+        input_t.get_grad().fill(1.0)
+        kernel_t.get_grad().fill(1.0)
+        nn.backward({out_t: grad_n}, grad_for_non_trainables=True)
+        assert np.array_equal(input_t.get_grad().np() - 1.0, dI), (n, ic, oc, hw, ks, stride, padding)
+        assert np.array_equal(kernel_t.get_grad().np() - 1.0, dK), (n, ic, oc, hw, ks, stride, padding)
+
+
+def test_permuted_weight_copy_is_shared_and_follows_the_weights(nn_backend, monkeypatch):
+    """Forward and data gradient read one cached copy of the kernel in the kernels' layout; the copy is made again
+    only after the kernel's contents may have changed (optimizer step, set, fill), and results stay exact."""
+    nn = nn_backend
+    from litenn_amd.core.hip import api
+    made = []
+    real = api.conv2d_permute_weights
+    monkeypatch.setattr(api, 'conv2d_permute_weights', lambda *a: (made.append(1), real(*a))[1])
+    rs = np.random.RandomState(9)
+    x_n = rs.randint(-2, 3, size=(2, 32, 7, 7)).astype(np.float32)
+    k_n = rs.randint(-2, 3, size=(32, 32, 3, 3)).astype(np.float32)
+    x_t, k_t = nn.Tensor_from_value(x_n), nn.Tensor_from_value(k_n)
+    opt = nn.optimizer.SGD([k_t], lr=0.5)
+
+    def step(expect_k):
+        y = nn.conv2D(x_t, k_t, stride=2)
+        g_n = np.ones(tuple(y.shape), np.float32)
+        ry, rdx, rdw = conv2d_all(x_n, expect_k, g_n, 2, 1, 'same')
+        assert np.array_equal(y.np(), ry)
+        opt.zero_grad()
+        nn.backward({y: g_n}, grad_for_non_trainables=True)
+        assert np.array_equal(x_t.get_grad().np(), rdx) and np.array_equal(k_t.get_grad().np(), rdw)
+        x_t.free_grad()
+        return rdw
+
+    dw = step(k_n)
+    assert len(made) == 1                       # forward made it, the data gradient reused it
+    nn.conv2D(x_t, k_t, stride=1).np()          # another geometry over the same kernel: same copy
+    step(k_n)
+    assert len(made) == 1
+    opt.step()                                  # the weights change ...
+    k2 = (k_n - 0.5 * dw).astype(np.float32)
+    step(k2)
+    assert len(made) == 2                       # ... and the copy follows
+    k_t.set(k_n)
+    step(k_n)
+    assert len(made) == 3
+    k_t.fill(1.0)
+    step(np.ones_like(k_n))
+    assert len(made) == 4
+    k_t.np()                                    # reading does not invalidate
+    step(np.ones_like(k_n))
+    assert len(made) == 4
+
+
 def test_conv2d_transpose_module_and_errors(nn_backend):
     nn = nn_backend
     rs = np.random.RandomState(2)

@@ -344,6 +344,105 @@ def test_conv_dgrad_few_input_channels_vector_kernel_integer_exact(hip):
             assert np.array_equal(dX.get() - (-2.0 if beta else 0.0), ref), (case, beta)
 
 
+def test_conv_dgrad_on_forward_permuted_weights_integer_exact(hip):
+    """With O a multiple of 32 and C a multiple of 4 (C > 4) the data gradient reads the weights in the forward
+    pass's layout Wp[o][tap][c], whatever the stride and the pixel class: channel counts that give one ragged,
+    one full and several row tiles of every tile shape, strides 1-3, dilation, every padding kind, '=' and '+=',
+    through lnn_conv2d_dgrad_f32 (copy made in scratch) and through lnn_conv2d_dgrad_pw_f32 on a copy made once
+    by lnn_conv2d_permute_weights_f32; the forward pass on the same copy where it reads one."""
+    rs = np.random.RandomState(61)
+    cnt = 0
+    for (C, O), s, d, ks, padding in itertools.product([(8, 32), (12, 64), (20, 32), (36, 96), (64, 64), (132, 32), (32, 160)],
+                                                       [1, 2, 3], [1, 2], [1, 2, 3, 5], ['same', 'valid', 1, (2, 0, 1, 3)]):
+        n, h, w_ = 2, 11 + s, 9 + 2 * s
+        try:
+            ci = info_conv2d(h, w_, ks, ks, s, d, padding)
+        except ValueError:
+            continue
+        if padding == 'valid' and min(h, w_) < (ks - 1) * d + 1:
+            continue
+        xs, ws = (n, C, h, w_), (O, C, ks, ks)
+        desc, _ = _desc(hip, xs, ws, s, d, padding)
+        assert hip.conv2d_weights_plan(desc, hip.PASS_DGRAD)
+        if cnt % 40 == 0:
+            say(f'dgrad on Wp case {cnt}: C={C} O={O} s={s} d={d} ks={ks} pad={padding}')
+        x = rs.randint(-3, 4, size=xs).astype(np.float32)
+        w = rs.randint(-3, 4, size=ws).astype(np.float32)
+        dy = rs.randint(-3, 4, size=(n, O, ci.OH, ci.OW)).astype(np.float32)
+        ry, rdx, _ = conv2d_all(x, w, dy, s, d, padding)
+        X, W, dY = DevArr(hip, x), DevArr(hip, w), DevArr(hip, dy)
+        Wp = DevArr(hip, shape=(O, ks * ks, C), fill=np.nan)
+        hip.conv2d_permute_weights(0, desc, W.ptr, hip.W_OIHW, Wp.ptr)
+        assert np.array_equal(Wp.get(), w.reshape(O, C, ks * ks).transpose(0, 2, 1))
+        beta, fill = (0, np.nan) if cnt % 2 else (1, 2.0)
+        for use_wp in (False, True):
+            dX = DevArr(hip, shape=xs, fill=fill)
+            if use_wp:
+                hip.conv2d_dgrad_pw(0, desc, dY.ptr, Wp.ptr, dX.ptr, beta)
+            else:
+                hip.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, beta)
+            assert np.array_equal(dX.get() - (2.0 if beta else 0.0), rdx), (C, O, s, d, ks, padding, use_wp)
+        if hip.conv2d_weights_plan(desc, hip.PASS_FWD):
+            Y = DevArr(hip, shape=dy.shape, fill=np.nan)
+            hip.conv2d_fwd_pw(0, desc, X.ptr, Wp.ptr, None, hip.ACT_NONE, 0.0, Y.ptr, 0)
+            assert np.array_equal(Y.get(), ry), (C, O, s, d, ks, padding)
+        cnt += 1
+    assert cnt > 500
+    # geometries whose kernels do not read Wp refuse the *_pw entry points
+    desc, _ = _desc(hip, (1, 3, 8, 8), (32, 3, 3, 3), 1, 1, 'same')
+    assert not hip.conv2d_weights_plan(desc, hip.PASS_DGRAD) and not hip.conv2d_weights_plan(desc, hip.PASS_FWD)
+    A = DevArr(hip, shape=(4096,), fill=0.0)
+    with pytest.raises(hip.HipException) as e:
+        hip.conv2d_dgrad_pw(0, desc, A.ptr, A.ptr, A.ptr, 0)
+    assert e.value.code == hip.ERR_INVALID
+    with pytest.raises(hip.HipException) as e:
+        hip.conv2d_fwd_pw(0, desc, A.ptr, A.ptr, None, hip.ACT_NONE, 0.0, A.ptr, 0)
+    assert e.value.code == hip.ERR_INVALID
+
+
+def test_conv_passes_on_weights_with_swapped_channel_axes(hip):
+    """A transposed convolution keeps its kernel as [C][O][KH][KW] relative to the convolution whose passes it
+    borrows.  lnn_conv2d_permute_weights_f32(LNN_W_IOHW) makes Wp straight from that storage, the *_pw passes run
+    on it, and lnn_conv2d_wgrad_iohw_f32 writes the weight gradient in that storage ('=' and '+=', split-K
+    reduction and direct epilogue), all exact against the oracle on the explicitly swapped kernel."""
+    rs = np.random.RandomState(62)
+    cases = [((2, 64, 12, 12), (64, 64, 5, 5), 2, 1, 2), ((3, 128, 9, 10), (32, 128, 3, 3), 1, 1, 'same'),
+             ((2, 128, 8, 8), (160, 128, 3, 3), 1, 2, 'same'), ((1, 32, 20, 20), (96, 32, 1, 1), 1, 1, 'valid'),
+             ((16, 128, 32, 32), (256, 128, 5, 5), 2, 1, 2), ((2, 64, 6, 33), (40, 64, 2, 2), 1, 1, 'valid')]
+    for xs, ws, s, d, padding in cases:
+        say(f'swapped-axes weights x={xs} w={ws} s={s} d={d} pad={padding}')
+        desc, ci = _desc(hip, xs, ws, s, d, padding)
+        O, C, KH, KW = ws
+        x = rs.randint(-2, 3, size=xs).astype(np.float32)
+        w = rs.randint(-2, 3, size=ws).astype(np.float32)
+        dy = rs.randint(-2, 3, size=(xs[0], O, ci.OH, ci.OW)).astype(np.float32)
+        ry, rdx, rdw = conv2d_all(x, w, dy, s, d, padding)
+        w_io = np.ascontiguousarray(w.transpose(1, 0, 2, 3))          # how the caller stores it
+        X, Wio, dY = DevArr(hip, x), DevArr(hip, w_io), DevArr(hip, dy)
+        Wp = DevArr(hip, shape=(O, KH * KW, C), fill=np.nan)
+        hip.conv2d_permute_weights(0, desc, Wio.ptr, hip.W_IOHW, Wp.ptr)
+        assert np.array_equal(Wp.get(), w.reshape(O, C, KH * KW).transpose(0, 2, 1))
+        assert hip.conv2d_weights_plan(desc, hip.PASS_FWD) and hip.conv2d_weights_plan(desc, hip.PASS_WGRAD)
+        Y = DevArr(hip, shape=dy.shape, fill=np.nan)
+        hip.conv2d_fwd_pw(0, desc, X.ptr, Wp.ptr, None, hip.ACT_NONE, 0.0, Y.ptr, 0)
+        assert np.array_equal(Y.get(), ry)
+        if hip.conv2d_weights_plan(desc, hip.PASS_DGRAD):
+            dX = DevArr(hip, shape=xs, fill=1.0)
+            hip.conv2d_dgrad_pw(0, desc, dY.ptr, Wp.ptr, dX.ptr, 1)
+            assert np.array_equal(dX.get() - 1.0, rdx)
+        for beta, fill in ((0, np.nan), (1, -3.0)):
+            dWio = DevArr(hip, shape=w_io.shape, fill=fill)
+            hip.conv2d_wgrad_iohw(0, desc, X.ptr, dY.ptr, dWio.ptr, beta)
+            assert np.array_equal(dWio.get() - (-3.0 if beta else 0.0), rdw.transpose(1, 0, 2, 3)), (xs, ws, beta)
+    # a geometry on the table-driven weight-gradient kernel cannot write swapped axes
+    desc, _ = _desc(hip, (1, 3, 8, 8), (8, 3, 3, 3), 1, 1, 'same')
+    assert not hip.conv2d_weights_plan(desc, hip.PASS_WGRAD)
+    A = DevArr(hip, shape=(4096,), fill=0.0)
+    with pytest.raises(hip.HipException) as e:
+        hip.conv2d_wgrad_iohw(0, desc, A.ptr, A.ptr, A.ptr, 0)
+    assert e.value.code == hip.ERR_UNSUPPORTED
+
+
 def test_conv_few_tiles_split_k_integer_exact(hip):
     """Deep layers on small images have a long K and few output tiles: forward
     and dgrad then split K over the idle compute units and a second kernel
