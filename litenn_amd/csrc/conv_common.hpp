@@ -30,6 +30,9 @@
 #ifndef LNN_SMALL_DGRAD
 #define LNN_SMALL_DGRAD 1
 #endif
+#ifndef LNN_WGRAD_ANYC
+#define LNN_WGRAD_ANYC 1
+#endif
 #ifndef LNN_WGRAD_B_DIRECT
 #define LNN_WGRAD_B_DIRECT 1
 #endif
@@ -125,6 +128,9 @@ __device__ __forceinline__ void reduce_body(float* out, const float* part, const
     col = (uint32_t)i - m * (uint32_t)a.ncols;
     const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
     const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+    // the additions stay in slice order; unrolled so that several slices' loads are in flight together (many
+    // slices over a tiny output, the weight gradient of an image stem, would otherwise pay one latency per slice)
+#pragma unroll 8
     for (int k = ls; k < ns; k += 8) s += part[(size_t)k * a.n + i];
   }
   red[ls][li] = s;
@@ -152,6 +158,7 @@ __device__ __forceinline__ void reduce_body4(float* out, const float* part, cons
     const uint32_t m = a.dN.div((uint32_t)i4), col = (uint32_t)i4 - m * (uint32_t)a.ncols;
     const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
     const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+#pragma unroll 4
     for (int k = ls; k < ns; k += 8) s += *reinterpret_cast<const f32x4*>(&part[(size_t)k * a.n + i4]);
   }
   *reinterpret_cast<f32x4*>(&red[ls][4 * q]) = s;
@@ -189,9 +196,10 @@ __global__ __launch_bounds__(256) void reduce_partials_batch(ReduceBatch b) {
 
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
 // PASS_WGRAD_TAP4: PASS_WGRAD_TAP with 128-bit transfers of the pixel gather too (stride 1, OW % 4 == 0, no padded columns)
+// PASS_WGRAD_ANYC: wgrad for any channel count with transfers straight into LDS, columns in (c, kh, kw) order
 // PASS_DGRAD_TAPW: tap-major dgrad that reads the weights in the forward pass's permuted layout (C % 4 == 0)
 enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5, PASS_WGRAD_TAP4 = 6,
-       PASS_DGRAD_TAPW = 7 };
+       PASS_DGRAD_TAPW = 7, PASS_WGRAD_ANYC = 8 };
 constexpr bool wgrad_tap(int pass) { return pass == PASS_WGRAD_TAP || pass == PASS_WGRAD_TAP4; }
 constexpr bool dgrad_tap(int pass) { return pass == PASS_DGRAD_TAP || pass == PASS_DGRAD_TAPW; }
 
@@ -231,12 +239,12 @@ template <int PASS, int WM, int NTMAX, bool FLAG>
 struct ConvCfg {
   static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
   // the tap-major passes send both operands straight into unpadded LDS tiles, three stages deep
-  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || dgrad_tap(PASS) || wgrad_tap(PASS);
+  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || dgrad_tap(PASS) || wgrad_tap(PASS) || PASS == PASS_WGRAD_ANYC;
   // A side is K-contiguous in LDS for all passes.
   static constexpr int SA = DIRECT ? BM * BK : LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
   static constexpr int SB = DIRECT ? BNMAX * BK : LdsSize<PASS == PASS_WGRAD, BNMAX>::value;
-  static constexpr int STAGES = !DIRECT ? 2 : (wgrad_tap(PASS) ? LNN_STAGES_WGRAD : LNN_STAGES_FD);
+  static constexpr int STAGES = !DIRECT ? 2 : (wgrad_tap(PASS) || PASS == PASS_WGRAD_ANYC ? LNN_STAGES_WGRAD : LNN_STAGES_FD);
 };
 
 // Loader selection and initialisation per pass.  FLAG:
@@ -313,6 +321,15 @@ struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
 };
 
 template <bool FLAG, int ST>
+struct ConvProblem<PASS_WGRAD_ANYC, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
+  template <int R> using LA = typename std::conditional<FLAG, ConvWgradTapA4Direct<R>, ConvWgradTapADirect<R>>::type;
+  template <int R> using LB = ConvWgradBAnyC<R>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A& la) const { l.init(rx, g, col0, Ncols, la, kend, kbeg); }
+};
+
+template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_TAP4, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = ConvWgradTapA4Direct<R>;
@@ -344,11 +361,11 @@ __host__ __device__ inline OutMap final_map(const ConvArgs& a) {
   return om;
 }
 
+// (bx, by): this workgroup's position in the problem's own grid (x: share of the output, y: K slice)
 template <int PASS, int WM, int NTMAX, bool FLAG>
-__device__ __forceinline__ void conv_body(const ConvArgs& a) {
+__device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
   using Cfg = ConvCfg<PASS, WM, NTMAX, FLAG>;
   __shared__ __attribute__((aligned(16))) float lds[Cfg::STAGES * (Cfg::SA + Cfg::SB)];
-  if ((int)blockIdx.x >= a.grid_x || (int)blockIdx.y >= (a.ksplit > 1 ? a.ksplit : 1)) return;   // batched launch: not ours
   ConvProblem<PASS, FLAG, Cfg::STAGES> p;
   p.g = a.g;
   p.tab = a.tab;
@@ -358,13 +375,13 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a) {
   p.kbeg = 0;
   p.kend = a.K;
   float* out = a.Out;
-  int chunk_i = blockIdx.x;
+  int chunk_i = bx;
   if (a.ksplit > 1) {
     // K slice of this workgroup: slices are in gridDim.y, except that the tap-major wgrad pass has a flat
     // grid in which the last chunk, if it holds less work, is cut into proportionally fewer slices
-    int slice = blockIdx.y, ns = a.ksplit;
+    int slice = by, ns = a.ksplit;
     if (wgrad_tap(PASS)) {
-      const int b = blockIdx.x, nfull = (a.n_chunks - 1) * a.ksplit;
+      const int b = bx, nfull = (a.n_chunks - 1) * a.ksplit;
       if (b < nfull) {
         chunk_i = b / a.ksplit;
         slice = b - chunk_i * a.ksplit;
@@ -391,23 +408,32 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a) {
                               a.chunk_units, chunk_i);
   else
     walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units,
-                          (int)blockIdx.x, a.grid_x);
+                          bx, a.grid_x);
 }
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
 __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
-  conv_body<PASS, WM, NTMAX, FLAG>(a);
+  conv_body<PASS, WM, NTMAX, FLAG>(a, (int)blockIdx.x, (int)blockIdx.y);
 }
 
-// Several independent problems of one pass in one launch (the pixel classes of a strided dgrad):
-// blockIdx.z selects the problem, each uses the leading part of the x / y grid it asked for.
+// Several independent problems of one pass in one launch (the pixel classes of a strided dgrad).  The grid is
+// flat and holds exactly the workgroups the problems asked for, problem after problem (first[i] = where problem
+// i's begin): a launch that also carried workgroups with nothing to do would, when the useful ones number as many
+// as the chip has compute units, leave some unit with two of them in a row.
 constexpr int kMaxBatch = 4;
 struct ConvArgsBatch {
   ConvArgs c[kMaxBatch];
+  int first[kMaxBatch + 1];
 };
 template <int PASS, int WM, int NTMAX>
 __global__ __launch_bounds__(512, 2) void conv_kernel_batch(ConvArgsBatch b) {
-  conv_body<PASS, WM, NTMAX, true>(b.c[blockIdx.z]);
+  const int lin = blockIdx.x;
+  int i = 0;
+#pragma unroll
+  for (int q = 1; q < kMaxBatch; ++q) i += lin >= b.first[q];
+  const int local = lin - b.first[i], gx = b.c[i].grid_x;
+  const int by = local / gx;
+  conv_body<PASS, WM, NTMAX, true>(b.c[i], local - by * gx, by);
 }
 
 // ---------------------------------------------------------------------------
@@ -576,7 +602,7 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   float* final_out = a.Out;
   const int final_beta = a.beta;
   int grid_y = 1;
-  if (PASS == PASS_WGRAD || wgrad_tap(PASS)) {
+  if (PASS == PASS_WGRAD || PASS == PASS_WGRAD_ANYC || wgrad_tap(PASS)) {
     const int m_tiles = (a.M + BM - 1) / BM;
     a.n_units = (a.Ncols + 32 * WN - 1) / (32 * WN);
     long long total = (long long)m_tiles * a.n_units;
@@ -639,7 +665,7 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     }
   }
   dim3 g(a.grid_x, grid_y, 1), b(512, 1, 1);
-  constexpr bool kUsesFlag = PASS == PASS_FWD || PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP;   // the other passes have one variant
+  constexpr bool kUsesFlag = PASS == PASS_FWD || PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP || PASS == PASS_WGRAD_ANYC;   // the other passes have one variant
   if (flag || !kUsesFlag) {
     hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, true>), g, b, 0, ctx->stream, a);
   } else if constexpr (kUsesFlag) {
@@ -663,26 +689,43 @@ static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_
   // (256 -> 512 channels at 16 x 16: 77 -> 63 us).
   std::vector<long long> share(n, equal);
   if (LNN_CLASS_SHARES && dgrad_tap(PASS) && n <= kMaxBatch) {
-    std::vector<long long> prop(n, equal);
-    long long total = 0, given = 0;
-    for (int i = 0; i < n; ++i) total += (long long)cls[i].K * cls[i].Ncols;
-    for (int i = 0; i < n && total > 0; ++i) {
-      prop[i] = (long long)ctx->cus * cls[i].K * cls[i].Ncols / total;
-      prop[i] = prop[i] < 1 ? 1 : prop[i];
-      given += prop[i];
-    }
-    for (int i = 0; given > ctx->cus && i < n; ++i)
-      if (prop[i] > 1) { --prop[i]; --given; }
     // Only where every class is cut along K anyway (few output tiles: any share divides into whole sub-tiles times
     // K slices).  Classes with many tiles and no K split lose more to the narrow sub-tiles of an odd share than
     // they gain (64 -> 128 channels at 64 x 64: 82 -> 121 us).
     bool all_split = true;
+    std::vector<long long> chunks(n), nkt(n);
     for (int i = 0; i < n; ++i) {
       ConvArgs a = cls[i];
       plan_tiles<WM, NTMAX>(a, equal);
       all_split = all_split && a.total_units >= 0 && a.ksplit > 1;
+      chunks[i] = a.grid_x;                       // full sub-tiles of this class
+      nkt[i] = (cls[i].K + BK - 1) / BK;
     }
-    if (all_split) share = prop;
+    if (all_split) {
+      // K slices per class so that the longest slice of any class is as short as the chip allows: start from one
+      // slice each and keep giving one more to the class whose slices are longest while workgroups are left
+      // (5x5 stride 2, 256 -> 512 channels at 16 x 16: 72 / 48 / 48 / 32 K steps in 5 / 4 / 4 / 3 slices instead of
+      // the 5 / 3 / 3 / 2 that shares in proportion to the work round down to)
+      std::vector<long long> ks(n, 1);
+      long long used = 0;
+      for (int i = 0; i < n; ++i) used += chunks[i];
+      for (;;) {
+        int best = -1;
+        for (int i = 0; i < n; ++i) {
+          if (used + chunks[i] > ctx->cus || ks[i] + 1 > nkt[i] / 8) continue;   // plan_tiles caps slices at nkt / 8
+          if (best < 0 || nkt[i] * ks[best] > nkt[best] * ks[i]) best = i;
+        }
+        if (best < 0) break;
+        // stop when the class with the longest slices cannot be helped: more slices elsewhere shorten nothing
+        int longest = 0;
+        for (int i = 1; i < n; ++i)
+          if (nkt[i] * ks[longest] > nkt[longest] * ks[i]) longest = i;
+        if (best != longest) break;
+        ++ks[best];
+        used += chunks[best];
+      }
+      for (int i = 0; i < n; ++i) share[i] = chunks[i] * ks[i];
+    }
   }
   std::vector<float*> final_out(n);
   std::vector<int> final_beta(n);
@@ -702,18 +745,17 @@ static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_
   for (int i0 = 0; i0 < n; i0 += kMaxBatch) {
     const int nb = n - i0 < kMaxBatch ? n - i0 : kMaxBatch;
     ConvArgsBatch b;
-    int gx = 1, gy = 1;
-    for (int i = 0; i < nb; ++i) {
-      b.c[i] = cls[i0 + i];
-      if (b.c[i].grid_x > gx) gx = b.c[i].grid_x;
-      if (b.c[i].ksplit > gy) gy = b.c[i].ksplit;
+    int total = 0;
+    for (int i = 0; i < kMaxBatch; ++i) {
+      b.c[i] = cls[i0 + (i < nb ? i : 0)];
+      b.first[i] = total;
+      if (i < nb) total += b.c[i].grid_x * (b.c[i].ksplit > 1 ? b.c[i].ksplit : 1);
     }
-    for (int i = nb; i < kMaxBatch; ++i) {
-      b.c[i] = cls[i0];
-      b.c[i].grid_x = 0;
+    b.first[kMaxBatch] = total;
+    if (total > 0) {
+      hipLaunchKernelGGL((conv_kernel_batch<PASS, WM, NTMAX>), dim3(total), dim3(512, 1, 1), 0, ctx->stream, b);
+      LNN_HIP(hipGetLastError());
     }
-    hipLaunchKernelGGL((conv_kernel_batch<PASS, WM, NTMAX>), dim3(gx, gy, nb), dim3(512, 1, 1), 0, ctx->stream, b);
-    LNN_HIP(hipGetLastError());
   }
   // the K-split classes' reductions, kMaxReduceBatch per launch
   ReduceBatch rb;

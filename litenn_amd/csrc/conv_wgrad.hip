@@ -28,7 +28,10 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
     return launch_by_m<PASS_WGRAD_TAP>(ctx, a, vec);
   }
   if (w_iohw) return set_error(LNN_ERR_UNSUPPORTED, "conv2d_wgrad: this geometry cannot write a gradient with swapped channel axes");
-  // the table-driven kernel: per-column gather entries
+  // any channel count: columns in the weights' own (c, kh, kw) order, both operands straight into LDS (the walkers
+  // move a lane's pixel by one K step with single wrap tests, as in the pixel-major kernels)
+  if (LNN_WGRAD_ANYC && g.OHW >= BK && BK / g.OW + 1 <= g.OH) return launch_by_m<PASS_WGRAD_ANYC>(ctx, a, vec);
+  // tiny images: the table-driven kernel with per-column gather entries
   st = reserve_tables(ctx, 1);
   if (st != LNN_OK) return st;
   st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);

@@ -32,6 +32,9 @@
 
 namespace lnn {
 
+#ifndef LNN_REQUEST_FIRST
+#define LNN_REQUEST_FIRST 0
+#endif
 constexpr int BK = 32;            // K extent of one LDS stage
 constexpr int KG = BK / 4;        // float4 groups along K
 constexpr int KR = BK / 4;        // K rows fetched per wavefront of a group in the pixel-major gathers
@@ -195,14 +198,16 @@ struct DirectKC {
       voff[e] = row < M ? (uint32_t)(row * ld + kg * 4) * 4u : OOB;
     }
   }
-  // off: first tile row of this group
-  __device__ __forceinline__ void issue(int k0, float* lds, int, int off) {
+  // off: first tile row of this group.  Returns the number of transfers this wavefront issued.
+  __device__ __forceinline__ int issue(int k0, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
+    int n = 0;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const int blk = wave + 4 * e;
-      if (NB % 4 == 0 || blk < NB) buf_load_lds16(rs, lds + (off + blk * 8) * BK, voff[e], (uint32_t)k0 * 4u);
+      if (NB % 4 == 0 || blk < NB) { buf_load_lds16(rs, lds + (off + blk * 8) * BK, voff[e], (uint32_t)k0 * 4u); ++n; }
     }
+    return n;
   }
 };
 
@@ -230,14 +235,16 @@ struct DirectMC {
       voff[e] = (k < BK && row0 + n < M) ? (uint32_t)(k * ld + row0 + n) * 4u : OOB;
     }
   }
-  __device__ __forceinline__ void issue(int k0, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const uint32_t soff = (uint32_t)(k0 * ld) * 4u;
+    int n = 0;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const int q = wave + 4 * e;
-      if (NI % 4 == 0 || q < NI) buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff);
+      if (NI % 4 == 0 || q < NI) { buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff); ++n; }
     }
+    return n;
   }
 };
 
@@ -451,7 +458,7 @@ struct ConvFwdBTap {
     }
   }
   // straight into the LDS stage: element (k = wave + 4e, column lane + 64c)
-  __device__ __forceinline__ void issue(int, float* lds, int ld, int off) {
+  __device__ __forceinline__ int issue(int, float* lds, int ld, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < KR; ++e) {
@@ -461,6 +468,7 @@ struct ConvFwdBTap {
         if (R % 64 == 0 || lane + 64 * c < R) buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);
     }
     advance();
+    return NLD;
   }
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
@@ -536,7 +544,7 @@ struct ConvDgradBTap {
     }
   }
   // straight into the LDS stage: element (k = wave + 4e, column lane + 64c)
-  __device__ __forceinline__ void issue(int, float* lds, int ld, int off) {
+  __device__ __forceinline__ int issue(int, float* lds, int ld, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < KR; ++e) {
@@ -546,6 +554,7 @@ struct ConvDgradBTap {
         if (R % 64 == 0 || lane + 64 * c < R) buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);
     }
     advance();
+    return NLD;
   }
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
@@ -591,13 +600,14 @@ struct ConvDgradATapMC {
       voff[e] = (k < BK && row0 + n < g.C) ? (uint32_t)(k * ld + row0 + n) * 4u : OOB;
     }
   }
-  __device__ __forceinline__ void issue(int, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const uint32_t soff = (uint32_t)(o0 * ld + cw * C) * 4u;
+    int n = 0;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const int q = wave + 4 * e;
-      if (NI % 4 == 0 || q < NI) buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff);
+      if (NI % 4 == 0 || q < NI) { buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff); ++n; }
     }
     o0 += BK;
     if (o0 >= O) {   // wave-uniform: next tap of the class
@@ -606,6 +616,7 @@ struct ConvDgradATapMC {
       cw = nw;
       nw = (tab + tap + 1)->w;
     }
+    return n;
   }
 };
 
@@ -962,7 +973,7 @@ struct ConvWgradTapADirect {
     rem = p - (int)img * g.OHW;
     aoff = (int)img * g.O * g.OHW + rem + (o0 + 2 * gwave() + (int)((threadIdx.x & 63) >> 5)) * g.OHW;
   }
-  __device__ __forceinline__ void issue(int, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     // rows past the last output channel are never stored, so they need no mask
     const uint32_t voff = p < kend ? (uint32_t)aoff * 4u : OOB;
@@ -971,6 +982,7 @@ struct ConvWgradTapADirect {
       buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, voff, (uint32_t)(8 * e * OHW) * 4u);
     p += BK; rem += BK; aoff += BK;
     if (rem >= OHW) { rem -= OHW; aoff += awrap; }
+    return E;
   }
 };
 
@@ -997,15 +1009,19 @@ struct ConvWgradTapA4Direct {
     rem = p - (int)img * g.OHW;
     aoff = (int)img * g.O * g.OHW + rem + (o0 + 8 * gwave() + rb) * g.OHW;
   }
-  __device__ __forceinline__ void issue(int, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const uint32_t voff = p < kend ? (uint32_t)aoff * 4u : OOB;   // kend is a multiple of 4 here: whole groups
+    int n = 0;
 #pragma unroll
     for (int e = 0; e < E; ++e)
-      if (NB % 4 == 0 || wave + 4 * e < NB)
+      if (NB % 4 == 0 || wave + 4 * e < NB) {
         buf_load_lds16(rs, lds + (off + (wave + 4 * e) * 8) * BK, voff, (uint32_t)(32 * e * OHW) * 4u);
+        ++n;
+      }
     p += BK; rem += BK; aoff += BK;
     if (rem >= OHW) { rem -= OHW; aoff += awrap; }
+    return n;
   }
 };
 
@@ -1046,7 +1062,7 @@ struct ConvWgradTapBDirect {
     iw = ow * g.S + kw * g.D - g.PADL;
     xoff = ((int)img * g.C + c0 + 2 * gwave() + (int)((threadIdx.x & 63) >> 5)) * g.IHW + ih * g.IW + iw;
   }
-  __device__ __forceinline__ void issue(int, float* lds, int, int off) { go<true>(lds, off); }
+  __device__ __forceinline__ int issue(int, float* lds, int, int off) { go<true>(lds, off); return E; }
   __device__ __forceinline__ void fetch(int) { go<false>(nullptr, 0); }
   __device__ __forceinline__ void commit(float* lds, int, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
@@ -1109,16 +1125,84 @@ struct ConvWgradTapB4Direct {
     ih = oh + kh * g.D - g.PADT;
     xoff = ((int)img * g.C + c0 + 8 * gwave() + rb) * g.IHW + ih * g.IW + ow + kw * g.D;
   }
-  __device__ __forceinline__ void issue(int, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const uint32_t voff = p < kend && (uint32_t)ih < (uint32_t)IH ? (uint32_t)xoff * 4u : OOB;
+    int n = 0;
 #pragma unroll
     for (int e = 0; e < E; ++e)
-      if (NB % 4 == 0 || wave + 4 * e < NB)
+      if (NB % 4 == 0 || wave + 4 * e < NB) {
         buf_load_lds16(rs, lds + (off + (wave + 4 * e) * 8) * BK, voff, (uint32_t)(32 * e * IHW) * 4u);
+        ++n;
+      }
     p += BK; oh += qh; ow += rw; ih += qh; xoff += x_step;
     if (ow >= OW) { ow -= OW; ++oh; ++ih; xoff += xwrap_w; }
     if (oh >= OH) { oh -= OH; ih -= OH; xoff += xwrap_h; }
+    return n;
+  }
+};
+
+// wgrad pixel gather for any channel count, GEMM columns in the weights' own order q = (c, kh, kw), sent straight
+// into a swizzled K-contiguous LDS tile like ConvWgradTapBDirect: a lane owns one fixed pixel position of the K
+// step (carried forward by additions and single wrap tests) and, per transfer, one column - lanes 0..31 the even
+// row of the pair, lanes 32..63 the odd one - whose three constants (element offset from the window's origin, row
+// and column displacement of its tap for the padding test) it keeps in registers for the whole kernel.  Lanes run
+// over consecutive output pixels, so a transfer reads a run of image-row floats S apart: a handful of cache lines,
+// where lanes over the columns of one pixel touch some thirty.  Columns past C*KH*KW arrive as zeros.
+template <int R>
+struct ConvWgradBAnyC {
+  static constexpr bool KC = true, DIRECT = true;
+  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int E = R / 8, NLD = E;
+  static_assert(R % 8 == 0, "whole row pairs for all four wavefronts");
+  rsrc_t rs;
+  int IH, IW, OH, OW, kend;
+  int coff[E], yy[E], zz[E];   // this lane's column of transfer e
+  int p, oh, ow;               // this lane's output pixel, its row and column inside the image
+  int ih, iw;                  // oh*S - PADT, ow*S - PADL: origin of the pixel's window
+  int xoff;                    // its element offset (channel 0)
+  int qh, rw, s_q, s_r, x_step, s_OW, s_OH, S, xwrap_w, xwrap_h;   // see ConvWgradTapBDirect
+  template <class LA>
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int col0, int Q, const LA&, int kend_, int k0) {
+    rs = r;
+    IH = g.IH; IW = g.IW; OH = g.OH; OW = g.OW; S = g.S;
+    kend = kend_;
+    const int half = (int)((threadIdx.x & 63) >> 5);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int q = col0 + 8 * e + 2 * gwave() + half;
+      const bool ok = q < Q;
+      const int qq = ok ? q : 0;
+      const int ch = qq / g.KK, tap = qq - ch * g.KK, kh = tap / g.KW, kw = tap - kh * g.KW;
+      yy[e] = ok ? kh * g.D : BIG;
+      zz[e] = kw * g.D;
+      coff[e] = ch * g.IHW + kh * g.D * g.IW + kw * g.D;
+    }
+    qh = BK / g.OW; rw = BK - qh * g.OW;
+    s_q = g.S * qh; s_r = g.S * rw; s_OW = g.S * g.OW; s_OH = g.S * g.OH;
+    x_step = s_q * g.IW + s_r;
+    xwrap_w = g.S * g.IW - s_OW;              // column wrap: one row down, OW columns back
+    xwrap_h = g.C * g.IHW - s_OH * g.IW;      // row wrap: next image, OH rows back
+    p = k0 + wgrad_direct_k();
+    const uint32_t img = g.dOHW.div((uint32_t)p), rem = (uint32_t)p - img * g.OHW;
+    oh = (int)g.dOW.div(rem);
+    ow = (int)rem - oh * g.OW;
+    ih = oh * g.S - g.PADT;
+    iw = ow * g.S - g.PADL;
+    xoff = (int)img * g.C * g.IHW + ih * g.IW + iw;
+  }
+  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+    const int ihm = p < kend ? ih : BIG;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const bool ok = (uint32_t)(ihm + yy[e]) < (uint32_t)IH && (uint32_t)(iw + zz[e]) < (uint32_t)IW;
+      buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, ok ? (uint32_t)(xoff + coff[e]) * 4u : OOB, 0);
+    }
+    p += BK; oh += qh; ow += rw; ih += s_q; iw += s_r; xoff += x_step;
+    if (ow >= OW) { ow -= OW; ++oh; iw -= s_OW; ih += S; xoff += xwrap_w; }
+    if (oh >= OH) { oh -= OH; ih -= s_OH; xoff += xwrap_h; }
+    return E;
   }
 };
 
@@ -1298,12 +1382,25 @@ __device__ __forceinline__ void wait_transfers() {
   if (ANY_DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// All global -> LDS transfers of this wavefront have landed except the n it issued last (they complete in order).
+// n is wave-uniform and, after inlining, a constant in nearly every instantiation.
+__device__ __forceinline__ void wait_transfers_but(int n) {
+#define LNN_W(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
+  switch (n) {
+    LNN_W(1) LNN_W(2) LNN_W(3) LNN_W(4) LNN_W(5) LNN_W(6) LNN_W(7) LNN_W(8) LNN_W(9) LNN_W(10) LNN_W(11) LNN_W(12)
+    LNN_W(13) LNN_W(14) LNN_W(15) LNN_W(16) LNN_W(17) LNN_W(18) LNN_W(19) LNN_W(20) LNN_W(21) LNN_W(22) LNN_W(23) LNN_W(24)
+    LNN_W(25) LNN_W(26) LNN_W(27) LNN_W(28) LNN_W(29) LNN_W(30) LNN_W(31) LNN_W(32)
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;   // none issued, or more than the counter is trusted for
+  }
+#undef LNN_W
+}
+
 template <class LB, class LA>
-__device__ __forceinline__ void issue_b(LB& lb, int k0, float* lds, int ld, int off, LA& la) {
+__device__ __forceinline__ int issue_b(LB& lb, int k0, float* lds, int ld, int off, LA& la) {
   if constexpr (needs_a<LB>::value)
-    lb.issue(k0, lds, ld, off, la);
+    return lb.issue(k0, lds, ld, off, la);
   else
-    lb.issue(k0, lds, ld, off);
+    return lb.issue(k0, lds, ld, off);
 }
 
 // Body of one group (G = 0 or 1) for one sub-tile: BM = 32*WM rows shared by
@@ -1344,11 +1441,13 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
   static_assert(ST == 3 || (!DA && !DB) || (DA && DB), "a mix of direct and register-staged loaders needs three stages");
   // request: ask global memory for a K step, into an LDS stage (direct loader) or into registers;
   // land: park a register-staged K step in its LDS stage
-  auto request = [&](int k0, int stage) {
-    if constexpr (DA) la.issue(k0, ldsA + stage * strideA, LDA, G * HALF); else la.fetch(k0);
+  auto request = [&](int k0, int stage) -> int {   // number of global -> LDS transfers issued by this wavefront
+    int n = 0;
+    if constexpr (DA) n += la.issue(k0, ldsA + stage * strideA, LDA, G * HALF); else la.fetch(k0);
     if constexpr (NT > 0) {
-      if constexpr (DB) issue_b(lb, k0, ldsB + stage * strideB, LDB, COFF, la); else fetch_b(lb, k0, la);
+      if constexpr (DB) n += issue_b(lb, k0, ldsB + stage * strideB, LDB, COFF, la); else fetch_b(lb, k0, la);
     }
+    return n;
   };
   auto land = [&](int stage) {
     if constexpr (!DA) la.commit(ldsA + stage * strideA, LDA, G * HALF);
@@ -1396,6 +1495,13 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
       for (int phase = 0; phase < 2; ++phase) {
         if (phase == G) {
           compute(cur);
+        } else if constexpr (DA && DB && LNN_REQUEST_FIRST) {
+          // K step t+2 goes out first (into the stage last read for step t-1), then the wait for step t+1, which
+          // has been in flight for a whole step, leaves those newest transfers outstanding: every transfer gets
+          // close to two steps to land, which short steps (narrow tiles) need
+          int n = 0;
+          if (t + 2 < nk) n = request(kbeg + (t + 2) * BK, nn);
+          if (t + 1 < nk) wait_transfers_but(n);
         } else {
           if (t + 1 < nk) {
             wait_transfers<DA || DB>();
