@@ -273,9 +273,9 @@ struct ConvProblem<PASS_FWD, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_FWD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  template <int R> using LA = DirectKC<R>;               // permuted weights [O][KK*C]
+  template <int R> using LA = ConvFwdATap<R>;            // permuted weights [O][KK*C]
   template <int R> using LB = ConvFwdBTap<R, LNN_FD_B_DIRECT != 0>;
-  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, M, kbeg); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, col0, Ncols, kbeg); }
 };
 template <bool FLAG, int ST>
@@ -298,9 +298,10 @@ template <bool FLAG, int ST>
 struct ConvProblem<PASS_DGRAD_TAPW, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = ConvDgradATapMC<R>;        // the forward pass's permuted weights [O][KK*C]
-  template <int R> using LB = ConvDgradBTap<R, LNN_FD_B_DIRECT != 0>;
-  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, tab, row0, kbeg); }
-  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
+  template <int R> using LB = ConvDgradBTap<R, LNN_FD_B_DIRECT != 0, LNN_CB_MAJOR != 0>;
+  // K = O * (taps of the pixel class)
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, tab, row0, kbeg, K / g.O); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg, K / g.O); }
 };
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD, FLAG, ST> : ConvProblemBase {

@@ -5,6 +5,9 @@
 
 #include "common.hpp"
 
+#ifndef LNN_GEMM_XCD_BLOCKS
+#define LNN_GEMM_XCD_BLOCKS 1
+#endif
 #ifndef LNN_STAGES_GEMM
 #define LNN_STAGES_GEMM 2
 #endif
@@ -20,6 +23,12 @@ struct GemmArgs {
   uint32_t bytesA, bytesB, bytesC;  // extent of one batch item
   int beta;
   int n_units, total_units;       // schedule: units of 32*WN columns per M tile
+  // Workgroup -> share of the output.  The hardware deals consecutive workgroups round-robin to the 8 XCDs (each
+  // with its own L2), so by default an XCD's workgroups sit in every row of tiles and share only the B operand.
+  // With xcd_bc > 0 the workgroups of one XCD own a block of xcd_br tile rows x xcd_bc shares per row instead,
+  // so that xcd_bc of them read the same A tiles and xcd_br the same B tiles out of their L2 (wg_per_row shares
+  // make up a row of tiles).
+  int xcd_br, xcd_bc, wg_per_row;
 };
 
 // MODE: how operands travel.  0: 32-bit loads through registers (any alignment,
@@ -65,7 +74,13 @@ __global__ __launch_bounds__(512, 2) void gemm_kernel(GemmArgs a) {
   p.kbeg = 0; p.kend = a.K; p.beta = a.beta;
   p.post.bias = nullptr; p.post.act = 0; p.post.slope = 0.0f;
   p.om.nchw = 0; p.om.ld = a.ldc; p.om.mtot = 0; p.om.dHW = FastDiv{0, 0, 1};
-  walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units, (int)blockIdx.x, (int)gridDim.x);
+  int wg = (int)blockIdx.x;
+  if (a.xcd_bc > 0) {
+    const int xcd = wg & 7, j = wg >> 3, blocks_per_row = a.wg_per_row / a.xcd_bc;
+    const int r = (xcd / blocks_per_row) * a.xcd_br + j / a.xcd_bc, c = (xcd % blocks_per_row) * a.xcd_bc + j % a.xcd_bc;
+    wg = r * a.wg_per_row + c;
+  }
+  walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units, wg, (int)gridDim.x);
 }
 
 template <int WM, int NTMAX, bool TA, bool TB>
@@ -79,6 +94,15 @@ static int launch_cfg(DeviceCtx* ctx, GemmArgs& a, int batch, int mode) {
   long long slots = (long long)ctx->cus / (batch > 1 ? (batch > 8 ? 8 : batch) : 1);
   if (slots < 1) slots = 1;
   const int grid = (int)(total < slots ? total : slots);
+  // XCD-local blocks of shares: when the shares tile the output exactly (every share the same run of units inside
+  // one row of tiles) and 8 blocks of 8 tile rows x 4 shares cover it
+  a.xcd_br = a.xcd_bc = a.wg_per_row = 0;
+  if (LNN_GEMM_XCD_BLOCKS && batch == 1 && grid % 8 == 0 && total % grid == 0 && a.n_units % (total / grid) == 0) {
+    const int per_row = (int)(a.n_units / (total / grid));
+    if (per_row % 4 == 0 && m_tiles % 8 == 0 && (per_row / 4) * (m_tiles / 8) == 8 && per_row * m_tiles == grid) {
+      a.xcd_br = 8; a.xcd_bc = 4; a.wg_per_row = per_row;
+    }
+  }
   dim3 g(grid, batch, 1), b(512, 1, 1);
   if (mode == 2)
     hipLaunchKernelGGL((gemm_kernel<WM, NTMAX, TA, TB, 2>), g, b, 0, ctx->stream, a);

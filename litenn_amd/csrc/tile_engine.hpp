@@ -32,6 +32,9 @@
 
 namespace lnn {
 
+#ifndef LNN_CB_MAJOR
+#define LNN_CB_MAJOR 1
+#endif
 #ifndef LNN_REQUEST_FIRST
 #define LNN_REQUEST_FIRST 0
 #endif
@@ -391,6 +394,35 @@ struct ConvFwdB {
   }
 };
 
+// The forward pass's weight operand Wp[o][tap][c], rows of K = KK*C floats, read in the K order of ConvFwdBTap
+// (see there): K step (channel block, tap) sits at row offset tap*C + block*BK.
+template <int R>
+struct ConvFwdATap : DirectKC<R> {
+  int C, KK, c0, tap;
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int row0, int M, int kbeg) {
+    DirectKC<R>::init(r, g.C * g.KK, row0, M, 0);
+    C = g.C; KK = g.KK;
+#if LNN_CB_MAJOR
+    const int t0 = kbeg / BK, cb = t0 / g.KK;
+    tap = t0 - cb * g.KK;
+    c0 = cb * BK;
+#else
+    tap = kbeg / g.C;
+    c0 = kbeg - tap * g.C;
+#endif
+  }
+  __device__ __forceinline__ int issue(int, float* lds, int ld, int off) {
+    const int n = DirectKC<R>::issue(tap * C + c0, lds, ld, off);
+#if LNN_CB_MAJOR
+    if (++tap == KK) { tap = 0; c0 += BK; }
+#else
+    c0 += BK;
+    if (c0 >= C) { c0 = 0; ++tap; }
+#endif
+    return n;
+  }
+};
+
 // Tap-major variants of the two pixel gathers, for channel counts that are a
 // multiple of BK.  K is ordered k = tap*CH + ch (tap = kh*KW + kw), so one K
 // step is BK consecutive channels of a single tap: the pixel part of the
@@ -398,13 +430,17 @@ struct ConvFwdB {
 // channel part is wave-uniform and rides in the scalar offset of the buffer
 // instruction.  No table, no per-element arithmetic.  fetch() must be called
 // with consecutive K steps starting at the kbeg given to init().
+// K order: with LNN_CB_MAJOR the channel block is the outer loop and the taps the inner one (k-step t = block * KK +
+// tap), so that the KK consecutive steps of one block of BK channels re-read the same pixels, shifted, while they
+// are still in the L2 of the XCD; tap-major order (all channels of a tap, then the next tap) revisits a pixel only
+// after the whole channel range, by when a 4 MB L2 shared by 32 workgroups has dropped it.
 template <int R, bool DIR = false>
 struct ConvFwdBTap {
   static constexpr bool KC = false, DIRECT = DIR;
   static constexpr int CC = (R + 63) / 64;
   static constexpr int NLD = KR * CC;
   rsrc_t rs;
-  int IH, IW, IHW, C, D, KW;
+  int IH, IW, IHW, C, D, KW, KH;
   int base[CC], ih0[CC], iw0[CC];
   uint32_t voff[CC];   // per-pixel byte offset for the current tap, or OOB
   int c0, kh, kw;   // K position of the next fetch
@@ -419,9 +455,14 @@ struct ConvFwdBTap {
   }
   __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int p0, int P, int kbeg) {
     rs = r;
-    IH = g.IH; IW = g.IW; IHW = g.IHW; C = g.C; D = g.D; KW = g.KW;
+    IH = g.IH; IW = g.IW; IHW = g.IHW; C = g.C; D = g.D; KW = g.KW; KH = g.KH;
+#if LNN_CB_MAJOR
+    const int t0 = kbeg / BK, cb = t0 / g.KK, tap = t0 - cb * g.KK;
+    c0 = cb * BK;
+#else
     const int tap = kbeg / g.C;
     c0 = kbeg - tap * g.C;
+#endif
     kh = tap / g.KW;
     kw = tap - kh * g.KW;
     const int lane = threadIdx.x & 63;
@@ -449,6 +490,15 @@ struct ConvFwdBTap {
     advance();
   }
   __device__ __forceinline__ void advance() {
+#if LNN_CB_MAJOR
+    ++kw;                                   // next tap of the same channel block ...
+    if (kw == KW) {
+      kw = 0;
+      ++kh;
+      if (kh == KH) { kh = 0; c0 += BK; }   // ... then the next block, from the first tap
+    }
+    set_tap();
+#else
     c0 += BK;
     if (c0 >= C) {   // wave-uniform: next tap
       c0 = 0;
@@ -456,6 +506,7 @@ struct ConvFwdBTap {
       if (kw == KW) { kw = 0; ++kh; }
       set_tap();
     }
+#endif
   }
   // straight into the LDS stage: element (k = wave + 4e, column lane + 64c)
   __device__ __forceinline__ int issue(int, float* lds, int ld, int off) {
@@ -480,14 +531,16 @@ struct ConvFwdBTap {
   }
 };
 
-template <int R, bool DIR = false>
+// OBM: K order with the block of BK output channels as the outer loop and the class's taps as the inner one (the
+// counterpart of LNN_CB_MAJOR in ConvFwdBTap, for the same reason); otherwise tap-major.
+template <int R, bool DIR = false, bool OBM = false>
 struct ConvDgradBTap {
   static constexpr bool KC = false, DIRECT = DIR;
   static constexpr int CC = (R + 63) / 64;
   static constexpr int NLD = KR * CC;
   rsrc_t rs;
   ktab_t tab;           // one entry per tap of the pixel class: y, z (see ConvDgradB)
-  int OH, OW, OHW, O;
+  int OH, OW, OHW, O, nt;
   int base[CC], a0[CC], b0[CC];
   uint32_t voff[CC];
   int o0, tap;          // K position of the next fetch
@@ -501,14 +554,23 @@ struct ConvDgradBTap {
     }
   }
   float v[KR][CC];
-  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P, int kbeg) {
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P, int kbeg, int nt_ = 0) {
     rs = r;
     tab = as_ktab(tab_);
-    OH = g.OH; OW = g.OW; OHW = g.OHW; O = g.O;
-    tap = kbeg / g.O;
-    o0 = kbeg - tap * g.O;
-    cy = (tab + tap)->y; cz = (tab + tap)->z;
-    ny = (tab + tap + 1)->y; nz = (tab + tap + 1)->z;
+    OH = g.OH; OW = g.OW; OHW = g.OHW; O = g.O; nt = nt_;
+    if (OBM) {
+      const int t0 = kbeg / BK, ob = nt > 0 ? t0 / nt : 0;
+      tap = t0 - ob * nt;
+      o0 = ob * BK;
+      const int nx = tap + 1 == nt ? 0 : tap + 1;
+      cy = (tab + tap)->y; cz = (tab + tap)->z;
+      ny = (tab + nx)->y; nz = (tab + nx)->z;
+    } else {
+      tap = kbeg / g.O;
+      o0 = kbeg - tap * g.O;
+      cy = (tab + tap)->y; cz = (tab + tap)->z;
+      ny = (tab + tap + 1)->y; nz = (tab + tap + 1)->z;
+    }
     const int lane = threadIdx.x & 63;
 #pragma unroll
     for (int c = 0; c < CC; ++c) {
@@ -534,13 +596,21 @@ struct ConvDgradBTap {
     advance();
   }
   __device__ __forceinline__ void advance() {
-    o0 += BK;
-    if (o0 >= O) {   // wave-uniform: next tap
-      o0 = 0;
-      ++tap;
+    if (OBM) {
+      if (++tap == nt) { tap = 0; o0 += BK; }
       cy = ny; cz = nz;
       set_tap();
-      ny = (tab + tap + 1)->y; nz = (tab + tap + 1)->z;
+      const int nx = tap + 1 == nt ? 0 : tap + 1;
+      ny = (tab + nx)->y; nz = (tab + nx)->z;
+    } else {
+      o0 += BK;
+      if (o0 >= O) {   // wave-uniform: next tap
+        o0 = 0;
+        ++tap;
+        cy = ny; cz = nz;
+        set_tap();
+        ny = (tab + tap + 1)->y; nz = (tab + tap + 1)->z;
+      }
     }
   }
   // straight into the LDS stage: element (k = wave + 4e, column lane + 64c)
@@ -583,16 +653,25 @@ struct ConvDgradATapMC {
   rsrc_t rs;
   ktab_t tab;           // one entry per tap of the pixel class: .w = kh*KW + kw
   uint32_t voff[E];
-  int ld, O, C;
+  int ld, O, C, nt;
   int o0, tap, cw, nw;  // K position of the next transfer; tap index of the current tap and of the one after it
-  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int row0, int kbeg) {
+  // nt_: taps of the pixel class.  K order as in ConvDgradBTap<R, DIR, true>: output-channel block outer, taps inner.
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int row0, int kbeg, int nt_) {
     rs = r;
     tab = as_ktab(tab_);
-    ld = g.KK * g.C; O = g.O; C = g.C;
+    ld = g.KK * g.C; O = g.O; C = g.C; nt = nt_;
+#if LNN_CB_MAJOR
+    const int t0 = kbeg / BK, ob = nt > 0 ? t0 / nt : 0;
+    tap = t0 - ob * nt;
+    o0 = ob * BK;
+    cw = (tab + tap)->w;
+    nw = (tab + (tap + 1 == nt ? 0 : tap + 1))->w;
+#else
     tap = kbeg / g.O;
     o0 = kbeg - tap * g.O;
     cw = (tab + tap)->w;
     nw = (tab + tap + 1)->w;
+#endif
     const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -609,6 +688,11 @@ struct ConvDgradATapMC {
       const int q = wave + 4 * e;
       if (NI % 4 == 0 || q < NI) { buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff); ++n; }
     }
+#if LNN_CB_MAJOR
+    if (++tap == nt) { tap = 0; o0 += BK; }
+    cw = nw;
+    nw = (tab + (tap + 1 == nt ? 0 : tap + 1))->w;
+#else
     o0 += BK;
     if (o0 >= O) {   // wave-uniform: next tap of the class
       o0 = 0;
@@ -616,6 +700,7 @@ struct ConvDgradATapMC {
       cw = nw;
       nw = (tab + tap + 1)->w;
     }
+#endif
     return n;
   }
 };
