@@ -60,6 +60,9 @@ struct ConvArgs {
   // dgrad: g describes one pixel class (g.IH, g.IW = class grid); the plane it is cut from:
   int full_IW, full_IHW, cls_org, cls_s;
   int w_iohw;        // wgrad: dW is stored [C][O][KH][KW]
+  // tap-major wgrad: the columns of an M tile form segs_per_mt segments of seg_units units; a group's columns stay
+  // inside one segment (one tap, for the loaders that assume it; the whole row for the one that does not)
+  int seg_units, segs_per_mt;
 };
 
 // One class of input pixels of a strided dgrad: pixels (h0 + S*i, w0 + S*j),
@@ -196,11 +199,12 @@ __global__ __launch_bounds__(256) void reduce_partials_batch(ReduceBatch b) {
 
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
 // PASS_WGRAD_TAP4: PASS_WGRAD_TAP with 128-bit transfers of the pixel gather too (stride 1, OW % 4 == 0, no padded columns)
-// PASS_WGRAD_ANYC: wgrad for any channel count with transfers straight into LDS, columns in (c, kh, kw) order
+// PASS_WGRAD_ANYC: wgrad for any channel count with transfers straight into LDS; a group's columns may span taps
 // PASS_DGRAD_TAPW: tap-major dgrad that reads the weights in the forward pass's permuted layout (C % 4 == 0)
 enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5, PASS_WGRAD_TAP4 = 6,
        PASS_DGRAD_TAPW = 7, PASS_WGRAD_ANYC = 8 };
-constexpr bool wgrad_tap(int pass) { return pass == PASS_WGRAD_TAP || pass == PASS_WGRAD_TAP4; }
+// the weight-gradient passes whose GEMM columns are tap-major (column tap*C + c)
+constexpr bool wgrad_tap(int pass) { return pass == PASS_WGRAD_TAP || pass == PASS_WGRAD_TAP4 || pass == PASS_WGRAD_ANYC; }
 constexpr bool dgrad_tap(int pass) { return pass == PASS_DGRAD_TAP || pass == PASS_DGRAD_TAPW; }
 
 // Wp[a][tap][b] = W[..] so that the tap-major K index tap*CH + ch is contiguous:
@@ -239,12 +243,12 @@ template <int PASS, int WM, int NTMAX, bool FLAG>
 struct ConvCfg {
   static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
   // the tap-major passes send both operands straight into unpadded LDS tiles, three stages deep
-  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || dgrad_tap(PASS) || wgrad_tap(PASS) || PASS == PASS_WGRAD_ANYC;
+  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || dgrad_tap(PASS) || wgrad_tap(PASS);
   // A side is K-contiguous in LDS for all passes.
   static constexpr int SA = DIRECT ? BM * BK : LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
   static constexpr int SB = DIRECT ? BNMAX * BK : LdsSize<PASS == PASS_WGRAD, BNMAX>::value;
-  static constexpr int STAGES = !DIRECT ? 2 : (wgrad_tap(PASS) || PASS == PASS_WGRAD_ANYC ? LNN_STAGES_WGRAD : LNN_STAGES_FD);
+  static constexpr int STAGES = !DIRECT ? 2 : (wgrad_tap(PASS) ? LNN_STAGES_WGRAD : LNN_STAGES_FD);
 };
 
 // Loader selection and initialisation per pass.  FLAG:
@@ -405,7 +409,7 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
   p.post = a.post;
   if (a.ksplit > 1) { p.post.bias = nullptr; p.post.act = 0; }   // applied by the slice reduction
   if (wgrad_tap(PASS))
-    walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.g.KK, a.total_units,
+    walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.seg_units, a.segs_per_mt, a.total_units,
                               a.chunk_units, chunk_i);
   else
     walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units,
@@ -542,7 +546,7 @@ static ReduceArgs reduce_args(const ConvArgs& a, int final_beta) {
   r.per_mt = 0; r.last_unit0 = 0x7fffffff;
   if (wgrad_tap(PASS)) {
     r.slices_last = a.ks_last;
-    r.per_mt = a.g.KK * a.n_units;
+    r.per_mt = a.seg_units * a.segs_per_mt;
     r.last_unit0 = (a.n_chunks - 1) * a.chunk_units;
   }
   r.dN = make_fastdiv((uint32_t)a.Ncols);
@@ -603,18 +607,26 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   float* final_out = a.Out;
   const int final_beta = a.beta;
   int grid_y = 1;
-  if (PASS == PASS_WGRAD || PASS == PASS_WGRAD_ANYC || wgrad_tap(PASS)) {
+  if (PASS == PASS_WGRAD || wgrad_tap(PASS)) {
     const int m_tiles = (a.M + BM - 1) / BM;
     a.n_units = (a.Ncols + 32 * WN - 1) / (32 * WN);
     long long total = (long long)m_tiles * a.n_units;
     a.chunk_units = 0;
     if (wgrad_tap(PASS)) {
-      // columns are tap-major: KK segments of C / (32*WN) units per M tile; a workgroup
-      // takes one sub-tile's worth of whole segments (or of one segment's halves)
-      a.n_units = a.g.C / (32 * WN);
-      const int per_group = a.n_units < NTMAX ? a.n_units : NTMAX;
-      a.chunk_units = 2 * per_group;
-      total = (long long)m_tiles * a.g.KK * a.n_units;
+      // columns are tap-major.  The loaders that keep one tap per group see KK segments of C / (32*WN) units per M
+      // tile, and a workgroup takes one sub-tile's worth of whole segments (or of one segment's halves); for the
+      // loader whose columns may span taps the whole row is one segment and every sub-tile is full.
+      if (PASS == PASS_WGRAD_ANYC) {
+        a.seg_units = a.n_units;
+        a.segs_per_mt = 1;
+        a.chunk_units = a.seg_units < 2 * NTMAX ? a.seg_units : 2 * NTMAX;
+      } else {
+        a.seg_units = a.g.C / (32 * WN);
+        a.segs_per_mt = a.g.KK;
+        a.chunk_units = 2 * (a.seg_units < NTMAX ? a.seg_units : NTMAX);
+      }
+      a.n_units = a.seg_units;
+      total = (long long)m_tiles * a.segs_per_mt * a.seg_units;
       a.dC = make_fastdiv((uint32_t)a.g.C);
     }
     if (total > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
@@ -798,11 +810,15 @@ static int launch_by_m(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   return launch_pass<PASS, 1, 1>(ctx, a, flag);
 }
 
-// The weight gradient runs on the pixel-major loaders (tap-major columns) when the channels fill whole units of
-// the tile shape chosen for O and a K step of pixels never wraps around an image more than once.
-static bool wgrad_is_pixel_major(const ConvGeom& g) {
+// The weight gradient's pixel walkers move a lane's pixel by one K step with single wrap tests: an image must hold a
+// K step of pixels, and a K step must not wrap around an image more than once.  (Tiny images outside this take the
+// table-driven kernel.)
+static bool wgrad_walkers_fit(const ConvGeom& g) { return g.OHW >= BK && BK / g.OW + 1 <= g.OH; }
+// ... and the loaders that keep one tap per group want the channels to fill whole units of the tile shape chosen for
+// O, enough of them for full sub-tiles (fewer channels: the loader whose columns span taps).
+static bool wgrad_one_tap_per_group(const ConvGeom& g) {
   const int unit = g.O > 64 ? 32 : (g.O > 32 ? 64 : 128);
-  return g.C % unit == 0 && BK / g.OW + 1 <= g.OH;
+  return wgrad_walkers_fit(g) && g.C % unit == 0;
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }

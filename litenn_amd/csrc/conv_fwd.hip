@@ -12,7 +12,7 @@ int conv_weights_plan(const lnn_conv2d_desc* d, int pass, int* yes) {
   if (!yes) return set_error(LNN_ERR_INVALID, "conv2d_weights_plan: null result pointer");
   if (pass == LNN_PASS_FWD) *yes = g.C % BK == 0;
   else if (pass == LNN_PASS_DGRAD) *yes = g.O % BK == 0 && g.C % 4 == 0 && g.C > 4;
-  else if (pass == LNN_PASS_WGRAD) *yes = wgrad_is_pixel_major(g);
+  else if (pass == LNN_PASS_WGRAD) *yes = wgrad_walkers_fit(g);
   else return set_error(LNN_ERR_INVALID, "conv2d_weights_plan: unknown pass");
   return LNN_OK;
 }

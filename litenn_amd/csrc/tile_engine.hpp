@@ -1227,7 +1227,8 @@ struct ConvWgradTapB4Direct {
   }
 };
 
-// wgrad pixel gather for any channel count, GEMM columns in the weights' own order q = (c, kh, kw), sent straight
+// wgrad pixel gather for any channel count, GEMM columns tap-major (q = tap*C + c) like the other pixel-major
+// loaders but free to span taps inside a group, sent straight
 // into a swizzled K-contiguous LDS tile like ConvWgradTapBDirect: a lane owns one fixed pixel position of the K
 // step (carried forward by additions and single wrap tests) and, per transfer, one column - lanes 0..31 the even
 // row of the pair, lanes 32..63 the odd one - whose three constants (element offset from the window's origin, row
@@ -1258,7 +1259,7 @@ struct ConvWgradBAnyC {
       const int q = col0 + 8 * e + 2 * gwave() + half;
       const bool ok = q < Q;
       const int qq = ok ? q : 0;
-      const int ch = qq / g.KK, tap = qq - ch * g.KK, kh = tap / g.KW, kw = tap - kh * g.KW;
+      const int tap = qq / g.C, ch = qq - tap * g.C, kh = tap / g.KW, kw = tap - kh * g.KW;
       yy[e] = ok ? kh * g.D : BIG;
       zz[e] = kw * g.D;
       coff[e] = ch * g.IHW + kh * g.D * g.IW + kw * g.D;

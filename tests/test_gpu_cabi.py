@@ -408,7 +408,10 @@ def test_conv_passes_on_weights_with_swapped_channel_axes(hip):
     rs = np.random.RandomState(62)
     cases = [((2, 64, 12, 12), (64, 64, 5, 5), 2, 1, 2), ((3, 128, 9, 10), (32, 128, 3, 3), 1, 1, 'same'),
              ((2, 128, 8, 8), (160, 128, 3, 3), 1, 2, 'same'), ((1, 32, 20, 20), (96, 32, 1, 1), 1, 1, 'valid'),
-             ((16, 128, 32, 32), (256, 128, 5, 5), 2, 1, 2), ((2, 64, 6, 33), (40, 64, 2, 2), 1, 1, 'valid')]
+             ((16, 128, 32, 32), (256, 128, 5, 5), 2, 1, 2), ((2, 64, 6, 33), (40, 64, 2, 2), 1, 1, 'valid'),
+             # few or odd channel counts: the weight-gradient kernel whose column groups span taps
+             ((4, 32, 20, 20), (8, 32, 3, 3), 1, 1, 'same'), ((2, 96, 14, 16), (40, 96, 3, 3), 2, 1, 1),
+             ((3, 32, 9, 14), (130, 32, 5, 5), 1, 1, 2)]
     for xs, ws, s, d, padding in cases:
         say(f'swapped-axes weights x={xs} w={ws} s={s} d={d} pad={padding}')
         desc, ci = _desc(hip, xs, ws, s, d, padding)
@@ -434,8 +437,8 @@ def test_conv_passes_on_weights_with_swapped_channel_axes(hip):
             dWio = DevArr(hip, shape=w_io.shape, fill=fill)
             hip.conv2d_wgrad_iohw(0, desc, X.ptr, dY.ptr, dWio.ptr, beta)
             assert np.array_equal(dWio.get() - (-3.0 if beta else 0.0), rdw.transpose(1, 0, 2, 3)), (xs, ws, beta)
-    # a geometry on the table-driven weight-gradient kernel cannot write swapped axes
-    desc, _ = _desc(hip, (1, 3, 8, 8), (8, 3, 3, 3), 1, 1, 'same')
+    # output planes smaller than a K step stay on the table-driven weight-gradient kernel, which cannot write swapped axes
+    desc, _ = _desc(hip, (1, 3, 4, 4), (8, 3, 3, 3), 1, 1, 'same')
     assert not hip.conv2d_weights_plan(desc, hip.PASS_WGRAD)
     A = DevArr(hip, shape=(4096,), fill=0.0)
     with pytest.raises(hip.HipException) as e:
