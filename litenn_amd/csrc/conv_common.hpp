@@ -30,6 +30,9 @@
 #ifndef LNN_SMALL_DGRAD
 #define LNN_SMALL_DGRAD 1
 #endif
+#ifndef LNN_FWD_ANYC
+#define LNN_FWD_ANYC 1
+#endif
 #ifndef LNN_WGRAD_ANYC
 #define LNN_WGRAD_ANYC 1
 #endif
@@ -199,10 +202,11 @@ __global__ __launch_bounds__(256) void reduce_partials_batch(ReduceBatch b) {
 
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
 // PASS_WGRAD_TAP4: PASS_WGRAD_TAP with 128-bit transfers of the pixel gather too (stride 1, OW % 4 == 0, no padded columns)
+// PASS_FWD_ANYC: PASS_FWD (any channel count, gather table) with both operands straight into LDS, three stages
 // PASS_WGRAD_ANYC: wgrad for any channel count with transfers straight into LDS; a group's columns may span taps
 // PASS_DGRAD_TAPW: tap-major dgrad that reads the weights in the forward pass's permuted layout (C % 4 == 0)
 enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5, PASS_WGRAD_TAP4 = 6,
-       PASS_DGRAD_TAPW = 7, PASS_WGRAD_ANYC = 8 };
+       PASS_DGRAD_TAPW = 7, PASS_WGRAD_ANYC = 8, PASS_FWD_ANYC = 9 };
 // the weight-gradient passes whose GEMM columns are tap-major (column tap*C + c)
 constexpr bool wgrad_tap(int pass) { return pass == PASS_WGRAD_TAP || pass == PASS_WGRAD_TAP4 || pass == PASS_WGRAD_ANYC; }
 constexpr bool dgrad_tap(int pass) { return pass == PASS_DGRAD_TAP || pass == PASS_DGRAD_TAPW; }
@@ -243,12 +247,12 @@ template <int PASS, int WM, int NTMAX, bool FLAG>
 struct ConvCfg {
   static constexpr int WN = 4 / WM, BM = 32 * WM, BNMAX = 32 * WN * 2 * NTMAX;
   // the tap-major passes send both operands straight into unpadded LDS tiles, three stages deep
-  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || dgrad_tap(PASS) || wgrad_tap(PASS);
+  static constexpr bool DIRECT = PASS == PASS_FWD_TAP || PASS == PASS_FWD_ANYC || dgrad_tap(PASS) || wgrad_tap(PASS);
   // A side is K-contiguous in LDS for all passes.
   static constexpr int SA = DIRECT ? BM * BK : LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
   static constexpr int SB = DIRECT ? BNMAX * BK : LdsSize<PASS == PASS_WGRAD, BNMAX>::value;
-  static constexpr int STAGES = !DIRECT ? 2 : (wgrad_tap(PASS) ? LNN_STAGES_WGRAD : LNN_STAGES_FD);
+  static constexpr int STAGES = !DIRECT ? 2 : (wgrad_tap(PASS) ? LNN_STAGES_WGRAD : (PASS == PASS_FWD_ANYC ? 3 : LNN_STAGES_FD));
 };
 
 // Loader selection and initialisation per pass.  FLAG:
@@ -271,6 +275,17 @@ struct ConvProblem<PASS_FWD, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = PlainKC<R, FLAG>;
   template <int R> using LB = ConvFwdB<R>;
+  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
+  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
+};
+template <bool FLAG, int ST>
+struct ConvProblem<PASS_FWD_ANYC, FLAG, ST> : ConvProblemBase {
+  static constexpr int STAGES = ST;
+  // few channels mean few K steps per sub-tile (a 7x7 stem on RGB: 5), each short: the transfers need the extra
+  // step in flight
+  static constexpr bool REQUEST_FIRST = true;
+  template <int R> using LA = DirectKC4<R>;
+  template <int R> using LB = ConvFwdBDirect<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
@@ -353,7 +368,7 @@ __host__ __device__ inline OutMap plain_map(int ncols) {
 template <int PASS>
 __host__ __device__ inline OutMap final_map(const ConvArgs& a) {
   OutMap om = plain_map(a.Ncols);
-  if (PASS == PASS_FWD || PASS == PASS_FWD_TAP) {
+  if (PASS == PASS_FWD || PASS == PASS_FWD_TAP || PASS == PASS_FWD_ANYC) {
     om.nchw = 1; om.ld = a.g.OHW; om.mtot = a.g.O; om.dHW = a.g.dOHW;
   } else if (PASS == PASS_DGRAD || dgrad_tap(PASS)) {
     om.nchw = 3; om.ld = a.full_IHW; om.mtot = a.g.C; om.dHW = a.g.dIHW;

@@ -67,6 +67,7 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   }
   st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);
   if (st != LNN_OK) return st;
+  if (LNN_FWD_ANYC) return launch_by_m<PASS_FWD_ANYC>(ctx, a, true);
   return launch_by_m<PASS_FWD>(ctx, a, a.K % 4 == 0 && aligned16(W));
 }
 

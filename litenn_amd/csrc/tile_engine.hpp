@@ -423,6 +423,100 @@ struct ConvFwdATap : DirectKC<R> {
   }
 };
 
+// Plain strided matrix, K-contiguous, any K and any alignment, straight into a swizzled LDS tile with 4-byte
+// transfers (the layout of DirectKC, filled like ConvWgradTapADirect fills it: one transfer = two adjacent tile rows,
+// lanes 0..31 the even one, and a lane's swizzled position is one fixed k of the K step).  K positions past the end
+// of a row arrive as zeros.
+__device__ __forceinline__ int direct_k4() {   // k (0..BK-1) whose swizzled position this lane fills
+  const int lane = threadIdx.x & 63, pos = lane & 31, key = 2 * gwave() + (lane >> 5);
+  return (((pos >> 2) ^ key) << 2) | (pos & 3);
+}
+template <int R>
+struct DirectKC4 {
+  static constexpr bool KC = true, DIRECT = true;
+  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int E = R / 8, NLD = E;
+  static_assert(R % 8 == 0, "whole row pairs for all four wavefronts");
+  rsrc_t rs;
+  uint32_t roff[E];   // byte offset of (this lane's row of transfer e, this lane's k), or OOB for a row past the end
+  int kk, K;
+  __device__ __forceinline__ void init(rsrc_t r, int ld, int row0, int M, int K_) {
+    rs = r;
+    K = K_;
+    kk = direct_k4();
+    const int half = (int)((threadIdx.x & 63) >> 5);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int row = row0 + 8 * e + 2 * gwave() + half;
+      roff[e] = row < M ? (uint32_t)(row * ld + kk) * 4u : OOB;
+    }
+  }
+  __device__ __forceinline__ int issue(int k0, float* lds, int, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+    const bool kok = k0 + kk < K;
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, kok ? roff[e] : OOB, (uint32_t)k0 * 4u);
+    return E;
+  }
+};
+
+// ConvFwdB with the gathered elements sent straight into the LDS stage (element (k = wave + 4e, column lane + 64c)
+// of the row-contiguous tile), no staging registers and no LDS writes.
+template <int R>
+struct ConvFwdBDirect {
+  static constexpr bool KC = false, DIRECT = true;
+  static constexpr int CC = (R + 63) / 64;
+  static constexpr int NLD = KR * CC;
+  rsrc_t rs;
+  ktab_t tab;
+  int IH, IW;
+  int base[CC], ih0[CC], iw0[CC];
+  int tx[KR], ty[KR], tz[KR];   // table entries of the next K step (scalar registers)
+  __device__ __forceinline__ void load_entries(int k0) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
+#pragma unroll
+    for (int e = 0; e < KR; ++e) {
+      const ktab_t t = tab + (k0 + wave + 4 * e);
+      tx[e] = t->x; ty[e] = t->y; tz[e] = t->z;
+    }
+  }
+  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P, int kbeg) {
+    rs = r;
+    tab = as_ktab(tab_);
+    load_entries(kbeg);
+    IH = g.IH;
+    IW = g.IW;
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int c = 0; c < CC; ++c) {
+      const int col = lane + 64 * c, p = p0 + col;
+      const bool ok = col < R && p < P;
+      const uint32_t pp = ok ? (uint32_t)p : 0u;
+      const uint32_t img = g.dOHW.div(pp), rem = pp - img * g.OHW;
+      const uint32_t oh = g.dOW.div(rem), ow = rem - oh * g.OW;
+      ih0[c] = (int)oh * g.S - g.PADT;
+      iw0[c] = ok ? (int)ow * g.S - g.PADL : -BIG;
+      base[c] = ((int)img * g.C * g.IH + ih0[c]) * g.IW + ((int)ow * g.S - g.PADL);
+    }
+  }
+  // must be called with consecutive K steps starting at the kbeg given to init()
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) {
+    const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
+#pragma unroll
+    for (int e = 0; e < KR; ++e) {
+#pragma unroll
+      for (int c = 0; c < CC; ++c) {
+        const bool ok = (uint32_t)(ih0[c] + ty[e]) < (uint32_t)IH && (uint32_t)(iw0[c] + tz[e]) < (uint32_t)IW;
+        if (R % 64 == 0 || lane + 64 * c < R)
+          buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, ok ? (uint32_t)(base[c] + tx[e]) * 4u : OOB, 0);
+      }
+    }
+    load_entries(k0 + BK);
+    return NLD;
+  }
+};
+
 // Tap-major variants of the two pixel gathers, for channel counts that are a
 // multiple of BK.  K is ordered k = tap*CH + ch (tap = kh*KW + kw), so one K
 // step is BK consecutive channels of a single tap: the pixel part of the
@@ -1481,6 +1575,14 @@ __device__ __forceinline__ void wait_transfers_but(int n) {
 #undef LNN_W
 }
 
+// A problem whose transfers come a long way relative to its K steps (short steps, operands not resident in L2)
+// declares `static constexpr bool REQUEST_FIRST = true`: its three-stage pipeline then sends K step t+2 off before it
+// waits for step t+1.
+template <class T, class = void>
+struct request_first : std::false_type {};
+template <class T>
+struct request_first<T, std::void_t<decltype(T::REQUEST_FIRST)>> : std::integral_constant<bool, T::REQUEST_FIRST> {};
+
 template <class LB, class LA>
 __device__ __forceinline__ int issue_b(LB& lb, int k0, float* lds, int ld, int off, LA& la) {
   if constexpr (needs_a<LB>::value)
@@ -1581,7 +1683,7 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
       for (int phase = 0; phase < 2; ++phase) {
         if (phase == G) {
           compute(cur);
-        } else if constexpr (DA && DB && LNN_REQUEST_FIRST) {
+        } else if constexpr (DA && DB && (LNN_REQUEST_FIRST || request_first<P>::value)) {
           // K step t+2 goes out first (into the stage last read for step t-1), then the wait for step t+1, which
           // has been in flight for a whole step, leaves those newest transfers outstanding: every transfer gets
           // close to two steps to land, which short steps (narrow tiles) need
