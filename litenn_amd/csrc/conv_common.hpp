@@ -18,7 +18,7 @@
 #define LNN_STAGES_WGRAD 3
 #endif
 #ifndef LNN_STAGES_FD
-#define LNN_STAGES_FD 2
+#define LNN_STAGES_FD 3
 #endif
 // B-side gathers: 1 = straight into LDS, 0 = through registers (needs three stages)
 #ifndef LNN_FD_B_DIRECT

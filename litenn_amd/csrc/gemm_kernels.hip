@@ -9,7 +9,7 @@
 #define LNN_GEMM_XCD_BLOCKS 1
 #endif
 #ifndef LNN_STAGES_GEMM
-#define LNN_STAGES_GEMM 2
+#define LNN_STAGES_GEMM 3
 #endif
 
 namespace lnn {

@@ -35,6 +35,10 @@ namespace lnn {
 #ifndef LNN_CB_MAJOR
 #define LNN_CB_MAJOR 1
 #endif
+// Three-stage pipelines of two direct loaders run without phases: one barrier per K step, inside the MFMA stream.
+#ifndef LNN_STREAM
+#define LNN_STREAM 1
+#endif
 #ifndef LNN_REQUEST_FIRST
 #define LNN_REQUEST_FIRST 0
 #endif
@@ -202,11 +206,15 @@ struct DirectKC {
     }
   }
   // off: first tile row of this group.  Returns the number of transfers this wavefront issued.
-  __device__ __forceinline__ int issue(int k0, float* lds, int, int off) {
+  // issue_part<PART, NPARTS> sends the PART-th of NPARTS shares of a K step's transfers (all loaders: the shares of
+  // one K step are asked for in order, and the loader moves on to the next K step with the last one).
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int k0, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     int n = 0;
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
+    for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e) {
       const int blk = wave + 4 * e;
       if (NB % 4 == 0 || blk < NB) { buf_load_lds16(rs, lds + (off + blk * 8) * BK, voff[e], (uint32_t)k0 * 4u); ++n; }
     }
@@ -238,12 +246,14 @@ struct DirectMC {
       voff[e] = (k < BK && row0 + n < M) ? (uint32_t)(k * ld + row0 + n) * 4u : OOB;
     }
   }
-  __device__ __forceinline__ int issue(int k0, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld_, int off) { return issue_part<0, 1>(k0, lds, ld_, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int k0, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const uint32_t soff = (uint32_t)(k0 * ld) * 4u;
     int n = 0;
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
+    for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e) {
       const int q = wave + 4 * e;
       if (NI % 4 == 0 || q < NI) { buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff); ++n; }
     }
@@ -411,14 +421,18 @@ struct ConvFwdATap : DirectKC<R> {
     c0 = kbeg - tap * g.C;
 #endif
   }
-  __device__ __forceinline__ int issue(int, float* lds, int ld, int off) {
-    const int n = DirectKC<R>::issue(tap * C + c0, lds, ld, off);
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int, float* lds, int ld, int off) {
+    const int n = DirectKC<R>::template issue_part<PART, NPARTS>(tap * C + c0, lds, ld, off);
+    if (PART == NPARTS - 1) {
 #if LNN_CB_MAJOR
-    if (++tap == KK) { tap = 0; c0 += BK; }
+      if (++tap == KK) { tap = 0; c0 += BK; }
 #else
-    c0 += BK;
-    if (c0 >= C) { c0 = 0; ++tap; }
+      c0 += BK;
+      if (c0 >= C) { c0 = 0; ++tap; }
 #endif
+    }
     return n;
   }
 };
@@ -451,13 +465,15 @@ struct DirectKC4 {
       roff[e] = row < M ? (uint32_t)(row * ld + kk) * 4u : OOB;
     }
   }
-  __device__ __forceinline__ int issue(int k0, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int k0, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const bool kok = k0 + kk < K;
 #pragma unroll
-    for (int e = 0; e < E; ++e)
+    for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e)
       buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, kok ? roff[e] : OOB, (uint32_t)k0 * 4u);
-    return E;
+    return E * (PART + 1) / NPARTS - E * PART / NPARTS;
   }
 };
 
@@ -501,10 +517,12 @@ struct ConvFwdBDirect {
     }
   }
   // must be called with consecutive K steps starting at the kbeg given to init()
-  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int k0, float* lds, int ld, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
 #pragma unroll
-    for (int e = 0; e < KR; ++e) {
+    for (int e = KR * PART / NPARTS; e < KR * (PART + 1) / NPARTS; ++e) {
 #pragma unroll
       for (int c = 0; c < CC; ++c) {
         const bool ok = (uint32_t)(ih0[c] + ty[e]) < (uint32_t)IH && (uint32_t)(iw0[c] + tz[e]) < (uint32_t)IW;
@@ -512,8 +530,8 @@ struct ConvFwdBDirect {
           buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, ok ? (uint32_t)(base[c] + tx[e]) * 4u : OOB, 0);
       }
     }
-    load_entries(k0 + BK);
-    return NLD;
+    if (PART == NPARTS - 1) load_entries(k0 + BK);
+    return (KR * (PART + 1) / NPARTS - KR * PART / NPARTS) * CC;
   }
 };
 
@@ -603,17 +621,19 @@ struct ConvFwdBTap {
 #endif
   }
   // straight into the LDS stage: element (k = wave + 4e, column lane + 64c)
-  __device__ __forceinline__ int issue(int, float* lds, int ld, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int, float* lds, int ld, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
 #pragma unroll
-    for (int e = 0; e < KR; ++e) {
+    for (int e = KR * PART / NPARTS; e < KR * (PART + 1) / NPARTS; ++e) {
       const uint32_t soff = (uint32_t)((c0 + wave + 4 * e) * IHW) * 4u;
 #pragma unroll
       for (int c = 0; c < CC; ++c)
         if (R % 64 == 0 || lane + 64 * c < R) buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);
     }
-    advance();
-    return NLD;
+    if (PART == NPARTS - 1) advance();
+    return (KR * (PART + 1) / NPARTS - KR * PART / NPARTS) * CC;
   }
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
@@ -708,17 +728,19 @@ struct ConvDgradBTap {
     }
   }
   // straight into the LDS stage: element (k = wave + 4e, column lane + 64c)
-  __device__ __forceinline__ int issue(int, float* lds, int ld, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int, float* lds, int ld, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
 #pragma unroll
-    for (int e = 0; e < KR; ++e) {
+    for (int e = KR * PART / NPARTS; e < KR * (PART + 1) / NPARTS; ++e) {
       const uint32_t soff = (uint32_t)((o0 + wave + 4 * e) * OHW) * 4u;
 #pragma unroll
       for (int c = 0; c < CC; ++c)
         if (R % 64 == 0 || lane + 64 * c < R) buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);
     }
-    advance();
-    return NLD;
+    if (PART == NPARTS - 1) advance();
+    return (KR * (PART + 1) / NPARTS - KR * PART / NPARTS) * CC;
   }
   __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
@@ -773,28 +795,32 @@ struct ConvDgradATapMC {
       voff[e] = (k < BK && row0 + n < g.C) ? (uint32_t)(k * ld + row0 + n) * 4u : OOB;
     }
   }
-  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld_, int off) { return issue_part<0, 1>(k0, lds, ld_, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const uint32_t soff = (uint32_t)(o0 * ld + cw * C) * 4u;
     int n = 0;
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
+    for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e) {
       const int q = wave + 4 * e;
       if (NI % 4 == 0 || q < NI) { buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff); ++n; }
     }
+    if (PART == NPARTS - 1) {
 #if LNN_CB_MAJOR
-    if (++tap == nt) { tap = 0; o0 += BK; }
-    cw = nw;
-    nw = (tab + (tap + 1 == nt ? 0 : tap + 1))->w;
-#else
-    o0 += BK;
-    if (o0 >= O) {   // wave-uniform: next tap of the class
-      o0 = 0;
-      ++tap;
+      if (++tap == nt) { tap = 0; o0 += BK; }
       cw = nw;
-      nw = (tab + tap + 1)->w;
-    }
+      nw = (tab + (tap + 1 == nt ? 0 : tap + 1))->w;
+#else
+      o0 += BK;
+      if (o0 >= O) {   // wave-uniform: next tap of the class
+        o0 = 0;
+        ++tap;
+        cw = nw;
+        nw = (tab + tap + 1)->w;
+      }
 #endif
+    }
     return n;
   }
 };
@@ -1152,16 +1178,20 @@ struct ConvWgradTapADirect {
     rem = p - (int)img * g.OHW;
     aoff = (int)img * g.O * g.OHW + rem + (o0 + 2 * gwave() + (int)((threadIdx.x & 63) >> 5)) * g.OHW;
   }
-  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     // rows past the last output channel are never stored, so they need no mask
     const uint32_t voff = p < kend ? (uint32_t)aoff * 4u : OOB;
 #pragma unroll
-    for (int e = 0; e < E; ++e)
+    for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e)
       buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, voff, (uint32_t)(8 * e * OHW) * 4u);
-    p += BK; rem += BK; aoff += BK;
-    if (rem >= OHW) { rem -= OHW; aoff += awrap; }
-    return E;
+    if (PART == NPARTS - 1) {
+      p += BK; rem += BK; aoff += BK;
+      if (rem >= OHW) { rem -= OHW; aoff += awrap; }
+    }
+    return E * (PART + 1) / NPARTS - E * PART / NPARTS;
   }
 };
 
@@ -1188,18 +1218,22 @@ struct ConvWgradTapA4Direct {
     rem = p - (int)img * g.OHW;
     aoff = (int)img * g.O * g.OHW + rem + (o0 + 8 * gwave() + rb) * g.OHW;
   }
-  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const uint32_t voff = p < kend ? (uint32_t)aoff * 4u : OOB;   // kend is a multiple of 4 here: whole groups
     int n = 0;
 #pragma unroll
-    for (int e = 0; e < E; ++e)
+    for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e)
       if (NB % 4 == 0 || wave + 4 * e < NB) {
         buf_load_lds16(rs, lds + (off + (wave + 4 * e) * 8) * BK, voff, (uint32_t)(32 * e * OHW) * 4u);
         ++n;
       }
-    p += BK; rem += BK; aoff += BK;
-    if (rem >= OHW) { rem -= OHW; aoff += awrap; }
+    if (PART == NPARTS - 1) {
+      p += BK; rem += BK; aoff += BK;
+      if (rem >= OHW) { rem -= OHW; aoff += awrap; }
+    }
     return n;
   }
 };
@@ -1241,29 +1275,36 @@ struct ConvWgradTapBDirect {
     iw = ow * g.S + kw * g.D - g.PADL;
     xoff = ((int)img * g.C + c0 + 2 * gwave() + (int)((threadIdx.x & 63) >> 5)) * g.IHW + ih * g.IW + iw;
   }
-  __device__ __forceinline__ int issue(int, float* lds, int, int off) { go<true>(lds, off); return E; }
-  __device__ __forceinline__ void fetch(int) { go<false>(nullptr, 0); }
+  __device__ __forceinline__ int issue(int, float* lds, int, int off) { go<true, 0, 1>(lds, off); return E; }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int, float* lds, int, int off) {
+    go<true, PART, NPARTS>(lds, off);
+    return E * (PART + 1) / NPARTS - E * PART / NPARTS;
+  }
+  __device__ __forceinline__ void fetch(int) { go<false, 0, 1>(nullptr, 0); }
   __device__ __forceinline__ void commit(float* lds, int, int off) const {
     const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < E; ++e) lds[(off + 8 * e + 2 * wave) * BK + lane] = v[e];
   }
-  template <bool TO_LDS>
+  template <bool TO_LDS, int PART, int NPARTS>
   __device__ __forceinline__ void go(float* lds, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const bool ok = p < kend && (uint32_t)ih < (uint32_t)IH && (uint32_t)iw < (uint32_t)IW;
     const uint32_t voff = ok ? (uint32_t)xoff * 4u : OOB;
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
+    for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e) {
       const uint32_t soff = (uint32_t)(8 * e * IHW) * 4u;
       if (TO_LDS)
         buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, voff, soff);
       else
         v[e] = buf_load_s(rs, voff, soff);
     }
-    p += BK; oh += qh; ow += rw; ih += s_q; iw += s_r; xoff += x_step;
-    if (ow >= OW) { ow -= OW; ++oh; iw -= s_OW; ih += S; xoff += xwrap_w; }
-    if (oh >= OH) { oh -= OH; ih -= s_OH; xoff += xwrap_h; }
+    if (PART == NPARTS - 1) {
+      p += BK; oh += qh; ow += rw; ih += s_q; iw += s_r; xoff += x_step;
+      if (ow >= OW) { ow -= OW; ++oh; iw -= s_OW; ih += S; xoff += xwrap_w; }
+      if (oh >= OH) { oh -= OH; ih -= s_OH; xoff += xwrap_h; }
+    }
   }
 };
 
@@ -1304,19 +1345,23 @@ struct ConvWgradTapB4Direct {
     ih = oh + kh * g.D - g.PADT;
     xoff = ((int)img * g.C + c0 + 8 * gwave() + rb) * g.IHW + ih * g.IW + ow + kw * g.D;
   }
-  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const uint32_t voff = p < kend && (uint32_t)ih < (uint32_t)IH ? (uint32_t)xoff * 4u : OOB;
     int n = 0;
 #pragma unroll
-    for (int e = 0; e < E; ++e)
+    for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e)
       if (NB % 4 == 0 || wave + 4 * e < NB) {
         buf_load_lds16(rs, lds + (off + (wave + 4 * e) * 8) * BK, voff, (uint32_t)(32 * e * IHW) * 4u);
         ++n;
       }
-    p += BK; oh += qh; ow += rw; ih += qh; xoff += x_step;
-    if (ow >= OW) { ow -= OW; ++oh; ++ih; xoff += xwrap_w; }
-    if (oh >= OH) { oh -= OH; ih -= OH; xoff += xwrap_h; }
+    if (PART == NPARTS - 1) {
+      p += BK; oh += qh; ow += rw; ih += qh; xoff += x_step;
+      if (ow >= OW) { ow -= OW; ++oh; ++ih; xoff += xwrap_w; }
+      if (oh >= OH) { oh -= OH; ih -= OH; xoff += xwrap_h; }
+    }
     return n;
   }
 };
@@ -1371,18 +1416,22 @@ struct ConvWgradBAnyC {
     iw = ow * g.S - g.PADL;
     xoff = (int)img * g.C * g.IHW + ih * g.IW + iw;
   }
-  __device__ __forceinline__ int issue(int, float* lds, int, int off) {
+  __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ int issue_part(int, float* lds, int, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const int ihm = p < kend ? ih : BIG;
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
+    for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e) {
       const bool ok = (uint32_t)(ihm + yy[e]) < (uint32_t)IH && (uint32_t)(iw + zz[e]) < (uint32_t)IW;
       buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, ok ? (uint32_t)(xoff + coff[e]) * 4u : OOB, 0);
     }
-    p += BK; oh += qh; ow += rw; ih += s_q; iw += s_r; xoff += x_step;
-    if (ow >= OW) { ow -= OW; ++oh; iw -= s_OW; ih += S; xoff += xwrap_w; }
-    if (oh >= OH) { oh -= OH; ih -= s_OH; xoff += xwrap_h; }
-    return E;
+    if (PART == NPARTS - 1) {
+      p += BK; oh += qh; ow += rw; ih += s_q; iw += s_r; xoff += x_step;
+      if (ow >= OW) { ow -= OW; ++oh; iw -= s_OW; ih += S; xoff += xwrap_w; }
+      if (oh >= OH) { oh -= OH; ih -= s_OH; xoff += xwrap_h; }
+    }
+    return E * (PART + 1) / NPARTS - E * PART / NPARTS;
   }
 };
 
@@ -1498,6 +1547,85 @@ __device__ __forceinline__ void mma_stage(const float* __restrict__ As, const fl
       __builtin_amdgcn_sched_group_barrier(0x008, 4 * NT, 0);       // last group
     }
   }
+}
+
+// One LDS stage of a pipeline that never leaves the MFMA stream (BK / 8 = 4 groups of 4*NT MFMAs).  On entry
+// fa[0] / fb[0] hold the fragments of the stage's first group, read by the previous stage (or by the prologue).
+// The global -> LDS transfers that refill the stage read one K step ago go out in four shares, send(share), one per
+// group, slotted between the MFMAs that carry no fragment read.  Late in the last group comes the K step's only
+// barrier, mid(): behind it the next stage is complete in LDS and this one is no longer read by anybody, so the
+// step's last MFMAs carry the reads of the next stage's first group (NEXT) and the next step may refill this stage.
+// Vector-memory and LDS instructions cost the matrix pipe nothing while they sit between the MFMAs of the same
+// wavefront; vector-ALU instructions stop it, and so does anything the other wavefront of the SIMD wants to issue.
+// NV: transfers per wavefront and K step if known (0: unknown or none).
+template <int N> using ic = std::integral_constant<int, N>;
+template <int NT, int LAY_A, int LAY_B, int RA, int RB, int NV, bool NEXT, class MID, class SEND>
+__device__ __forceinline__ void mma_stage_stream(const float* __restrict__ As, const float* __restrict__ Bs,
+                                                 const float* __restrict__ Asn, const float* __restrict__ Bsn,
+                                                 f32x16 (&acc)[NT], float (&fa)[2][4], float (&fb)[2][NT][4], int arow,
+                                                 int brow, MID mid, SEND send) {
+  constexpr int NG = BK / 8;
+  static_assert(NG == 4, "four groups, four shares of transfers; the next stage's first group lands in buffer 0");
+  constexpr int RD = (LAY_A <= LAY_KC_SWZ ? 1 : 2) + (LAY_B <= LAY_KC_SWZ ? NT : 2 * NT);
+  constexpr int G = 4 * NT;                       // MFMAs per group
+  constexpr int PAIRS = RD < G ? RD : G;          // MFMAs of a group that carry a fragment read
+  constexpr int FREE = G - PAIRS;                 // ... and those that do not
+  // transfers slotted into one group (the scheduler takes them in program order, whichever share they belong to)
+  constexpr int SHARE = (NV + NG - 1) / NG;
+  constexpr int PER = FREE > 0 ? (SHARE + FREE - 1) / FREE : SHARE;
+  auto mfmas = [&](auto curc, auto loc, auto hic) {
+    constexpr int cur = decltype(curc)::value, lo = decltype(loc)::value, hi = decltype(hic)::value;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        if (t * NT + j >= lo && t * NT + j < hi)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur][t], fb[cur][j][t], acc[j], 0, 0, 0);
+  };
+  auto read_slots = [&] {
+#pragma unroll
+    for (int i = 0; i < PAIRS; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    if (RD > G) __builtin_amdgcn_sched_group_barrier(0x100, RD - G, 0);
+  };
+  auto transfer_slots = [&] {
+    if (NV > 0) {
+#pragma unroll
+      for (int i = 0; i < FREE; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i * PER < SHARE) __builtin_amdgcn_sched_group_barrier(0x020, PER, 0);   // the last one may stay short
+      }
+      if (FREE == 0) __builtin_amdgcn_sched_group_barrier(0x020, SHARE, 0);
+    } else if (FREE > 0) {
+      __builtin_amdgcn_sched_group_barrier(0x008, FREE, 0);
+    }
+  };
+  auto group = [&](auto kkc) {
+    constexpr int kk = decltype(kkc)::value, cur = kk & 1;
+    if constexpr (kk + 1 < NG) {
+      load_frags<NT, LAY_A, LAY_B, RA, RB>(As, Bs, arow, brow, kk + 1, fa[cur ^ 1], fb[cur ^ 1]);
+      mfmas(ic<cur>(), ic<0>(), ic<G>());
+      send(kkc);
+      read_slots();
+      transfer_slots();
+    } else {
+      mfmas(ic<cur>(), ic<0>(), ic<FREE>());
+      send(kkc);
+      transfer_slots();
+      __builtin_amdgcn_sched_barrier(0);
+      mid();
+      __builtin_amdgcn_sched_barrier(0);
+      if (NEXT) load_frags<NT, LAY_A, LAY_B, RA, RB>(Asn, Bsn, arow, brow, 0, fa[cur ^ 1], fb[cur ^ 1]);
+      mfmas(ic<cur>(), ic<FREE>(), ic<G>());
+      if (NEXT) read_slots(); else __builtin_amdgcn_sched_group_barrier(0x008, PAIRS, 0);
+    }
+  };
+  group(ic<0>());
+  group(ic<1>());
+  group(ic<2>());
+  group(ic<3>());
 }
 
 template <bool KC, int R>
@@ -1662,6 +1790,67 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
           barrier_after_issue();
         }
       }
+    }
+  } else if constexpr (DA && DB && ST == 3 && LNN_STREAM) {
+    // No phases: both groups run the same schedule side by side and share the matrix pipes as they come; whenever
+    // one wavefront of a SIMD waits (for fragments, at the barrier) the other one's MFMAs fill the pipe.  During K
+    // step t every wavefront sends the transfers of step t+2 off, in shares between its MFMAs, into the stage that
+    // step t-1 read.  Per step there is one barrier, late in the step's MFMAs.  Before it every wavefront waits
+    // until only the transfers it sent off in this step are still in flight: its part of step t+1, sent a whole
+    // step earlier, has then landed.  Behind the barrier stage t+1 is therefore complete - the step's last MFMAs
+    // already carry the reads of its first fragments - and stage t, which no wavefront reads any more, is free
+    // for the transfers of step t+3.
+    static_assert(!needs_a<LB>::value, "direct loaders stand alone");
+    constexpr int NVT = (LA::NLD >= 0 && (NT == 0 || LB::NLD >= 0)) ? LA::NLD + (NT > 0 ? LB::NLD : 0) : 0;
+    float fa[2][4], fb[2][NTC][4];
+    int n1 = 0;
+    if (nk > 0) request(kbeg, 0);
+    if (nk > 1) n1 = request(kbeg + BK, 1);
+    if (nk > 0) wait_transfers_but(n1);
+    barrier_after_compute();
+    if constexpr (NT > 0)
+      if (nk > 0) load_frags<NTC, LAY_A, LAY_B, BM, RB>(ldsA, ldsBr, arow, brow, 0, fa[0], fb[0]);
+    auto nothing = [](auto...) {};
+    int cur = 0, t = 0;
+    for (; t + 2 < nk; ++t) {
+      const int nxt = cur + 1 == ST ? 0 : cur + 1, nn = nxt + 1 == ST ? 0 : nxt + 1;
+      const int k0 = kbeg + (t + 2) * BK;
+      int n = 0;   // transfers this wavefront has sent off in this step
+      auto send = [&](auto share) {
+        constexpr int S = decltype(share)::value;
+        n += la.template issue_part<S, 4>(k0, ldsA + nn * strideA, LDA, G * HALF);
+        if constexpr (NT > 0) n += lb.template issue_part<S, 4>(k0, ldsB + nn * strideB, LDB, COFF);
+      };
+      auto mid = [&] {
+        wait_transfers_but(n);
+        asm volatile("s_barrier" ::: "memory");
+      };
+      if constexpr (NT > 0) {
+        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, NVT, true>(ldsA + cur * strideA, ldsBr + cur * strideB,
+                                                              ldsA + nxt * strideA, ldsBr + nxt * strideB, acc, fa, fb,
+                                                              arow, brow, mid, send);
+      } else {
+        send(ic<0>()); send(ic<1>()); send(ic<2>()); send(ic<3>());
+        mid();
+      }
+      cur = nxt;
+    }
+    auto drain = [] { asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory"); };
+    if (t + 1 < nk) {   // last but one step: nothing left to send
+      const int nxt = cur + 1 == ST ? 0 : cur + 1;
+      if constexpr (NT > 0)
+        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, 0, true>(ldsA + cur * strideA, ldsBr + cur * strideB,
+                                                            ldsA + nxt * strideA, ldsBr + nxt * strideB, acc, fa, fb,
+                                                            arow, brow, drain, nothing);
+      else
+        drain();
+      cur = nxt;
+      ++t;
+    }
+    if (t < nk) {       // last step
+      if constexpr (NT > 0)
+        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, 0, false>(ldsA + cur * strideA, ldsBr + cur * strideB, ldsA, ldsBr,
+                                                             acc, fa, fb, arow, brow, nothing, nothing);
     }
   } else {
     // "moving data" in step t = completing K step t+1 (requested in step t-1:
