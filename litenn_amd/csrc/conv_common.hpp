@@ -334,6 +334,7 @@ struct ConvProblem<PASS_WGRAD, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
+  static constexpr bool STREAM_UNROLL = false;   // measured: slower with constant stages (registers)
   template <int R> using LA = typename std::conditional<FLAG, ConvWgradTapA4Direct<R>, ConvWgradTapADirect<R>>::type;
   template <int R> using LB = ConvWgradTapBDirect<R, LNN_WGRAD_B_DIRECT != 0>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }
@@ -343,6 +344,7 @@ struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_ANYC, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
+  static constexpr bool STREAM_UNROLL = false;   // measured: slower with constant stages (registers)
   template <int R> using LA = typename std::conditional<FLAG, ConvWgradTapA4Direct<R>, ConvWgradTapADirect<R>>::type;
   template <int R> using LB = ConvWgradBAnyC<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }
@@ -352,6 +354,7 @@ struct ConvProblem<PASS_WGRAD_ANYC, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_TAP4, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
+  static constexpr bool STREAM_UNROLL = false;   // measured: slower with constant stages (registers)
   template <int R> using LA = ConvWgradTapA4Direct<R>;
   template <int R> using LB = ConvWgradTapB4Direct<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }

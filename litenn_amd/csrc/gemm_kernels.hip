@@ -48,6 +48,7 @@ struct GemmCfg {
 template <bool TA, bool TB, int MODE, int ST>
 struct GemmProblem {
   static constexpr int STAGES = ST;
+  static constexpr bool STREAM_UNROLL = !TB;   // measured: A * B^T is slower with constant stages
   static constexpr bool VEC = MODE >= 1, DIR = MODE == 2;
   template <int R> using KCL = typename std::conditional<DIR, DirectKC<R>, PlainKC<R, VEC>>::type;
   template <int R> using MCL = typename std::conditional<DIR, DirectMC<R>, PlainMC<R, VEC>>::type;

@@ -39,6 +39,9 @@ namespace lnn {
 #ifndef LNN_STREAM
 #define LNN_STREAM 1
 #endif
+#ifndef LNN_STREAM_UNROLL
+#define LNN_STREAM_UNROLL 1
+#endif
 #ifndef LNN_REQUEST_FIRST
 #define LNN_REQUEST_FIRST 0
 #endif
@@ -1711,6 +1714,13 @@ struct request_first : std::false_type {};
 template <class T>
 struct request_first<T, std::void_t<decltype(T::REQUEST_FIRST)>> : std::integral_constant<bool, T::REQUEST_FIRST> {};
 
+// A problem whose streaming loop should keep a running stage index (no threefold unrolling: register pressure or code
+// size cost it more than the address arithmetic) declares `static constexpr bool STREAM_UNROLL = false`.
+template <class T, class = void>
+struct stream_unroll : std::integral_constant<bool, LNN_STREAM_UNROLL != 0> {};
+template <class T>
+struct stream_unroll<T, std::void_t<decltype(T::STREAM_UNROLL)>> : std::integral_constant<bool, T::STREAM_UNROLL && LNN_STREAM_UNROLL> {};
+
 template <class LB, class LA>
 __device__ __forceinline__ int issue_b(LB& lb, int k0, float* lds, int ld, int off, LA& la) {
   if constexpr (needs_a<LB>::value)
@@ -1812,8 +1822,10 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
       if (nk > 0) load_frags<NTC, LAY_A, LAY_B, BM, RB>(ldsA, ldsBr, arow, brow, 0, fa[0], fb[0]);
     auto nothing = [](auto...) {};
     int cur = 0, t = 0;
-    for (; t + 2 < nk; ++t) {
-      const int nxt = cur + 1 == ST ? 0 : cur + 1, nn = nxt + 1 == ST ? 0 : nxt + 1;
+    // one step that sends; the stage index may be a constant (then all LDS addresses of the step are loop invariants
+    // or immediates, where a running index costs some twenty vector-ALU instructions a step)
+    auto step = [&](auto curv) {
+      const int nxt = curv + 1 == ST ? 0 : curv + 1, nn = nxt + 1 == ST ? 0 : nxt + 1;
       const int k0 = kbeg + (t + 2) * BK;
       int n = 0;   // transfers this wavefront has sent off in this step
       auto send = [&](auto share) {
@@ -1826,14 +1838,27 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
         asm volatile("s_barrier" ::: "memory");
       };
       if constexpr (NT > 0) {
-        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, NVT, true>(ldsA + cur * strideA, ldsBr + cur * strideB,
+        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, NVT, true>(ldsA + curv * strideA, ldsBr + curv * strideB,
                                                               ldsA + nxt * strideA, ldsBr + nxt * strideB, acc, fa, fb,
                                                               arow, brow, mid, send);
       } else {
         send(ic<0>()); send(ic<1>()); send(ic<2>()); send(ic<3>());
         mid();
       }
-      cur = nxt;
+      ++t;
+    };
+    if constexpr (stream_unroll<P>::value) {
+      static_assert(ST == 3, "three steps per turn");
+      while (t + 4 < nk) {   // three sending steps with constant stages: 0, 1, 2
+        step(ic<0>());
+        step(ic<1>());
+        step(ic<2>());
+      }
+    }
+    cur = t % ST;
+    while (t + 2 < nk) {
+      step(cur);
+      cur = cur + 1 == ST ? 0 : cur + 1;
     }
     auto drain = [] { asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory"); };
     if (t + 1 < nk) {   // last but one step: nothing left to send
