@@ -10,12 +10,19 @@ namespace {
 // rh = (ih + PADT) % S, rw = (iw + PADW) % S form a class that sees the taps kh = rh, rh + S, ... (NKH of them) and
 // kw = rw, rw + S, ..., spaced one output pixel apart:
 //   dX[n][c][h0 + S*y][w0 + S*x] (+)= sum over o, jh, jw of dY[n][o][y + ah - jh][x + aw - jw] * W[o][c][rh + S*jh][rw + S*jw]
-// A block owns the 32 x 32 pixels (y, x) of ALL S*S classes of one image, i.e. one region of dY, which it brings to
-// LDS once per chunk of kDsOC output channels (row by row with global -> LDS transfers, all in flight together).
-// A thread owns 2 x 2 pixels of every class: per output channel and class it reads its (NKH+1) x (NKW+1) window once;
-// the weights (4 floats per tap, channels past C zero) have the same address in every lane and come through the
-// scalar cache.  4 * NKH * NKW * C multiply-adds per window.
-constexpr int kDsOC = 8, kDsTile = 32;
+// A block owns the 16 x 16 pixels (y, x) of ALL S*S classes of one image, i.e. one region of dY; each of its four
+// wavefronts sums a quarter of the output channels over that region, on its own: it brings its channels' planes of
+// the region to its own part of LDS, kDsOC at a time (global -> LDS transfers of 64 consecutive tile elements, all in
+// flight together), and waits for nobody but itself.  A lane owns 2 x 2 pixels of every class: per output channel
+// and class it reads its (NKH+1) x (NKW+1) window once; the weights (4 floats per tap, channels past C zero) travel
+// to LDS with the planes and are read from there, the same address in every lane (through the scalar cache, whose
+// loads return out of order, every pair of taps waited for its own load: 0.242 against 0.224 ms for a 7 x 7 stride 2
+// stem at batch 32).  4 * NKH * NKW * C multiply-adds per window.
+// At the end wavefronts 1..3 hand their sums over through LDS, one after the other, and wavefront 0 adds them in
+// that order and stores.
+// (A block of 32 x 32 pixels with one wavefront per 8 rows was measured first: a 112 x 112 class plane is 3.5 such
+// tiles wide and tall, and 31 % of the lanes worked on pixels that do not exist.)
+constexpr int kDsOC = 4, kDsTile = 16;
 struct SmallDgradArgs {
   const float* dY;
   const float* wc;        // [O][K*K taps, class by class][4]
@@ -73,7 +80,7 @@ struct SmallDgradClass {
       for (int jh = 0; jh < NKH; ++jh)
 #pragma unroll
         for (int jw = 0; jw < NKW; ++jw) {
-          const f32x4 w4 = *reinterpret_cast<const f32x4*>(wo + (TAP0 + jh * NKW + jw) * 4);
+          const f32x4 w4 = *reinterpret_cast<const f32x4*>(wo + (TAP0 + jh * NKW + jw) * 4);   // LDS, same address in every lane
 #pragma unroll
           for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -108,12 +115,20 @@ struct SmallDgradClass {
 template <int S, int K, int CN>
 __global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
   constexpr int NCLS = S * S, KK = K * K;
-  constexpr int TMAX = kDsTile + (K + S - 1) / S + 1, PITCH = TMAX | 1, PLANE = (TMAX * PITCH + 63) / 64 * 64;
-  __shared__ float tile[kDsOC * PLANE + 64];
-  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  constexpr int TMAX = kDsTile + (K + S - 1) / S + 1, PITCH = TMAX | 1, PLANE = TMAX * PITCH;
+  constexpr int CHUNK = kDsOC * PLANE, NTR = (CHUNK + 63) / 64;   // floats / transfers per chunk of channels
+  constexpr int WCH = kDsOC * KK * 4, NTW = (WCH + 63) / 64;       // the chunk's weights
+  constexpr int NACC = NCLS * 4 * CN;                              // sums per lane
+  constexpr int WOFF = NTR * 64;                                   // weights behind the planes (16-byte aligned)
+  constexpr int WAVE_LDS = WOFF + NTW * 64;
+  static_assert(NACC * 64 <= 4 * WAVE_LDS, "one wavefront's sums fit the block's LDS");
+  __shared__ float lds[4 * WAVE_LDS];
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const int tx = lane & 7, ty = lane >> 3;
   const int by = blockIdx.x / a.tiles_x, bx = blockIdx.x - by * a.tiles_x, n = blockIdx.y;
   const int y0 = by * kDsTile, x0 = bx * kDsTile;
   const int oh0 = a.oh_base + y0, ow0 = a.ow_base + x0;
+  float* const tile = lds + wave * WAVE_LDS;
   float acc[NCLS][2][2][CN];
 #pragma unroll
   for (int q = 0; q < NCLS; ++q)
@@ -124,28 +139,38 @@ __global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
 #pragma unroll
         for (int c = 0; c < CN; ++c) acc[q][i][j][c] = 0.0f;
   const uint32_t plane = (uint32_t)a.OH * a.OW;
-  const rsrc_t rs = make_rsrc(a.dY, (uint32_t)a.N * a.O * plane * 4u);
-  // this lane's column of a tile row; lanes past the tile width take no part in the transfers
-  const int ow = ow0 + lane;
-  const bool col_lane = lane < a.tw, col_ok = (uint32_t)ow < (uint32_t)a.OW;
-  for (int o0 = 0; o0 < a.O; o0 += kDsOC) {
-    __syncthreads();
-    if (col_lane) {
-      for (int q = wave; q < kDsOC * a.th; q += 4) {   // (channel, row) pairs of the chunk, one transfer each
-        const int o = q / a.th, r = q - o * a.th, oh = oh0 + r;
-        const bool ok = col_ok && o0 + o < a.O && (uint32_t)oh < (uint32_t)a.OH;
-        const uint32_t voff = ok ? (((uint32_t)n * a.O + o0 + o) * plane + (uint32_t)oh * a.OW + ow) * 4u : OOB;
-        buf_load_lds4(rs, tile + o * PLANE + r * PITCH, voff, 0);
-      }
-    }
+  // this image's dY: a channel past the last one lies past the end of the buffer and reads as zero
+  const rsrc_t rs = make_rsrc(a.dY + (size_t)n * a.O * plane, (uint32_t)a.O * plane * 4u);
+  // where this lane's element of each transfer lies in dY, relative to the chunk's first channel
+  uint32_t voff[NTR];
+#pragma unroll
+  for (int t = 0; t < NTR; ++t) {
+    const int f = t * 64 + lane, o = f / PLANE, rem = f - o * PLANE, r = rem / PITCH, c = rem - r * PITCH;
+    const int oh = oh0 + r, ow = ow0 + c;
+    const bool ok = f < CHUNK && r < a.th && c < a.tw && (uint32_t)oh < (uint32_t)a.OH && (uint32_t)ow < (uint32_t)a.OW;
+    voff[t] = ok ? ((uint32_t)o * plane + (uint32_t)oh * a.OW + (uint32_t)ow) * 4u : OOB;
+  }
+  // the weights Wc[o][tap][4] of a chunk are WCH consecutive floats; output channels past the last read as zero
+  const rsrc_t rw = make_rsrc(a.wc, (uint32_t)a.O * KK * 16u);
+  uint32_t woff[NTW];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) woff[t] = t * 64 + lane < WCH ? (uint32_t)(t * 64 + lane) * 4u : OOB;
+  // this wavefront's output channels: [obeg, oend), whole chunks except at the end
+  const int per = ((a.O + 3) / 4 + kDsOC - 1) / kDsOC * kDsOC;
+  const int obeg = wave * per, oend = obeg + per < a.O ? obeg + per : a.O;
+  for (int o0 = obeg; o0 < oend; o0 += kDsOC) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the previous chunk has been read
+    const uint32_t soff = (uint32_t)o0 * plane * 4u;
+#pragma unroll
+    for (int t = 0; t < NTR; ++t) buf_load_lds4(rs, tile + t * 64, voff[t], soff);
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) buf_load_lds4(rw, tile + WOFF + t * 64, woff[t], (uint32_t)o0 * KK * 16u);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    const int on = a.O - o0 < kDsOC ? a.O - o0 : kDsOC;
+    const int on = oend - o0 < kDsOC ? oend - o0 : kDsOC;
 #pragma unroll 1
     for (int o = 0; o < on; ++o) {
       const float* t = tile + o * PLANE;
-      // the same address in every lane: the weights arrive through the scalar cache
-      const float* wo = a.wc + (size_t)(o0 + o) * KK * 4;
+      const float* wo = tile + WOFF + o * KK * 4;
       SmallDgradClass<S, K, CN, 0>::accumulate(a, t, PITCH, wo, ty, tx, acc[0]);
       if constexpr (NCLS > 1) {
         SmallDgradClass<S, K, CN, 1>::accumulate(a, t, PITCH, wo, ty, tx, acc[1]);
@@ -154,6 +179,36 @@ __global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
       }
     }
   }
+  // sums of wavefronts 1..3 to wavefront 0, one after the other through the (now idle) planes, added in that order
+  __syncthreads();
+#pragma unroll 1
+  for (int w = 1; w < 4; ++w) {
+    if (wave == w) {
+      int k = 0;
+#pragma unroll
+      for (int q = 0; q < NCLS; ++q)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int c = 0; c < CN; ++c, ++k) lds[k * 64 + lane] = acc[q][i][j][c];
+    }
+    __syncthreads();
+    if (wave == 0) {
+      int k = 0;
+#pragma unroll
+      for (int q = 0; q < NCLS; ++q)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int c = 0; c < CN; ++c, ++k) acc[q][i][j][c] += lds[k * 64 + lane];
+    }
+    __syncthreads();
+  }
+  if (wave != 0) return;
   SmallDgradClass<S, K, CN, 0>::store(a, n, y0, x0, ty, tx, acc[0]);
   if constexpr (NCLS > 1) {
     SmallDgradClass<S, K, CN, 1>::store(a, n, y0, x0, ty, tx, acc[1]);
@@ -174,7 +229,7 @@ static bool small_dgrad_applies(int cus, const ConvGeom& g) {
   const long long ph = (g.IH + g.S - 1) / g.S, pw = (g.IW + g.S - 1) / g.S;
   const long long blocks = ((ph + kDsTile - 1) / kDsTile) * ((pw + kDsTile - 1) / kDsTile) * g.N;
   if ((uint64_t)g.N * g.O * g.OHW * 4 > kMaxTensorBytes) return false;
-  return blocks * 2 >= cus;
+  return blocks >= cus;   // at least one block of four wavefronts per compute unit
 }
 
 constexpr int kNotHere = 1;   // plan_small_dgrad: a geometry it leaves to the general path (no error)
@@ -214,7 +269,7 @@ static int plan_small_dgrad(const ConvGeom& g, int beta, SmallDgradArgs& a, int*
   a.oh_base = lo_h; a.ow_base = lo_w;
   a.th = kDsTile + hi_h - lo_h; a.tw = kDsTile + hi_w - lo_w;
   const int tmax = kDsTile + (K + S - 1) / S + 1;
-  if (a.th > tmax || a.tw > tmax || a.tw > 64) return kNotHere;
+  if (a.th > tmax || a.tw > tmax) return kNotHere;
   a.tiles_x = (max_pw + kDsTile - 1) / kDsTile;
   *grid_x = a.tiles_x * ((max_ph + kDsTile - 1) / kDsTile);
   return LNN_OK;
@@ -264,9 +319,9 @@ int conv_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* 
         for (int cls = 0; cls < S * S; ++cls) {
           const int nkh = ds_nk(K, S, cls / S), nkw = ds_nk(K, S, cls % S);
           if (nkh == 0 || nkw == 0) continue;
-          // thread (ty, tx), ty, tx < 16, reads rows dh + 2*ty - (nkh-1) ... + nkh, likewise columns
-          lo_r = std::min(lo_r, a.dh[cls] - (nkh - 1)); hi_r = std::max(hi_r, a.dh[cls] + 2 * 15 + 1);
-          lo_c = std::min(lo_c, a.dw[cls] - (nkw - 1)); hi_c = std::max(hi_c, a.dw[cls] + 2 * 15 + 1);
+          // lane (ty, tx), ty, tx < 8, reads rows dh + 2*ty - (nkh-1) ... dh + 2*ty + 1, likewise columns
+          lo_r = std::min(lo_r, a.dh[cls] - (nkh - 1)); hi_r = std::max(hi_r, a.dh[cls] + 2 * 7 + 1);
+          lo_c = std::min(lo_c, a.dw[cls] - (nkw - 1)); hi_c = std::max(hi_c, a.dw[cls] + 2 * 7 + 1);
         }
         tile_info[0] = a.th; tile_info[1] = a.tw; tile_info[2] = kDsTile + (K + S - 1) / S + 1;
         tile_info[3] = lo_r; tile_info[4] = lo_c; tile_info[5] = hi_r; tile_info[6] = hi_c;

@@ -30,8 +30,7 @@ def test_vector_path_tiles_stay_inside_their_lds_plane():
                 n_vec += 1
                 tag = (s, K, padding, H, W, C, beta, t)
                 assert 0 < t['rows'] <= t['max_extent'] and 0 < t['cols'] <= t['max_extent'], tag
-                assert t['cols'] <= 64, tag                          # one lane of a wavefront per tile column
-                assert t['max_extent'] == 32 + (K + s - 1) // s + 1, tag
+                assert t['max_extent'] == 16 + (K + s - 1) // s + 1, tag
                 assert t['min_row'] >= 0 and t['min_col'] >= 0, tag
                 assert t['max_row'] < t['rows'] and t['max_col'] < t['cols'], tag
     assert n_vec > 1000
@@ -51,10 +50,10 @@ def test_selection_rules():
     assert path(3, 7, 1) == api.DGRAD_PATH_MFMA_TABLE             # 7 x 7 at stride 1
     assert path(3, 3, 1, O=32) == api.DGRAD_PATH_VECTOR           # C decides, not O
     assert path(8, 3, 1, O=32) == api.DGRAD_PATH_MFMA_TAP
-    # too few tiles for the chip: 3 x 3 tiles of 32 x 32 per 70 x 66 image at stride 1
-    assert path(3, 3, 1, N=14, cus=256) == api.DGRAD_PATH_MFMA_TABLE       # 126 blocks < 128
-    assert path(3, 3, 1, N=15, cus=256) == api.DGRAD_PATH_VECTOR           # 135 blocks
-    assert path(3, 3, 1, N=14, cus=128) == api.DGRAD_PATH_VECTOR           # the same problem on a smaller part
+    # too few tiles for the chip: 5 x 5 tiles of 16 x 16 per 70 x 66 image at stride 1, one block each
+    assert path(3, 3, 1, N=10, cus=256) == api.DGRAD_PATH_MFMA_TABLE       # 250 blocks < 256
+    assert path(3, 3, 1, N=11, cus=256) == api.DGRAD_PATH_VECTOR           # 275 blocks
+    assert path(3, 3, 1, N=10, cus=128) == api.DGRAD_PATH_VECTOR           # the same problem on a smaller part
     assert path(3, 3, 1, N=1, cus=304) == api.DGRAD_PATH_MFMA_TABLE
 
 

@@ -307,18 +307,19 @@ def test_conv_wgrad_128bit_pixel_gather_integer_exact(hip):
 
 def test_conv_dgrad_few_input_channels_vector_kernel_integer_exact(hip):
     """C <= 4, dilation 1, stride 1 (K = 1, 3, 5) or 2 (K = 3, 4, 5, 7) with enough tiles for the chip takes the
-    vector-ALU data gradient (all pixel classes of a 32 x 32 tile in one block).  Image sizes that are not multiples
+    vector-ALU data gradient (all pixel classes of a 16 x 16 tile in one block, a quarter of the output channels per
+    wavefront).  Image sizes that are not multiples
     of the tile, every padding kind, '=' and '+=', and the neighbouring shapes that stay on the MFMA path."""
     rs = np.random.RandomState(41)
     vec = [(16, 3, 1, 3, 'same', 5), (16, 4, 1, 5, 'valid', 3), (16, 1, 1, 1, 'same', 6), (16, 2, 1, 3, 2, 4),
            (16, 3, 1, 5, (1, 0, 3, 2), 3), (40, 3, 2, 7, 3, 1), (40, 3, 2, 5, 'same', 3), (40, 4, 2, 4, 1, 3),
            (40, 1, 2, 3, 'valid', 4), (40, 2, 2, 5, (0, 2, 1, 0), 3), (40, 3, 2, 3, 0, 5), (40, 3, 2, 4, (2, 1, 0, 3), 2),
-           # output channels are walked in chunks of 8 held in LDS: exactly one chunk, one chunk and a ragged second,
-           # several chunks with a ragged last, eight full chunks
+           # each wavefront walks its quarter of the output channels in chunks of 4 held in LDS: wavefronts without
+           # channels, ragged last chunks, ragged last quarters, four full chunks each
            (40, 3, 2, 7, 3, 8), (40, 3, 2, 7, 3, 9), (40, 3, 2, 7, 3, 20), (40, 3, 2, 7, 3, 64),
            (16, 3, 1, 3, 'same', 9), (16, 4, 1, 5, 'same', 20), (16, 3, 1, 3, 'same', 64), (16, 1, 1, 5, 2, 8),
            (40, 4, 2, 4, 1, 17), (40, 3, 2, 5, 'same', 64), (40, 2, 2, 3, 1, 16), (16, 3, 1, 1, 0, 33)]
-    mfma = [# fewer images, i.e. fewer tiles than half the chip: these stay on the MFMA path
+    mfma = [# fewer images, i.e. fewer tiles than compute units: these stay on the MFMA path
             (16, 3, 2, 5, 'same', 3), (16, 4, 2, 7, 3, 2), (6, 3, 1, 3, 'same', 4), (6, 2, 1, 5, (2, 0, 1, 3), 3),
             (16, 1, 2, 4, 1, 3), (16, 3, 2, 3, (1, 0, 0, 1), 4), (16, 3, 2, 7, 3, 20),
             # not covered by the kernel: dilation, stride 3, 7 x 7 at stride 1
@@ -769,7 +770,7 @@ def test_conv_full_size_adjoint_and_linearity(hip, xs, ws, s, d, padding):
     dy = rs.normal(0, 1, (xs[0], ws[0], ci.OH, ci.OW)).astype(np.float32)
     say(f'full-size identities x={xs} w={ws}')
     if xs[1] == 3 and hip.device_info(0)['compute_units'] == 256:
-        # the image stem at full batch is the shape the vector-ALU data gradient exists for (8 chunks of output channels)
+        # the image stem at full batch is the shape the vector-ALU data gradient exists for (four chunks of output channels per wavefront)
         assert hip.conv2d_dgrad_path(desc, 0, 256)[0] == hip.DGRAD_PATH_VECTOR
     X, W, W2, dY = DevArr(hip, x), DevArr(hip, w), DevArr(hip, w2), DevArr(hip, dy)
     Y, Y2, Y12 = (DevArr(hip, shape=dy.shape, fill=np.nan) for _ in range(3))
