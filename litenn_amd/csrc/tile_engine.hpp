@@ -58,7 +58,16 @@ constexpr int BIG = 0x40000000;   // coordinate that fails every range test
 //   LAY_MC        tile[k][R]:     row contiguous, one tile shared by both groups
 //   LAY_MC_SPLIT  one tile[k][R'] per group, back to back: a group's slab of R' rows
 //                 starting at tile row `off` begins at float off*BK
-enum { LAY_KC = 0, LAY_KC_SWZ = 1, LAY_MC = 2, LAY_MC_SPLIT = 3 };
+enum { LAY_KC = 0, LAY_KC_SWZ = 1, LAY_MC = 2, LAY_MC_SPLIT = 3, LAY_KC_SWZP = 4 };
+//   LAY_KC_SWZP   the same with group g of row r in slot g ^ ((r / 2) % 8).  LDS has 64 banks of 4 bytes and serves a
+//                 128-bit read 16 lanes at a time; rows of 128 bytes alternate between the two bank halves, so 16
+//                 consecutive rows reading the same group are conflict free only if the eight rows of each parity sit
+//                 in eight different slots.  Keyed by r % 8 (LAY_KC_SWZ) rows r and r + 8 collide: measured 32 cycles
+//                 per ds_read_b128 against 16.  Loaders that move 16 bytes per lane use this key; those that move 4
+//                 bytes per lane fill a row pair per instruction and need one key per wavefront, which only the r % 8
+//                 key gives them.
+constexpr bool lay_kc(int l) { return l == LAY_KC || l == LAY_KC_SWZ || l == LAY_KC_SWZP; }
+constexpr bool lay_swz(int l) { return l == LAY_KC_SWZ || l == LAY_KC_SWZP; }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -188,12 +197,12 @@ struct PlainKC {
 // Plain strided matrix, K-contiguous, straight into LDS (needs K % BK == 0 and
 // 16-byte aligned rows).  The LDS tile is [row][BK] without padding; to keep
 // the 128-bit fragment reads conflict free the k groups of a row are stored
-// XOR-swizzled: group g of row r sits in slot g ^ (r % 8).  One instruction
+// XOR-swizzled: group g of row r sits in slot g ^ ((r / 2) % 8) (LAY_KC_SWZP).  One instruction
 // moves 8 rows (1 KiB): lane l carries slot l % 8 of row l / 8.
 template <int R>
 struct DirectKC {
   static constexpr bool KC = true, DIRECT = true;
-  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int LAYOUT = LAY_KC_SWZP;
   static constexpr int NB = R / 8, E = (NB + 3) / 4;
   static constexpr int NLD = NB % 4 == 0 ? E : -1;   // transfers per wavefront and K step (-1: differs between wavefronts)
   static_assert(R % 8 == 0, "whole 8-row blocks");
@@ -201,7 +210,8 @@ struct DirectKC {
   uint32_t voff[E];
   __device__ __forceinline__ void init(rsrc_t r, int ld, int row0, int M, int) {
     rs = r;
-    const int wave = gwave(), lane = threadIdx.x & 63, rb = lane >> 3, kg = (lane & 7) ^ rb;
+    // tile row = 8 * (wave + 4e) + rb (plus the group's offset, a multiple of 16): (row / 2) % 8 is the same for all e
+    const int wave = gwave(), lane = threadIdx.x & 63, rb = lane >> 3, kg = (lane & 7) ^ (((wave & 1) << 2) | (rb >> 1));
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const int row = row0 + (wave + 4 * e) * 8 + rb;
@@ -1204,7 +1214,7 @@ struct ConvWgradTapADirect {
 template <int R>
 struct ConvWgradTapA4Direct {
   static constexpr bool KC = true, DIRECT = true;
-  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int LAYOUT = LAY_KC_SWZP;
   static constexpr int NB = R / 8, E = (NB + 3) / 4;
   static constexpr int NLD = NB % 4 == 0 ? E : -1;
   static_assert(R % 8 == 0, "whole 8-row blocks");
@@ -1216,7 +1226,7 @@ struct ConvWgradTapA4Direct {
     kend = kend_;
     awrap = g.O * g.OHW - g.OHW;
     const int lane = threadIdx.x & 63, rb = lane >> 3;
-    p = k0 + 4 * ((lane & 7) ^ rb);
+    p = k0 + 4 * ((lane & 7) ^ ((((int)gwave() & 1) << 2) | (rb >> 1)));   // LAY_KC_SWZP: key (row / 2) % 8
     const uint32_t img = g.dOHW.div((uint32_t)p);
     rem = p - (int)img * g.OHW;
     aoff = (int)img * g.O * g.OHW + rem + (o0 + 8 * gwave() + rb) * g.OHW;
@@ -1321,7 +1331,7 @@ struct ConvWgradTapBDirect {
 template <int R>
 struct ConvWgradTapB4Direct {
   static constexpr bool KC = true, DIRECT = true;
-  static constexpr int LAYOUT = LAY_KC_SWZ;
+  static constexpr int LAYOUT = LAY_KC_SWZP;
   static constexpr int NB = R / 8, E = (NB + 3) / 4;
   static constexpr int NLD = NB % 4 == 0 ? E : -1;
   static_assert(R % 8 == 0, "whole 8-row blocks");
@@ -1341,7 +1351,7 @@ struct ConvWgradTapB4Direct {
     xwrap_w = g.IW - g.OW;
     xwrap_h = g.C * g.IHW - g.OH * g.IW;
     const int lane = threadIdx.x & 63, rb = lane >> 3;
-    p = k0 + 4 * ((lane & 7) ^ rb);
+    p = k0 + 4 * ((lane & 7) ^ ((((int)gwave() & 1) << 2) | (rb >> 1)));   // LAY_KC_SWZP: key (row / 2) % 8
     const uint32_t img = g.dOHW.div((uint32_t)p), rem = (uint32_t)p - img * g.OHW;
     oh = (int)g.dOW.div(rem);
     ow = (int)rem - oh * g.OW;
@@ -1485,9 +1495,10 @@ __device__ __forceinline__ void load_frags(const float* __restrict__ As, const f
                                            int brow, int kk, float (&a)[4], float (&b)[NT][4]) {
   const int lane = threadIdx.x & 63, i = lane & 31, h = lane >> 5;
   const int kb = kk * 8 + h * 4;
-  const int sw = ((2 * kk + h) ^ (i & 7)) << 2;   // swizzled position of k group 2*kk + h; row offsets are multiples of 32
-  if (LAY_A == LAY_KC || LAY_A == LAY_KC_SWZ) {
-    const f32x4 t = *reinterpret_cast<const f32x4*>(LAY_A == LAY_KC ? &As[(arow + i) * LDK + kb] : &As[(arow + i) * BK + sw]);
+  // swizzled position of k group 2*kk + h; row offsets are multiples of 32
+  const int sw = ((2 * kk + h) ^ (i & 7)) << 2, swp = ((2 * kk + h) ^ ((i >> 1) & 7)) << 2;
+  if (lay_kc(LAY_A)) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(LAY_A == LAY_KC ? &As[(arow + i) * LDK + kb] : &As[(arow + i) * BK + (LAY_A == LAY_KC_SWZP ? swp : sw)]);
     a[0] = t[0]; a[1] = t[1]; a[2] = t[2]; a[3] = t[3];
   } else if (LAY_A == LAY_MC) {
     const float* ap = As + (arow + i + h * (4 * RA));   // one address per lane, k as immediate offsets
@@ -1503,9 +1514,9 @@ __device__ __forceinline__ void load_frags(const float* __restrict__ As, const f
   }
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
-    if (LAY_B == LAY_KC || LAY_B == LAY_KC_SWZ) {
+    if (lay_kc(LAY_B)) {
       const int r = brow + 32 * j + i;
-      const f32x4 t = *reinterpret_cast<const f32x4*>(LAY_B == LAY_KC ? &Bs[r * LDK + kb] : &Bs[r * BK + sw]);
+      const f32x4 t = *reinterpret_cast<const f32x4*>(LAY_B == LAY_KC ? &Bs[r * LDK + kb] : &Bs[r * BK + (LAY_B == LAY_KC_SWZP ? swp : sw)]);
       b[j][0] = t[0]; b[j][1] = t[1]; b[j][2] = t[2]; b[j][3] = t[3];
     } else {   // shared tile or the group's own slab: the caller passes the matching base, pitch and brow
       // one address per lane and accumulator tile; kk and t are immediate offsets, so with RB a multiple
@@ -1527,7 +1538,7 @@ __device__ __forceinline__ void mma_stage(const float* __restrict__ As, const fl
   constexpr int NG = BK / 8;
   float fa[2][4], fb[2][NT][4];
   // LDS read instructions per group: A is one b128 or four b32; B is NT b128 or 4*NT b32 (paired into read2)
-  constexpr int RD = (LAY_A <= LAY_KC_SWZ ? 1 : 2) + (LAY_B <= LAY_KC_SWZ ? NT : 2 * NT);
+  constexpr int RD = (lay_kc(LAY_A) ? 1 : 2) + (lay_kc(LAY_B) ? NT : 2 * NT);
   load_frags<NT, LAY_A, LAY_B, RA, RB>(As, Bs, arow, brow, 0, fa[0], fb[0]);
   __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);              // DS reads of group 0
 #pragma unroll
@@ -1569,7 +1580,7 @@ __device__ __forceinline__ void mma_stage_stream(const float* __restrict__ As, c
                                                  int brow, MID mid, SEND send) {
   constexpr int NG = BK / 8;
   static_assert(NG == 4, "four groups, four shares of transfers; the next stage's first group lands in buffer 0");
-  constexpr int RD = (LAY_A <= LAY_KC_SWZ ? 1 : 2) + (LAY_B <= LAY_KC_SWZ ? NT : 2 * NT);
+  constexpr int RD = (lay_kc(LAY_A) ? 1 : 2) + (lay_kc(LAY_B) ? NT : 2 * NT);
   constexpr int G = 4 * NT;                       // MFMAs per group
   constexpr int PAIRS = RD < G ? RD : G;          // MFMAs of a group that carry a fragment read
   constexpr int FREE = G - PAIRS;                 // ... and those that do not
@@ -1739,8 +1750,8 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
   using LA = typename P::template LA<HALF>;
   using LB = typename P::template LB<BN>;
   constexpr int LAY_A = layout_of<LA>::value, LAY_B = layout_of<LB>::value;
-  constexpr int LDA = LAY_A == LAY_KC ? LDK : (LAY_A == LAY_KC_SWZ ? BK : BM);
-  constexpr int LDB = LAY_B == LAY_KC ? LDK : (LAY_B == LAY_KC_SWZ ? BK : BNTOT);
+  constexpr int LDA = LAY_A == LAY_KC ? LDK : (lay_swz(LAY_A) ? BK : BM);
+  constexpr int LDB = LAY_B == LAY_KC ? LDK : (lay_swz(LAY_B) ? BK : BNTOT);
   const int wave = gwave(), lane = threadIdx.x & 63;
   const int wm = wave % WM, wn = wave / WM;
   // fragment addressing: a split B tile is read through the group's own slab
