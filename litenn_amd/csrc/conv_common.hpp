@@ -14,6 +14,10 @@
 
 #include "common.hpp"
 
+// Forward / dgrad: remainder units cut along K (see plan_tiles).
+#ifndef LNN_TAIL_SPLIT
+#define LNN_TAIL_SPLIT 1
+#endif
 #ifndef LNN_STAGES_WGRAD
 #define LNN_STAGES_WGRAD 3
 #endif
@@ -66,6 +70,12 @@ struct ConvArgs {
   // tap-major wgrad: the columns of an M tile form segs_per_mt segments of seg_units units; a group's columns stay
   // inside one segment (one tap, for the loaders that assume it; the whole row for the one that does not)
   int seg_units, segs_per_mt;
+  // forward / dgrad without a K split: units that do not divide evenly among the workgroups.  The first main_units
+  // units (a whole number per workgroup) are computed as usual; each of the tail_units left over is cut into
+  // tail_split K slices, one per workgroup, whose partial sums go to tail_part[slice][unit][BM][unit width] and are
+  // added up by reduce_tail.  tail_units = 0: no tail.
+  int main_units, tail_units, tail_split;
+  float* tail_part;
 };
 
 // One class of input pixels of a strided dgrad: pixels (h0 + S*i, w0 + S*j),
@@ -429,9 +439,54 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
   if (wgrad_tap(PASS))
     walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.seg_units, a.segs_per_mt, a.total_units,
                               a.chunk_units, chunk_i);
-  else
+  else if (a.tail_units == 0) {
     walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units,
                           bx, a.grid_x);
+  } else {
+    walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.main_units,
+                          bx, a.grid_x);
+    if (bx < a.tail_units * a.tail_split) {
+      constexpr int WN = 4 / WM, BM = 32 * WM, UW = 32 * WN;
+      const int j = bx / a.tail_split, slice = bx - j * a.tail_split;
+      const int u = a.main_units + j, mt = u / a.n_units, n0 = (u - mt * a.n_units) * UW;
+      const int nkt = (a.K + BK - 1) / BK;
+      const int t0 = (int)((long long)nkt * slice / a.tail_split), t1 = (int)((long long)nkt * (slice + 1) / a.tail_split);
+      p.kbeg = t0 * BK;
+      p.kend = t1 * BK < a.K ? t1 * BK : a.K;
+      // element (m, n) of the unit at (m - mt*BM) * UW + (n - n0) of its block: a plain map of pitch UW over a
+      // buffer that begins that much before the block
+      const int shift = mt * BM * UW + n0;
+      p.rc = make_rsrc(a.tail_part + (size_t)(slice * a.tail_units + j) * (BM * UW) - shift, (uint32_t)(shift + BM * UW) * 4u);
+      p.om = plain_map(UW);
+      p.beta = 0;
+      p.post.bias = nullptr; p.post.act = 0;   // applied by reduce_tail
+      run_pair<WM, NTMAX, false>(1, 0, p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, mt * BM, n0, n0 + UW);
+    }
+  }
+}
+
+// Sum of the K slices of the tail units (see ConvArgs), one thread per element, slices added in order; applies the
+// final output mapping, '+=' and the bias / activation epilogue.
+struct TailArgs {
+  const float* part;
+  int tail_units, tail_split, main_units, n_units, M, Ncols, beta, bm, uw;
+  OutMap om;
+  PostOp post;
+};
+__global__ __launch_bounds__(256) void reduce_tail(float* out, TailArgs t) {
+  const int per = t.bm * t.uw;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= t.tail_units * per) return;
+  const int j = i / per, e = i - j * per, row = e / t.uw, col = e - row * t.uw;
+  const int u = t.main_units + j, mt = u / t.n_units;
+  const int m = mt * t.bm + row, n = (u - mt * t.n_units) * t.uw + col;
+  if (m >= t.M || n >= t.Ncols) return;
+  float v = 0.0f;
+  for (int s = 0; s < t.tail_split; ++s) v += t.part[(size_t)(s * t.tail_units + j) * per + e];
+  float* dst = out + ((size_t)t.om.col((uint32_t)n) + (size_t)m * t.om.ld);
+  if (t.beta) v += *dst;
+  else if (t.post.any()) v = t.post.apply(v, t.post.bias != nullptr ? t.post.bias[m] : 0.0f);
+  *dst = v;
 }
 
 template <int PASS, int WM, int NTMAX, bool FLAG>
@@ -589,7 +644,7 @@ static int launch_reduce(DeviceCtx* ctx, const ConvArgs& a, float* final_out, in
 // Forward / dgrad: units, grid and K split of one problem that may use `slots` workgroups.
 // Returns the bytes of partial sums it needs (0 without a K split).
 template <int WM, int NTMAX>
-static size_t plan_tiles(ConvArgs& a, long long slots) {
+static size_t plan_tiles(ConvArgs& a, long long slots, bool allow_tail = false) {
   constexpr int WN = 4 / WM, BM = 32 * WM;
   const int m_tiles = (a.M + BM - 1) / BM;
   a.n_units = (a.Ncols + 32 * WN - 1) / (32 * WN);
@@ -600,6 +655,7 @@ static size_t plan_tiles(ConvArgs& a, long long slots) {
   a.ks_last = 1;
   a.ksplit = 1;
   a.grid_x = (int)(total < slots ? total : slots);
+  a.main_units = a.total_units; a.tail_units = 0; a.tail_split = 1; a.tail_part = nullptr;
   // Few output tiles (small images, deep layers): a workgroup's share would be a sliver of a sub-tile and
   // most of its time data movement.  Cut the output into full sub-tiles instead and split K over the
   // workgroups that are left, as wgrad does.
@@ -615,6 +671,19 @@ static size_t plan_tiles(ConvArgs& a, long long slots) {
       return (size_t)a.ksplit * a.M * a.Ncols * sizeof(float);
     }
   }
+  // A few units per workgroup and a remainder: the workgroups that would take one unit more set the pace
+  // (3136 units on 256 workgroups: 13 against 12.25).  Cut the remainder along K instead, one slice per workgroup.
+  if (allow_tail && LNN_TAIL_SPLIT && total > slots && total <= 64 * slots) {
+    const long long q = total / slots, r = total - q * slots;
+    long long ts = r > 0 ? slots / r : 0;
+    if (ts > nkt / 6) ts = nkt / 6;   // a slice should still hold a handful of K steps
+    if (ts >= 2) {
+      a.main_units = (int)(q * slots);
+      a.tail_units = (int)r;
+      a.tail_split = (int)ts;
+      return (size_t)ts * r * BM * (32 * WN) * sizeof(float);
+    }
+  }
   return 0;
 }
 
@@ -625,6 +694,7 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   float* final_out = a.Out;
   const int final_beta = a.beta;
   int grid_y = 1;
+  a.main_units = 0; a.tail_units = 0; a.tail_split = 1; a.tail_part = nullptr;
   if (PASS == PASS_WGRAD || wgrad_tap(PASS)) {
     const int m_tiles = (a.M + BM - 1) / BM;
     a.n_units = (a.Ncols + 32 * WN - 1) / (32 * WN);
@@ -684,15 +754,20 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
       a.beta = 0;
     }
   } else {
-    const size_t need = plan_tiles<WM, NTMAX>(a, slots);
+    const size_t need = plan_tiles<WM, NTMAX>(a, slots, true);
     if (a.total_units < 0) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
     if (need) {
       // the scratch buffer may already hold this call's permuted weights: keep them in front
       int st = ensure_workspace(ctx, a.ws_used + need);
       if (st != LNN_OK) return st;
-      a.Out = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + a.ws_used);
-      a.beta = 0;
-      grid_y = a.ksplit;
+      float* scratch = reinterpret_cast<float*>(static_cast<char*>(ctx->ws) + a.ws_used);
+      if (a.tail_units > 0) {
+        a.tail_part = scratch;
+      } else {
+        a.Out = scratch;
+        a.beta = 0;
+        grid_y = a.ksplit;
+      }
     }
   }
   dim3 g(a.grid_x, grid_y, 1), b(512, 1, 1);
@@ -704,6 +779,17 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   }
   LNN_HIP(hipGetLastError());
   if (a.ksplit > 1) return launch_reduce<PASS, WM>(ctx, a, final_out, final_beta);
+  if (a.tail_units > 0) {
+    TailArgs t;
+    t.part = a.tail_part;
+    t.tail_units = a.tail_units; t.tail_split = a.tail_split; t.main_units = a.main_units; t.n_units = a.n_units;
+    t.M = a.M; t.Ncols = a.Ncols; t.beta = final_beta; t.bm = BM; t.uw = 32 * WN;
+    t.om = final_map<PASS>(a);
+    t.post = a.post;
+    const int n = a.tail_units * BM * 32 * WN;
+    hipLaunchKernelGGL(reduce_tail, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, final_out, t);
+    LNN_HIP(hipGetLastError());
+  }
   return LNN_OK;
 }
 

@@ -539,8 +539,8 @@ struct ConvFwdBDirect {
 #pragma unroll
       for (int c = 0; c < CC; ++c) {
         const bool ok = (uint32_t)(ih0[c] + ty[e]) < (uint32_t)IH && (uint32_t)(iw0[c] + tz[e]) < (uint32_t)IW;
-        if (R % 64 == 0 || lane + 64 * c < R)
-          buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, ok ? (uint32_t)(base[c] + tx[e]) * 4u : OOB, 0);
+        // all 64 lanes, also where the group is narrower (see run_tile): no lane mask around a transfer
+        buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, ok ? (uint32_t)(base[c] + tx[e]) * 4u : OOB, 0);
       }
     }
     if (PART == NPARTS - 1) load_entries(k0 + BK);
@@ -643,7 +643,7 @@ struct ConvFwdBTap {
       const uint32_t soff = (uint32_t)((c0 + wave + 4 * e) * IHW) * 4u;
 #pragma unroll
       for (int c = 0; c < CC; ++c)
-        if (R % 64 == 0 || lane + 64 * c < R) buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);
+        buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);   // all 64 lanes (see run_tile)
     }
     if (PART == NPARTS - 1) advance();
     return (KR * (PART + 1) / NPARTS - KR * PART / NPARTS) * CC;
@@ -750,7 +750,7 @@ struct ConvDgradBTap {
       const uint32_t soff = (uint32_t)((o0 + wave + 4 * e) * OHW) * 4u;
 #pragma unroll
       for (int c = 0; c < CC; ++c)
-        if (R % 64 == 0 || lane + 64 * c < R) buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);
+        buf_load_lds4(rs, lds + (wave + 4 * e) * ld + off + 64 * c, voff[c], soff);   // all 64 lanes (see run_tile)
     }
     if (PART == NPARTS - 1) advance();
     return (KR * (PART + 1) / NPARTS - KR * PART / NPARTS) * CC;
@@ -1990,13 +1990,20 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
 template <int WM, int NT0, int NT1, class P>
 __device__ __forceinline__ void run_tile(const P& p, float* ldsA, float* ldsB, int strideA, int strideB, int m0,
                                          int n0a, int n0b) {
-  constexpr int WN = 4 / WM, BNTOT = 32 * WN * (NT0 + NT1);
+  // In LDS each group's columns start at a multiple of 64 and the tile is a multiple of 64 wide: a global -> LDS
+  // transfer of a pixel gather always deposits 64 lanes, so a group with an odd number of 32-column units would
+  // otherwise need its last transfer masked to 32 lanes - and a lane mask around these transfers is not safe: the
+  // compiler threads the code behind the branch into both paths and then takes the LDS address (M0, one per
+  // wavefront) from whichever path lane 0 took.  The lanes past a group's columns carry the out-of-range offset and
+  // deposit zeros in columns nobody reads.
+  constexpr int WN = 4 / WM, W0 = 32 * WN * NT0, W1 = 32 * WN * NT1;
+  constexpr int COFF1 = (W0 + 63) & ~63, BNTOT = COFF1 + ((W1 + 63) & ~63);
   // wave-uniform by construction; read through a scalar so the two bodies are
   // separate uniform branches (each wavefront executes exactly one of them)
   if (__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8)) == 0)
     group_body<WM, NT0, 0, 0, BNTOT>(p, ldsA, ldsB, strideA, strideB, m0, n0a);
   else
-    group_body<WM, NT1, 1, 32 * WN * NT0, BNTOT>(p, ldsA, ldsB, strideA, strideB, m0, n0b);
+    group_body<WM, NT1, 1, COFF1, BNTOT>(p, ldsA, ldsB, strideA, strideB, m0, n0b);
   __syncthreads();   // the next sub-tile's prologue overwrites stage 0
 }
 

@@ -401,6 +401,45 @@ def test_conv_dgrad_on_forward_permuted_weights_integer_exact(hip):
     assert e.value.code == hip.ERR_INVALID
 
 
+def test_conv_remainder_units_cut_along_k_integer_exact(hip):
+    """Forward and stride-1 data gradient with a few column units per workgroup and a remainder: the remainder
+    units are cut into K slices, one per workgroup, and summed by a small reduction that also applies '+=' and the
+    bias / activation epilogue.  Shapes with 256 q + r units (r <= 128) on the 256 compute units of the MI355X, for
+    the tap-major kernels (one and two row tiles, 3x3 and 1x1) and the any-channel forward; exact on small integers."""
+    rs = np.random.RandomState(63)
+    cases = [((3, 64, 56, 56), (128, 64, 3, 3), 1, 1, 'same'),      # 294 units: 38 left over, 3 slices of 6 K steps
+             ((5, 128, 41, 40), (256, 128, 1, 1), 1, 1, 'valid'),   # two row tiles, 1x1: 4 K steps, no cut possible
+             ((2, 96, 70, 66), (160, 96, 3, 3), 1, 1, 1),           # two row tiles, ragged second; 27 K steps
+             ((20, 32, 33, 31), (64, 32, 5, 5), 1, 2, 'same'),      # 64 rows: units of 64 columns
+             ((4, 24, 50, 50), (96, 24, 5, 5), 1, 1, 'same'),       # any-channel forward (table gather), dgrad on Wp
+             ((8, 160, 64, 72), (32, 160, 3, 3), 1, 1, (0, 1, 1, 0)),   # 32 rows: units of 128 columns
+             # any-channel forward with more than 64 output channels: groups of one and three 32-column units, whose
+             # last transfer per K row covers 32 columns (six and seven units per workgroup; with a K split)
+             ((20, 24, 50, 50), (96, 24, 3, 3), 1, 1, 'same'), ((2, 24, 50, 50), (128, 24, 5, 5), 1, 1, 'same'),
+             ((23, 20, 50, 50), (96, 20, 3, 3), 1, 1, 'valid')]
+    for xs, ws, s, d, padding in cases:
+        say(f'remainder units x={xs} w={ws} s={s} d={d} pad={padding}')
+        desc, ci = _desc(hip, xs, ws, s, d, padding)
+        O = ws[0]
+        x = rs.randint(-2, 3, size=xs).astype(np.float32)
+        w = rs.randint(-2, 3, size=ws).astype(np.float32)
+        dy = rs.randint(-2, 3, size=(xs[0], O, ci.OH, ci.OW)).astype(np.float32)
+        b = rs.randint(-3, 4, size=(O,)).astype(np.float32)
+        ry, rdx, _ = conv2d_all(x, w, dy, s, d, padding)
+        X, W, dY, B = DevArr(hip, x), DevArr(hip, w), DevArr(hip, dy), DevArr(hip, b)
+        for beta, fill in ((0, np.nan), (1, 3.0)):
+            Y = DevArr(hip, shape=dy.shape, fill=fill)
+            hip.conv2d_fwd(0, desc, X.ptr, W.ptr, Y.ptr, beta)
+            assert np.array_equal(Y.get() - (3.0 if beta else 0.0), ry), (xs, ws, beta)
+            dX = DevArr(hip, shape=xs, fill=fill)
+            hip.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, beta)
+            assert np.array_equal(dX.get() - (3.0 if beta else 0.0), rdx), (xs, ws, beta)
+        Y = DevArr(hip, shape=dy.shape, fill=np.nan)
+        hip.conv2d_fwd_bias_act(0, desc, X.ptr, W.ptr, B.ptr, hip.ACT_LEAKY_RELU, 0.25, Y.ptr)
+        pre = ry + b[None, :, None, None]
+        assert np.array_equal(Y.get(), np.where(pre >= 0, pre, 0.25 * pre).astype(np.float32)), (xs, ws)
+
+
 def test_conv_passes_on_weights_with_swapped_channel_axes(hip):
     """A transposed convolution keeps its kernel as [C][O][KH][KW] relative to the convolution whose passes it
     borrows.  lnn_conv2d_permute_weights_f32(LNN_W_IOHW) makes Wp straight from that storage, the *_pw passes run
