@@ -49,6 +49,7 @@ template <bool TA, bool TB, int MODE, int ST>
 struct GemmProblem {
   static constexpr int STAGES = ST;
   static constexpr bool STREAM_UNROLL = !TB;   // measured: A * B^T is slower with constant stages
+  static constexpr bool STREAM_REGIONS = false;   // measured: A * B^T 0.948 -> 0.96 ms with one region per group
   static constexpr bool VEC = MODE >= 1, DIR = MODE == 2;
   template <int R> using KCL = typename std::conditional<DIR, DirectKC<R>, PlainKC<R, VEC>>::type;
   template <int R> using MCL = typename std::conditional<DIR, DirectMC<R>, PlainMC<R, VEC>>::type;

@@ -39,6 +39,12 @@ namespace lnn {
 #ifndef LNN_STREAM
 #define LNN_STREAM 1
 #endif
+#ifndef LNN_GROUP_REGIONS
+#define LNN_GROUP_REGIONS 1
+#endif
+#ifndef LNN_VALU_FIRST
+#define LNN_VALU_FIRST 64
+#endif
 #ifndef LNN_STREAM_UNROLL
 #define LNN_STREAM_UNROLL 1
 #endif
@@ -1573,7 +1579,7 @@ __device__ __forceinline__ void mma_stage(const float* __restrict__ As, const fl
 // wavefront; vector-ALU instructions stop it, and so does anything the other wavefront of the SIMD wants to issue.
 // NV: transfers per wavefront and K step if known (0: unknown or none).
 template <int N> using ic = std::integral_constant<int, N>;
-template <int NT, int LAY_A, int LAY_B, int RA, int RB, int NV, bool NEXT, class MID, class SEND>
+template <int NT, int LAY_A, int LAY_B, int RA, int RB, int NV, bool NEXT, bool REGIONS, class MID, class SEND>
 __device__ __forceinline__ void mma_stage_stream(const float* __restrict__ As, const float* __restrict__ Bs,
                                                  const float* __restrict__ Asn, const float* __restrict__ Bsn,
                                                  f32x16 (&acc)[NT], float (&fa)[2][4], float (&fb)[2][NT][4], int arow,
@@ -1624,6 +1630,10 @@ __device__ __forceinline__ void mma_stage_stream(const float* __restrict__ As, c
       send(kkc);
       read_slots();
       transfer_slots();
+      // REGIONS (the loops that keep a running stage index): each group is a scheduling region of its own.  With
+      // the whole stage in one region their slots were honoured for the first share only and the other transfers
+      // went out in one burst (config 3 wgrad 0.242 -> 0.235 ms); the unrolled loops schedule well as one region
+      if (LNN_GROUP_REGIONS && REGIONS) __builtin_amdgcn_sched_barrier(0);
     } else {
       mfmas(ic<cur>(), ic<0>(), ic<FREE>());
       send(kkc);
@@ -1636,6 +1646,12 @@ __device__ __forceinline__ void mma_stage_stream(const float* __restrict__ As, c
       if (NEXT) read_slots(); else __builtin_amdgcn_sched_group_barrier(0x008, PAIRS, 0);
     }
   };
+#if LNN_VALU_FIRST
+  if (REGIONS)
+  // vector-ALU instructions of the step (fragment addresses, the loaders' address walks) in one batch at the start:
+  // one alone between two MFMAs costs the matrix pipe 13-18 cycles, in a batch 5-9 each
+    __builtin_amdgcn_sched_group_barrier(0x002, LNN_VALU_FIRST, 0);
+#endif
   group(ic<0>());
   group(ic<1>());
   group(ic<2>());
@@ -1731,6 +1747,13 @@ template <class T, class = void>
 struct stream_unroll : std::integral_constant<bool, LNN_STREAM_UNROLL != 0> {};
 template <class T>
 struct stream_unroll<T, std::void_t<decltype(T::STREAM_UNROLL)>> : std::integral_constant<bool, T::STREAM_UNROLL && LNN_STREAM_UNROLL> {};
+
+// Whether the streaming stage makes each MFMA group a scheduling region of its own (see mma_stage_stream): by default
+// the loops that are not unrolled; a problem overrides it with `static constexpr bool STREAM_REGIONS`.
+template <class T, class = void>
+struct stream_regions : std::integral_constant<bool, !stream_unroll<T>::value> {};
+template <class T>
+struct stream_regions<T, std::void_t<decltype(T::STREAM_REGIONS)>> : std::integral_constant<bool, T::STREAM_REGIONS> {};
 
 template <class LB, class LA>
 __device__ __forceinline__ int issue_b(LB& lb, int k0, float* lds, int ld, int off, LA& la) {
@@ -1849,7 +1872,7 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
         asm volatile("s_barrier" ::: "memory");
       };
       if constexpr (NT > 0) {
-        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, NVT, true>(ldsA + curv * strideA, ldsBr + curv * strideB,
+        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, NVT, true, stream_regions<P>::value>(ldsA + curv * strideA, ldsBr + curv * strideB,
                                                               ldsA + nxt * strideA, ldsBr + nxt * strideB, acc, fa, fb,
                                                               arow, brow, mid, send);
       } else {
@@ -1875,7 +1898,7 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
     if (t + 1 < nk) {   // last but one step: nothing left to send
       const int nxt = cur + 1 == ST ? 0 : cur + 1;
       if constexpr (NT > 0)
-        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, 0, true>(ldsA + cur * strideA, ldsBr + cur * strideB,
+        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, 0, true, stream_regions<P>::value>(ldsA + cur * strideA, ldsBr + cur * strideB,
                                                             ldsA + nxt * strideA, ldsBr + nxt * strideB, acc, fa, fb,
                                                             arow, brow, drain, nothing);
       else
@@ -1885,7 +1908,7 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
     }
     if (t < nk) {       // last step
       if constexpr (NT > 0)
-        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, 0, false>(ldsA + cur * strideA, ldsBr + cur * strideB, ldsA, ldsBr,
+        mma_stage_stream<NTC, LAY_A, LAY_B, BM, RB, 0, false, stream_regions<P>::value>(ldsA + cur * strideA, ldsBr + cur * strideB, ldsA, ldsBr,
                                                              acc, fa, fb, arow, brow, nothing, nothing);
     }
   } else {
