@@ -18,6 +18,9 @@
 #ifndef LNN_TAIL_SPLIT
 #define LNN_TAIL_SPLIT 1
 #endif
+#ifndef LNN_WGRAD_UNROLL
+#define LNN_WGRAD_UNROLL 0
+#endif
 #ifndef LNN_STAGES_WGRAD
 #define LNN_STAGES_WGRAD 3
 #endif
@@ -344,7 +347,8 @@ struct ConvProblem<PASS_WGRAD, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  static constexpr bool STREAM_UNROLL = false;   // measured: slower with constant stages (registers)
+  static constexpr bool STREAM_UNROLL = LNN_WGRAD_UNROLL != 0;   // measured: slower with constant stages (config 3: 0.235 -> 0.247 ms)
+  static constexpr bool STREAM_REGIONS = true;
   template <int R> using LA = typename std::conditional<FLAG, ConvWgradTapA4Direct<R>, ConvWgradTapADirect<R>>::type;
   template <int R> using LB = ConvWgradTapBDirect<R, LNN_WGRAD_B_DIRECT != 0>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }
@@ -354,7 +358,8 @@ struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_ANYC, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  static constexpr bool STREAM_UNROLL = false;   // measured: slower with constant stages (registers)
+  static constexpr bool STREAM_UNROLL = LNN_WGRAD_UNROLL != 0;   // measured: slower with constant stages (config 3: 0.235 -> 0.247 ms)
+  static constexpr bool STREAM_REGIONS = true;
   template <int R> using LA = typename std::conditional<FLAG, ConvWgradTapA4Direct<R>, ConvWgradTapADirect<R>>::type;
   template <int R> using LB = ConvWgradBAnyC<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }
@@ -364,7 +369,8 @@ struct ConvProblem<PASS_WGRAD_ANYC, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_TAP4, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  static constexpr bool STREAM_UNROLL = false;   // measured: slower with constant stages (registers)
+  static constexpr bool STREAM_UNROLL = LNN_WGRAD_UNROLL != 0;   // measured: slower with constant stages (config 3: 0.235 -> 0.247 ms)
+  static constexpr bool STREAM_REGIONS = true;
   template <int R> using LA = ConvWgradTapA4Direct<R>;
   template <int R> using LB = ConvWgradTapB4Direct<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }
