@@ -21,6 +21,9 @@
 #ifndef LNN_WGRAD_UNROLL
 #define LNN_WGRAD_UNROLL 0
 #endif
+#ifndef LNN_KSPLIT_HALF
+#define LNN_KSPLIT_HALF 1
+#endif
 #ifndef LNN_STAGES_WGRAD
 #define LNN_STAGES_WGRAD 3
 #endif
@@ -246,6 +249,27 @@ __device__ __forceinline__ void permute_one(float* wp, const float* w, int O, in
 }
 __global__ void permute_weights(float* wp, const float* w, int O, int C, int KK, int mode, ConvGeom g, PixelClass pc) {
   permute_one(wp, w, O, C, KK, mode, g, pc, blockIdx.x * blockDim.x + threadIdx.x);
+}
+// Modes 0 and 2 through LDS: a block moves 64 channels of one output row, so that its reads and its writes both run
+// along contiguous floats (the element-wise kernel above reads with a stride of KK floats, or of O * KK).
+constexpr int kPermuteMaxKK = 200;   // 64 * (KK | 1) floats of LDS
+__global__ __launch_bounds__(256) void permute_weights_tiled(float* wp, const float* w, int O, int C, int KK, int mode) {
+  extern __shared__ float permute_tile[];
+  const int kkp = KK | 1;   // odd row pitch: the transposed reads spread over the banks
+  const int cblocks = (C + 63) / 64;
+  const int o = blockIdx.x / cblocks, c0 = (blockIdx.x - o * cblocks) * 64;
+  const int nc = C - c0 < 64 ? C - c0 : 64;
+  const int n = nc * KK;
+  const float* src = w + ((size_t)o * C + c0) * KK;
+  for (int j = threadIdx.x; j < n; j += 256) {
+    const int cl = j / KK, tap = j - cl * KK;
+    permute_tile[cl * kkp + tap] = mode == 0 ? src[j] : w[((size_t)(c0 + cl) * O + o) * KK + tap];
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < 64 * KK; j += 256) {
+    const int tap = j >> 6, cl = j & 63;
+    if (cl < nc) wp[((size_t)o * KK + tap) * C + c0 + cl] = permute_tile[cl * kkp + tap];
+  }
 }
 // mode 1 for up to four pixel classes at once: blockIdx.y = class
 struct PermuteBatch {
@@ -596,6 +620,20 @@ static int get_table(DeviceCtx* ctx, const ConvGeom& g, int mode, const PixelCla
   return LNN_OK;
 }
 
+// Weights into a permuted layout (modes as in permute_one).
+static int launch_permute(DeviceCtx* ctx, float* wp, const float* W, const ConvGeom& g, int mode, const PixelClass& pc) {
+  if (mode != 1 && g.KK <= kPermuteMaxKK) {
+    const int blocks = g.O * ((g.C + 63) / 64);
+    hipLaunchKernelGGL(permute_weights_tiled, dim3(blocks), dim3(256), (size_t)64 * (g.KK | 1) * sizeof(float), ctx->stream,
+                       wp, W, g.O, g.C, g.KK, mode);
+  } else {
+    const int n = g.O * g.C * (mode == 1 ? pc.nkh * pc.nkw : g.KK);
+    hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, wp, W, g.O, g.C, g.KK, mode, g, pc);
+  }
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
 // Channel-permuted copy of the weights in the library's scratch buffer (valid
 // until the next call that uses scratch; the stream orders it before its reader).
 static int permuted_weights(DeviceCtx* ctx, const ConvGeom& g, const float* W, int mode, const PixelClass& pc,
@@ -607,9 +645,8 @@ static int permuted_weights(DeviceCtx* ctx, const ConvGeom& g, const float* W, i
   int st = ensure_workspace(ctx, *used + (size_t)ctx->cus * 32768 * sizeof(float));
   if (st != LNN_OK) return st;
   if (n > 0) {
-    hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream,
-                       static_cast<float*>(ctx->ws), W, g.O, g.C, g.KK, mode, g, pc);
-    LNN_HIP(hipGetLastError());
+    st = launch_permute(ctx, static_cast<float*>(ctx->ws), W, g, mode, pc);
+    if (st != LNN_OK) return st;
   }
   *out = static_cast<const float*>(ctx->ws);
   return LNN_OK;
@@ -665,10 +702,10 @@ static size_t plan_tiles(ConvArgs& a, long long slots, bool allow_tail = false) 
   // Few output tiles (small images, deep layers): a workgroup's share would be a sliver of a sub-tile and
   // most of its time data movement.  Cut the output into full sub-tiles instead and split K over the
   // workgroups that are left, as wgrad does.
-  const int chunk = 2 * NTMAX;
+  const int chunk = (2 * NTMAX) >> LNN_KSPLIT_HALF > 1 ? (2 * NTMAX) >> LNN_KSPLIT_HALF : 2;
   const long long chunks = (total + chunk - 1) / chunk;
   const int nkt = (a.K + BK - 1) / BK;
-  if (total < slots * (chunk / 2 + 1) && chunks * 2 <= slots && nkt >= 16) {
+  if (total < slots * (NTMAX + 1) && chunks * 2 <= slots && nkt >= 16) {
     long long s = slots / chunks;
     if (s > nkt / 8) s = nkt / 8;
     if (s > 1) {

@@ -25,11 +25,7 @@ int launch_permute_weights(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float
   if (!W || !Wp) return set_error(LNN_ERR_INVALID, "conv2d_permute_weights: null pointer");
   if (w_layout != LNN_W_OIHW && w_layout != LNN_W_IOHW) return set_error(LNN_ERR_INVALID, "conv2d_permute_weights: unknown layout");
   if (!aligned16(Wp)) return set_error(LNN_ERR_INVALID, "conv2d_permute_weights: the destination must be 16-byte aligned");
-  const int n = g.O * g.C * g.KK;
-  hipLaunchKernelGGL(permute_weights, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, Wp, W, g.O, g.C, g.KK,
-                     w_layout == LNN_W_OIHW ? 0 : 2, g, PixelClass{});
-  LNN_HIP(hipGetLastError());
-  return LNN_OK;
+  return launch_permute(ctx, Wp, W, g, w_layout == LNN_W_OIHW ? 0 : 2, PixelClass{});
 }
 
 int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta,

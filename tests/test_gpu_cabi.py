@@ -389,6 +389,16 @@ def test_conv_dgrad_on_forward_permuted_weights_integer_exact(hip):
             assert np.array_equal(Y.get(), ry), (C, O, s, d, ks, padding)
         cnt += 1
     assert cnt > 500
+    # the copy itself for both source layouts: more taps than the tiled copy holds in LDS, an even tap count,
+    # channel counts off and on the 64-channel blocks
+    for (O, C, kh, kw) in [(3, 70, 15, 15), (5, 64, 2, 4), (2, 130, 7, 7), (33, 4, 3, 3)]:
+        desc, _ = _desc(hip, (1, C, 16, 16), (O, C, kh, kw), 1, 1, 'same')
+        w = rs.randint(-9, 10, size=(O, C, kh, kw)).astype(np.float32)
+        want = w.reshape(O, C, kh * kw).transpose(0, 2, 1)
+        for layout, src in ((hip.W_OIHW, w), (hip.W_IOHW, np.ascontiguousarray(w.transpose(1, 0, 2, 3)))):
+            Wsrc, Wp = DevArr(hip, src), DevArr(hip, shape=(O, kh * kw, C), fill=np.nan)
+            hip.conv2d_permute_weights(0, desc, Wsrc.ptr, layout, Wp.ptr)
+            assert np.array_equal(Wp.get(), want), (O, C, kh, kw, layout)
     # geometries whose kernels do not read Wp refuse the *_pw entry points
     desc, _ = _desc(hip, (1, 3, 8, 8), (32, 3, 3, 3), 1, 1, 'same')
     assert not hip.conv2d_weights_plan(desc, hip.PASS_DGRAD) and not hip.conv2d_weights_plan(desc, hip.PASS_FWD)
