@@ -196,8 +196,61 @@ __device__ __forceinline__ void reduce_body4(float* out, const float* part, cons
     out[o] = a.beta ? out[o] + t : t;
   }
 }
+// ... and with at most kFewSlices slices: nothing to gain from lanes striding over the slices (most of them would
+// idle), so every thread adds up the slices of four consecutive elements itself, all its loads in flight together,
+// and a block covers 1024 elements, which leave through LDS so that consecutive lanes store consecutive elements.
+// The additions are the ones reduce_body4 makes, in the same order.
+constexpr int kFewSlices = 8;
+template <int NS>
+__device__ __forceinline__ f32x4 sum_slices(const float* part, size_t n, int i4, int ns) {
+  f32x4 v[NS];
+#pragma unroll
+  for (int k = 0; k < NS; ++k) v[k] = *reinterpret_cast<const f32x4*>(&part[(size_t)(k < ns ? k : 0) * n + i4]);
+  f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+  const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int k = 0; k < NS; ++k) s += k < ns ? v[k] : zero;
+  return s;
+}
+__device__ __forceinline__ void reduce_body4_few(float* out, const float* part, const ReduceArgs& a) {
+  __shared__ float red[1024];
+  const int i4 = ((int)blockIdx.x * 256 + (int)threadIdx.x) * 4;
+  f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (i4 < a.n) {
+    const uint32_t m = a.dN.div((uint32_t)i4), col = (uint32_t)i4 - m * (uint32_t)a.ncols;
+    const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
+    const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+    // the slice count of the problem is uniform: one straight run of loads per count; a unit of the last chunk,
+    // which may have fewer slices, reads slice 0 again in their place and adds zeros
+    switch (a.slices) {
+      case 2: s = sum_slices<2>(part, (size_t)a.n, i4, ns); break;
+      case 3: s = sum_slices<3>(part, (size_t)a.n, i4, ns); break;
+      case 4: s = sum_slices<4>(part, (size_t)a.n, i4, ns); break;
+      case 5: s = sum_slices<5>(part, (size_t)a.n, i4, ns); break;
+      case 6: s = sum_slices<6>(part, (size_t)a.n, i4, ns); break;
+      case 7: s = sum_slices<7>(part, (size_t)a.n, i4, ns); break;
+      default: s = sum_slices<8>(part, (size_t)a.n, i4, ns); break;
+    }
+  }
+  *reinterpret_cast<f32x4*>(&red[4 * threadIdx.x]) = s;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = (int)threadIdx.x + 256 * j, i = (int)blockIdx.x * 1024 + e;
+    if (i < a.n) {
+      float t = red[e];
+      const uint32_t m = a.dN.div((uint32_t)i), col = (uint32_t)i - m * (uint32_t)a.ncols;
+      const uint32_t o = a.om.col(col) + m * (uint32_t)a.om.ld;
+      if (a.post.any()) t = a.post.apply(t, a.post.bias != nullptr ? a.post.bias[m] : 0.0f);
+      out[o] = a.beta ? out[o] + t : t;
+    }
+  }
+}
+// elements per block of the 128-bit reductions
+__host__ __device__ inline int reduce4_block(const ReduceArgs& a) { return a.slices <= kFewSlices ? 1024 : 128; }
 __global__ __launch_bounds__(256) void reduce_partials4(float* out, const float* part, ReduceArgs a) {
-  reduce_body4(out, part, a);
+  if (a.slices <= kFewSlices) reduce_body4_few(out, part, a);
+  else reduce_body4(out, part, a);
 }
 
 // The reductions of the pixel classes of one strided dgrad in one launch: blockIdx.y = class.
@@ -210,9 +263,10 @@ struct ReduceBatch {
 };
 __global__ __launch_bounds__(256) void reduce_partials_batch(ReduceBatch b) {
   const int c = blockIdx.y;
-  const int per_block = b.vec[c] ? 128 : 32;
+  const int per_block = b.vec[c] ? reduce4_block(b.r[c]) : 32;
   if ((long long)blockIdx.x * per_block >= b.r[c].n) return;   // the whole block leaves together
-  if (b.vec[c]) reduce_body4(b.out[c], b.part[c], b.r[c]);
+  if (b.vec[c] && b.r[c].slices <= kFewSlices) reduce_body4_few(b.out[c], b.part[c], b.r[c]);
+  else if (b.vec[c]) reduce_body4(b.out[c], b.part[c], b.r[c]);
   else reduce_body(b.out[c], b.part[c], b.r[c]);
 }
 
@@ -675,7 +729,7 @@ template <int PASS, int WM>
 static int launch_reduce(DeviceCtx* ctx, const ConvArgs& a, float* final_out, int final_beta) {
   const ReduceArgs r = reduce_args<PASS, WM>(a, final_beta);
   if (a.Ncols % 4 == 0)   // partial buffers start 256-byte aligned
-    hipLaunchKernelGGL(reduce_partials4, dim3((r.n + 127) / 128), dim3(256), 0, ctx->stream, final_out,
+    hipLaunchKernelGGL(reduce_partials4, dim3((r.n + reduce4_block(r) - 1) / reduce4_block(r)), dim3(256), 0, ctx->stream, final_out,
                        static_cast<const float*>(a.Out), r);
   else
     hipLaunchKernelGGL(reduce_partials, dim3((r.n + 31) / 32), dim3(256), 0, ctx->stream, final_out,
@@ -933,7 +987,8 @@ static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_
       rb.out[nr] = final_out[i];
       rb.part[nr] = cls[i].Out;
       rb.vec[nr] = cls[i].Ncols % 4 == 0;
-      const unsigned blocks = (unsigned)((rb.r[nr].n + (rb.vec[nr] ? 127 : 31)) / (rb.vec[nr] ? 128 : 32));
+      const unsigned per_block = rb.vec[nr] ? (unsigned)reduce4_block(rb.r[nr]) : 32u;
+      const unsigned blocks = ((unsigned)rb.r[nr].n + per_block - 1) / per_block;
       gx = blocks > gx ? blocks : gx;
       if (++nr == kMaxReduceBatch) flush();
     }
