@@ -129,6 +129,14 @@ int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, con
 #define LNN_DGRAD_PATH_MFMA_TAP 1   /* implicit GEMM, tap-major K over channel-permuted weights (O % 32 == 0) */
 #define LNN_DGRAD_PATH_VECTOR 2     /* C <= 4: vector-ALU kernel, all pixel classes of a 32 x 32 tile per block */
 int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* path, int32_t* tile_info);
+/* Which kernel family lnn_conv2d_fwd_f32 / lnn_conv2d_fwd_bias_act_f32 use for a geometry on a device with
+ * `compute_units` compute units.  Host arithmetic only: works without a device.  No counterpart in the reference,
+ * whose forward pass always runs unfold + GeMM (conv2D.py:39-42); it lets a caller, or a test, see which code a
+ * shape exercises. */
+#define LNN_FWD_PATH_IMPLICIT_GEMM 0 /* implicit GEMM on the matrix cores, operands gathered tile by tile */
+#define LNN_FWD_PATH_STEM_PATCH 1    /* 3 input channels, 33-64 output channels, 3x3 / 5x5 / 7x7: MFMA operands read
+                                        from an input patch in LDS (problems with at least 4 tiles per compute unit) */
+int lnn_conv2d_fwd_path(const lnn_conv2d_desc* d, int compute_units, int* path);
 /* dW (+)= wgrad(X, dY)                   conv2D.py:52-54 (the reference always accumulates) */
 int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
                          float* dW, int beta);

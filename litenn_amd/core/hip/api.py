@@ -76,6 +76,7 @@ SIGNATURES = {
     'lnn_conv2d_dgrad_pw_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_wgrad_iohw_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_wgrad_noalloc_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
+    'lnn_conv2d_fwd_path': [ctypes.POINTER(ConvDesc), _c_int, ctypes.POINTER(_c_int)],
     'lnn_conv2d_dgrad_path': [ctypes.POINTER(ConvDesc), _c_int, _c_int, ctypes.POINTER(_c_int), _i32arr],
     'lnn_unfold2d_f32': [_c_int] + [_c_int] * 14 + [_ptr, _ptr, _c_int],
     'lnn_transpose_f32': [_c_int, _c_int, _i32arr, _i32arr, _ptr, _ptr, _c_int],
@@ -263,6 +264,17 @@ def conv2d_wgrad_noalloc(dev, desc, X, dY, dW, beta=1):
     """conv2d_wgrad without device allocation: scratch is a fixed array inside the library (NOALLOC_SCRATCH_BYTES);
     problems that need more raise ERR_UNSUPPORTED."""
     check(lib.lnn_conv2d_wgrad_noalloc_f32(dev, ctypes.byref(desc), X, dY, dW, int(beta)))
+
+
+FWD_PATH_IMPLICIT_GEMM, FWD_PATH_STEM_PATCH = 0, 1
+
+
+def conv2d_fwd_path(desc, compute_units):
+    """The kernel family conv2d_fwd picks for this geometry on a device with that many compute units (host
+    arithmetic, needs no device)."""
+    path = _c_int(-1)
+    check(lib.lnn_conv2d_fwd_path(ctypes.byref(desc), int(compute_units), ctypes.byref(path)))
+    return path.value
 
 
 DGRAD_PATH_MFMA_TABLE, DGRAD_PATH_MFMA_TAP, DGRAD_PATH_VECTOR = 0, 1, 2

@@ -49,6 +49,11 @@ int launch_gemm(DeviceCtx* ctx, int ta, int tb, int batch, int M, int N, int K, 
 // Wp: the weights in the permuted layout (made by launch_permute_weights), or null; W may be null when Wp is given
 int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta,
                     const float* bias, int act, float slope, const float* Wp = nullptr);
+// image stems (3 input channels, 33-64 output channels, 3x3 / 5x5 / 7x7, enough tiles): forward from an input patch in LDS
+bool stem_fwd_applies(const lnn_conv2d_desc* d, int compute_units);
+int launch_stem_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta,
+                    const float* bias, int act, float slope);
+int conv_fwd_path(const lnn_conv2d_desc* d, int compute_units, int* path);
 int conv_weights_plan(const lnn_conv2d_desc* d, int pass, int* yes);
 int launch_permute_weights(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* W, int w_layout, float* Wp);
 int launch_dw_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* K, float* Y, int beta);

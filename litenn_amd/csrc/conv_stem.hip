@@ -1,0 +1,267 @@
+// Convolution forward pass for image stems: three input channels, 33-64 output channels, a small dense kernel.
+//
+// The implicit-GEMM passes gather the B operand element by element, with a range test per element; with K = C*KH*KW
+// of only a few K steps that address arithmetic costs as much as the matrix instructions.  Here a block brings the
+// input patch under its 256 output pixels to LDS once (C planes of R rows), and the B operand of every MFMA is read
+// straight from that patch: the address of tap k of a lane's pixel is the pixel's base address plus a constant known
+// at compile time, so the K loop is nothing but ds_read_b32 with immediate offsets and MFMAs.  K is not padded to a
+// multiple of 32 either: v_mfma_f32_32x32x2_f32 takes two k per instruction, so K = 147 costs 74 steps.
+// A block lays the weights out in LDS once and walks over tiles; the next tile's patch travels global -> LDS (no
+// registers) into a second buffer while the current tile is computed.
+#include <utility>
+
+#include "common.hpp"
+
+namespace lnn {
+namespace {
+
+// LDS row pitch of the patch.  A 32-lane block of pixels is one tile row (TW = 32) or two (TW = 16); with two, the
+// second row's addresses should fall into the banks the first leaves free: S*PW = 16*S (mod 64).
+constexpr int stem_pitch(int qn, int s, int tw) {
+  if (tw == 32) return qn;
+  int pw = qn;
+  while ((s * pw) % 64 != (16 * s) % 64) ++pw;
+  return pw;
+}
+// Two blocks share a compute unit: 80 KB of LDS each.
+constexpr int kStemLdsFloats = 80 * 1024 / 4;
+
+template <int KH_, int KW_, int S_, int TW_>
+struct StemCfg {
+  static constexpr int C = 3, KH = KH_, KW = KW_, S = S_, TW = TW_, TH = 256 / TW_;
+  static constexpr int K = C * KH * KW, T = (K + 1) / 2;   // MFMA steps: k = 2t and 2t + 1
+  static constexpr int R = (TH - 1) * S + KH;              // patch rows
+  static constexpr int QN = (TW - 1) * S + KW;             // patch columns
+  // weights in LDS: [t][row block][k parity][32 rows], steps 129 floats apart: a block fills them reading W in memory
+  // order (lanes along k), and the odd pitch spreads those writes over the banks
+  static constexpr int WPITCH = 129;
+  static constexpr int WL = (T * WPITCH + 3) & ~3;
+  // the conflict-free pitch where two patch buffers of it fit beside the weights, else the next multiple of 8
+  static constexpr int PW_FREE = stem_pitch(QN, S, TW);
+  static constexpr int PW = WL + 2 * ((C * R * PW_FREE + 63) & ~63) <= kStemLdsFloats ? PW_FREE : (QN + 7) & ~7;
+  static constexpr int PLANE = R * PW;
+  static constexpr int CHUNKS = (C * PLANE + 63) / 64;     // global -> LDS transfers (64 floats each) per patch
+  static constexpr int PATCH = CHUNKS * 64;
+  static constexpr int PER_WAVE = (CHUNKS + 3) / 4;
+  static constexpr int LDS_FLOATS = WL + 2 * PATCH;
+  // where tap k = (c, kh, kw) lies relative to a pixel's window origin
+  static constexpr int off(int k) { return (k / (KH * KW)) * PLANE + ((k % (KH * KW)) / KW) * PW + k % KW; }
+  // the odd k of step t relative to the even one: 1 inside a kernel row, else the jump to the next row or plane;
+  // 0 for the padding k behind an odd K (its weight is zero, and it rereads an element of the pixel's own window)
+  static constexpr int delta(int t) { return 2 * t + 1 < K ? off(2 * t + 1) - off(2 * t) : 0; }
+  static constexpr int D_ROW = PW - (KW - 1), D_PLANE = PLANE - ((KH - 1) * PW + KW - 1);
+};
+
+struct StemArgs {
+  const float* X;
+  const float* W;
+  float* Y;
+  int N, IH, IW, O, OH, OW, PADT, PADL, tiles_w, tiles_h, tiles, beta;
+  uint32_t bytesX;
+  PostOp post;
+};
+
+// The operands of step T: two weights (row blocks 0 and 1) and two pixels (pixel blocks 0 and 1) per lane.
+template <class Cfg, int T>
+__device__ __forceinline__ void stem_load(const float* wlane, const float* patch, const int (&b1)[2], const int (&br)[2],
+                                          const int (&bp)[2], const int (&b0)[2], float (&a)[2], float (&b)[2]) {
+  constexpr int o0 = Cfg::off(2 * T), d = Cfg::delta(T);
+  a[0] = wlane[T * Cfg::WPITCH];
+  a[1] = wlane[T * Cfg::WPITCH + 64];
+#pragma unroll
+  for (int pb = 0; pb < 2; ++pb) {
+    const int base = d == 1 ? b1[pb] : (d == Cfg::D_ROW ? br[pb] : (d == Cfg::D_PLANE ? bp[pb] : b0[pb]));
+    b[pb] = patch[base + o0];
+  }
+}
+// Step T: the next step's operands are requested first, then this step's four MFMAs go out - an LDS read takes about
+// as long as two MFMAs, and a wavefront that asked only when it needed the values would idle the pipe every step.
+// Every step is a scheduling region of its own so that this order survives.
+template <class Cfg, int T>
+__device__ __forceinline__ void stem_step(const float* wlane, const float* patch, const int (&b1)[2], const int (&br)[2],
+                                          const int (&bp)[2], const int (&b0)[2], float (&a)[2][2], float (&b)[2][2],
+                                          f32x16 (&acc)[2][2]) {
+  if (T + 1 < Cfg::T) stem_load<Cfg, (T + 1 < Cfg::T ? T + 1 : T)>(wlane, patch, b1, br, bp, b0, a[(T + 1) & 1], b[(T + 1) & 1]);
+#pragma unroll
+  for (int pb = 0; pb < 2; ++pb) {
+    acc[0][pb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[T & 1][0], b[T & 1][pb], acc[0][pb], 0, 0, 0);
+    acc[1][pb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[T & 1][1], b[T & 1][pb], acc[1][pb], 0, 0, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // the LDS reads (the compiler may have paired some)
+  __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);   // then the MFMAs
+  __builtin_amdgcn_sched_barrier(0);
+}
+template <class Cfg, int... Ts>
+__device__ __forceinline__ void stem_steps(std::integer_sequence<int, Ts...>, const float* wlane, const float* patch,
+                                           const int (&b1)[2], const int (&br)[2], const int (&bp)[2], const int (&b0)[2],
+                                           f32x16 (&acc)[2][2]) {
+  float a[2][2], b[2][2];
+  stem_load<Cfg, 0>(wlane, patch, b1, br, bp, b0, a[0], b[0]);
+  __builtin_amdgcn_sched_barrier(0);
+  (stem_step<Cfg, Ts>(wlane, patch, b1, br, bp, b0, a, b, acc), ...);
+}
+
+// A block of 256 threads walks over tiles of TH x TW output pixels (tile = blockIdx.x, + gridDim.x, ...), all (at
+// most 64) output channels each.  (Handing tiles out through a counter instead made no difference.)
+// Wavefront w owns the pixel blocks 2w and 2w + 1 of a tile (32 pixels each, in row-major tile order) and both row
+// blocks.
+template <class Cfg>
+__global__ __launch_bounds__(256, 2) void stem_fwd_kernel(StemArgs a) {
+  __shared__ __attribute__((aligned(16))) float smem[Cfg::LDS_FLOATS];
+  float* wl = smem;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, i = lane & 31, h = lane >> 5;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const rsrc_t rx = make_rsrc(a.X, a.bytesX);
+  constexpr uint32_t OOB = 0x80000000u;
+
+  // Patch transfers: chunk j of this wavefront fills LDS floats [(w + 4j)*64, +64) of a patch buffer; a lane's
+  // float is element (c, r, q) of the patch (or pitch padding / the tail of the last chunk: never read, zeros).
+  // rel: its offset in X relative to the patch origin; rq: r and q for the range tests of each tile.
+  int rel[Cfg::PER_WAVE], rq[Cfg::PER_WAVE];
+#pragma unroll
+  for (int j = 0; j < Cfg::PER_WAVE; ++j) {
+    const int e = (w + 4 * j) * 64 + lane;
+    const int c = e / Cfg::PLANE, rem = e - c * Cfg::PLANE, r = rem / Cfg::PW, q = rem - r * Cfg::PW;
+    const bool used = e < Cfg::C * Cfg::PLANE && q < Cfg::QN;
+    rel[j] = (c * a.IH + r) * a.IW + q;
+    rq[j] = used ? (r | (q << 16)) : -1;
+  }
+  auto request = [&](int tile, float* patch) {
+    const int tw = tile % a.tiles_w, rest = tile / a.tiles_w, th = rest % a.tiles_h, n = rest / a.tiles_h;
+    const int ih0 = th * Cfg::TH * Cfg::S - a.PADT, iw0 = tw * Cfg::TW * Cfg::S - a.PADL;
+    const int origin = (n * Cfg::C * a.IH + ih0) * a.IW + iw0;   // may be negative; valid elements are not
+#pragma unroll
+    for (int j = 0; j < Cfg::PER_WAVE; ++j) {
+      if (w + 4 * j < Cfg::CHUNKS) {   // wave-uniform
+        const int ih = ih0 + (rq[j] & 0xffff), iw = iw0 + (rq[j] >> 16);
+        const bool ok = rq[j] >= 0 && (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
+        buf_load_lds4(rx, patch + (w + 4 * j) * 64, ok ? (uint32_t)(origin + rel[j]) * 4u : OOB, 0);
+      }
+    }
+  };
+
+  request((int)blockIdx.x, smem + Cfg::WL);
+  // weights: element (o, k) of W[O][K] goes to wl[k/2][o/32][k%2][o%32]; zeros for the rows past O and the padding k
+  constexpr int KP = 2 * Cfg::T;
+  constexpr int WITER = (64 * KP + 255) / 256;
+  float wv[WITER];
+#pragma unroll
+  for (int it = 0; it < WITER; ++it) {   // all loads in flight together
+    const int e = tid + 256 * it, o = e / KP, k = e - o * KP;
+    wv[it] = (o < a.O && k < Cfg::K) ? a.W[o * Cfg::K + k] : 0.0f;
+  }
+#pragma unroll
+  for (int it = 0; it < WITER; ++it) {
+    const int e = tid + 256 * it, o = e / KP, k = e - o * KP;
+    if (e < 64 * KP) wl[(k >> 1) * Cfg::WPITCH + (o >> 5) * 64 + (k & 1) * 32 + (o & 31)] = wv[it];
+  }
+
+  // lane bases inside a patch: pixel (row, col) of the tile, plus the odd k's displacement for each kind of step
+  int b1[2], br[2], bp[2], b0[2];
+#pragma unroll
+  for (int pb = 0; pb < 2; ++pb) {
+    const int pl = (2 * w + pb) * 32 + i, row = pl / Cfg::TW, col = pl % Cfg::TW;
+    b0[pb] = row * Cfg::S * Cfg::PW + col * Cfg::S;
+    b1[pb] = b0[pb] + h;
+    br[pb] = b0[pb] + h * Cfg::D_ROW;
+    bp[pb] = b0[pb] + h * Cfg::D_PLANE;
+  }
+
+  int cur = 0;
+  for (int tile = (int)blockIdx.x; tile < a.tiles; tile += (int)gridDim.x, cur ^= 1) {
+    // this tile's patch has landed (and this thread's stores of the last tile have left); behind the barrier every
+    // wavefront is done reading the other buffer, which the next tile's patch may now overwrite
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const float* patch = smem + Cfg::WL + cur * Cfg::PATCH;
+    if (tile + (int)gridDim.x < a.tiles) request(tile + (int)gridDim.x, smem + Cfg::WL + (cur ^ 1) * Cfg::PATCH);
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mb][pb][r] = 0.0f;
+    stem_steps<Cfg>(std::make_integer_sequence<int, Cfg::T>{}, wl + h * 32 + i, patch, b1, br, bp, b0, acc);
+
+    // Element r of an accumulator: channel 8*(r/4) + 4*h + r%4 of the row block, pixel i of the pixel block.  Stores
+    // go through a descriptor of this image's O planes: the lane's part of the address (pixel, and 4*h channels) is
+    // computed once per pixel block, the rest of the channel index travels in the scalar offset, and channels past O
+    // fall outside the descriptor and are dropped - no vector arithmetic per store.
+    const int tw = tile % a.tiles_w, rest = tile / a.tiles_w, th = rest % a.tiles_h, n = rest / a.tiles_h;
+    const int ohw = a.OH * a.OW;
+    const rsrc_t ry = make_rsrc(a.Y + (size_t)n * a.O * ohw, (uint32_t)(a.O * ohw) * 4u);
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+      const int pl = (2 * w + pb) * 32 + i, oh = th * Cfg::TH + pl / Cfg::TW, ow = tw * Cfg::TW + pl % Cfg::TW;
+      const uint32_t voff = (oh < a.OH && ow < a.OW) ? (uint32_t)(oh * a.OW + ow + 4 * h * ohw) * 4u : OOB;
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int mc = mb * 32 + 8 * (r >> 2) + (r & 3);   // + 4*h: this lane's channel
+          const int soff = mc * ohw * 4;
+          float v = acc[mb][pb][r];
+          if (a.post.any()) {
+            const int m = mc + 4 * h;
+            v = a.post.apply(v, (a.post.bias != nullptr && m < a.O) ? a.post.bias[m] : 0.0f);
+          }
+          if (a.beta) v += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ry, (int)voff, soff, 0));
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ry, (int)voff, soff, 0);
+        }
+    }
+  }
+}
+
+template <int KH, int KW, int S>
+int launch_stem_shape(DeviceCtx* ctx, StemArgs& a) {
+  // the tile shape that covers the output plane with less overhang
+  auto count = [&](int tw_) { return (long long)((a.OW + tw_ - 1) / tw_) * ((a.OH + 256 / tw_ - 1) / (256 / tw_)); };
+  const bool wide = count(32) <= count(16);
+  using Wide = StemCfg<KH, KW, S, 32>;
+  using Square = StemCfg<KH, KW, S, 16>;
+  static_assert(Wide::LDS_FLOATS <= kStemLdsFloats && Square::LDS_FLOATS <= kStemLdsFloats, "two blocks per compute unit");
+  const int tw_ = wide ? 32 : 16, th_ = 256 / tw_;
+  a.tiles_w = (a.OW + tw_ - 1) / tw_;
+  a.tiles_h = (a.OH + th_ - 1) / th_;
+  const long long tiles = (long long)a.N * a.tiles_w * a.tiles_h;
+  if (tiles > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
+  a.tiles = (int)tiles;
+  const long long blocks = tiles < 2ll * ctx->cus ? tiles : 2ll * ctx->cus;   // two blocks per compute unit
+  if (wide) hipLaunchKernelGGL((stem_fwd_kernel<Wide>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((stem_fwd_kernel<Square>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
+}  // namespace
+
+// Geometries the patch kernel takes.  With fewer than four tiles per compute unit the implicit-GEMM pass, which cuts
+// the work more finely, is as fast or faster (16 x 3 x 128 x 128, 5x5 stride 2, 256 tiles: 23 against 18 us).
+bool stem_fwd_applies(const lnn_conv2d_desc* d, int compute_units) {
+  if (d->C != 3 || d->O <= 32 || d->O > 64 || d->dilation != 1 || d->KH != d->KW) return false;
+  const int k = d->KH, s = d->stride;
+  if (!((k == 7 && s == 2) || (k == 5 && s == 2) || (k == 3 && (s == 1 || s == 2)))) return false;
+  return (long long)d->N * (((long long)d->OH * d->OW + 255) / 256) >= 4ll * compute_units;
+}
+
+// Y (+)= conv(X, W) with the bias / activation epilogue, for the geometries stem_fwd_applies() accepts
+int launch_stem_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta,
+                    const float* bias, int act, float slope) {
+  StemArgs a;
+  a.X = X; a.W = W; a.Y = Y;
+  a.N = d->N; a.IH = d->IH; a.IW = d->IW; a.O = d->O; a.OH = d->OH; a.OW = d->OW; a.PADT = d->PADT; a.PADL = d->PADL;
+  a.beta = beta ? 1 : 0;
+  a.bytesX = (uint32_t)((uint64_t)d->N * d->C * d->IH * d->IW * 4);
+  a.post = PostOp{bias, act, slope};
+  const int k = d->KH, s = d->stride;
+  if (k == 7 && s == 2) return launch_stem_shape<7, 7, 2>(ctx, a);
+  if (k == 5 && s == 2) return launch_stem_shape<5, 5, 2>(ctx, a);
+  if (k == 3 && s == 1) return launch_stem_shape<3, 3, 1>(ctx, a);
+  if (k == 3 && s == 2) return launch_stem_shape<3, 3, 2>(ctx, a);
+  return set_error(LNN_ERR_INVALID, "conv2d_fwd: not a stem geometry");
+}
+
+}  // namespace lnn

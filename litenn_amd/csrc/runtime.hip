@@ -368,6 +368,10 @@ int lnn_conv2d_wgrad_iohw_f32(int dev, const lnn_conv2d_desc* d, const float* X,
   return launch_conv_wgrad(ctx, d, X, dY, dW, beta, 1);
 }
 
+int lnn_conv2d_fwd_path(const lnn_conv2d_desc* d, int compute_units, int* path) {
+  return conv_fwd_path(d, compute_units, path);
+}
+
 int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* path, int32_t* tile_info) {
   return conv_dgrad_path(d, beta, compute_units, path, tile_info);
 }

@@ -450,6 +450,75 @@ def test_conv_remainder_units_cut_along_k_integer_exact(hip):
         assert np.array_equal(Y.get(), np.where(pre >= 0, pre, 0.25 * pre).astype(np.float32)), (xs, ws)
 
 
+def test_conv_stem_forward_from_lds_patch_integer_exact(hip):
+    """Three input channels, 33-64 output channels, 3x3 (stride 1 and 2), 5x5 and 7x7 (stride 2), at least four
+    tiles of 256 pixels per compute unit: the forward pass reads its B operand from an input patch in LDS (tiles of
+    8 x 32 or 16 x 16 output pixels, whichever covers the plane with less overhang; blocks take tiles from a
+    counter).  Planes that are whole tiles and ragged in both directions, every padding kind including asymmetric
+    and none, '=' and '+=', bias and leaky ReLU in the epilogue; lnn_conv2d_fwd_path confirms that every case reaches
+    the kernel.  Batches this large are slow on the CPU oracle: the first and the last image are checked against it,
+    all images against the implicit-GEMM pass run on part of the batch at a time (too few tiles for the patch
+    kernel), which the other tests pin to the oracle.  Exact on small integers.  Neighbouring geometries (other channel counts,
+    dilation, kernel shapes, few tiles) go the implicit-GEMM way."""
+    rs = np.random.RandomState(64)
+    cus = hip.device_info(0)['compute_units']
+    for (k, s) in [(7, 2), (5, 2), (3, 1), (3, 2)]:
+        for (oh, ow, O, padding) in [(64, 64, 64, 'same'), (61, 53, 48, 'same'), (70, 40, 33, 'valid'),
+                                     (93, 90, 64, (1, 0, 2, 3)), (25, 27, 40, 'same'), (130, 34, 64, 0)]:
+            ih, iw = oh * s, ow * s
+            if padding in ('valid', 0):
+                ih, iw = ih + k - 1, iw + k - 1
+            ci = info_conv2d(ih, iw, k, k, s, 1, padding)
+            n = -(-4 * cus // ((ci.OH * ci.OW + 255) // 256)) + 1
+            xs, ws = (n, 3, ih, iw), (O, 3, k, k)
+            desc, _ = _desc(hip, xs, ws, s, 1, padding)
+            assert hip.conv2d_fwd_path(desc, cus) == hip.FWD_PATH_STEM_PATCH, (xs, ws, s, padding)
+            say(f'stem forward x={xs} w={ws} s={s} pad={padding} -> y {ci.OH}x{ci.OW}')
+            x = rs.randint(-3, 4, size=xs).astype(np.float32)
+            w = rs.randint(-3, 4, size=ws).astype(np.float32)
+            b = rs.randint(-3, 4, size=(O,)).astype(np.float32)
+            X, W, B = DevArr(hip, x), DevArr(hip, w), DevArr(hip, b)
+            # the same convolution in batches just too small for the patch kernel
+            ref = np.empty((n, O, ci.OH, ci.OW), np.float32)
+            step = max(1, (4 * cus - 1) // ((ci.OH * ci.OW + 255) // 256))
+            for i0 in range(0, n, step):
+                m = min(step, n - i0)
+                dpart, _ = _desc(hip, (m,) + xs[1:], ws, s, 1, padding)
+                assert hip.conv2d_fwd_path(dpart, cus) == hip.FWD_PATH_IMPLICIT_GEMM
+                Xp, Yp = DevArr(hip, x[i0:i0 + m]), DevArr(hip, shape=(m, O, ci.OH, ci.OW), fill=np.nan)
+                hip.conv2d_fwd(0, dpart, Xp.ptr, W.ptr, Yp.ptr, 0)
+                ref[i0:i0 + m] = Yp.get()
+            for img in (0, n - 1):
+                assert np.array_equal(ref[img:img + 1], conv2d_fwd(x[img:img + 1], w, s, 1, padding, dtype=np.float32))
+            for beta, fill in ((0, np.nan), (1, -2.0)):
+                Y = DevArr(hip, shape=ref.shape, fill=fill)
+                hip.conv2d_fwd(0, desc, X.ptr, W.ptr, Y.ptr, beta)
+                assert np.array_equal(Y.get() - (-2.0 if beta else 0.0), ref), (xs, ws, s, padding, beta)
+            Y = DevArr(hip, shape=ref.shape, fill=np.nan)
+            hip.conv2d_fwd_bias_act(0, desc, X.ptr, W.ptr, B.ptr, hip.ACT_LEAKY_RELU, 0.25, Y.ptr)
+            pre = ref + b[None, :, None, None]
+            assert np.array_equal(Y.get(), np.where(pre >= 0, pre, 0.25 * pre).astype(np.float32)), (xs, ws, s, padding)
+    # neighbours of the stem geometries stay on the other kernels
+    for xs, ws, s, d in [((70, 3, 128, 128), (32, 3, 7, 7), 2, 1), ((70, 3, 64, 64), (96, 3, 3, 3), 1, 1),
+                         ((70, 4, 128, 128), (64, 4, 5, 5), 2, 1), ((70, 3, 64, 64), (64, 3, 3, 3), 1, 2),
+                         ((70, 3, 64, 64), (64, 3, 3, 5), 1, 1), ((70, 3, 64, 64), (64, 3, 5, 5), 1, 1),
+                         ((8, 3, 128, 128), (64, 3, 7, 7), 2, 1)]:
+        desc, _ = _desc(hip, xs, ws, s, d, 'same')
+        assert hip.conv2d_fwd_path(desc, 256) == hip.FWD_PATH_IMPLICIT_GEMM, (xs, ws, s, d)
+    # float data at a stem's real size against the fp64 restatement (first and last image)
+    xs, ws = (24, 3, 224, 224), (64, 3, 7, 7)
+    desc, ci = _desc(hip, xs, ws, 2, 1, 'same')
+    assert cus != 256 or hip.conv2d_fwd_path(desc, cus) == hip.FWD_PATH_STEM_PATCH
+    x = rs.uniform(-1, 1, size=xs).astype(np.float32)
+    w = rs.uniform(-1, 1, size=ws).astype(np.float32)
+    X, W = DevArr(hip, x), DevArr(hip, w)
+    Y = DevArr(hip, shape=(xs[0], 64, ci.OH, ci.OW), fill=np.nan)
+    hip.conv2d_fwd(0, desc, X.ptr, W.ptr, Y.ptr, 0)
+    y = Y.get()
+    for img in (0, xs[0] - 1):
+        assert rel_err(y[img:img + 1], conv2d_fwd(x[img:img + 1], w, 2, 1, 'same')) <= TOL
+
+
 def test_conv_passes_on_weights_with_swapped_channel_axes(hip):
     """A transposed convolution keeps its kernel as [C][O][KH][KW] relative to the convolution whose passes it
     borrows.  lnn_conv2d_permute_weights_f32(LNN_W_IOHW) makes Wp straight from that storage, the *_pw passes run
