@@ -135,7 +135,9 @@ int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units,
  * shape exercises. */
 #define LNN_FWD_PATH_IMPLICIT_GEMM 0 /* implicit GEMM on the matrix cores, operands gathered tile by tile */
 #define LNN_FWD_PATH_STEM_PATCH 1    /* 3 input channels, 33-64 output channels, 3x3 / 5x5 / 7x7: MFMA operands read
-                                        from an input patch in LDS (problems with at least 4 tiles per compute unit) */
+                                        from an input patch in LDS (problems with at least 4 tiles per compute unit);
+                                        lnn_conv2d_wgrad_f32 takes the matching kernel for such a geometry when
+                                        OW % 4 == 0 and dY is 16-byte aligned */
 int lnn_conv2d_fwd_path(const lnn_conv2d_desc* d, int compute_units, int* path);
 /* dW (+)= wgrad(X, dY)                   conv2D.py:52-54 (the reference always accumulates) */
 int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,

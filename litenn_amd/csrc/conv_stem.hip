@@ -41,8 +41,8 @@ struct StemCfg {
   static constexpr int PW = WL + 2 * ((C * R * PW_FREE + 63) & ~63) <= kStemLdsFloats ? PW_FREE : (QN + 7) & ~7;
   static constexpr int PLANE = R * PW;
   static constexpr int CHUNKS = (C * PLANE + 63) / 64;     // global -> LDS transfers (64 floats each) per patch
-  static constexpr int PATCH = CHUNKS * 64;
-  static constexpr int PER_WAVE = (CHUNKS + 3) / 4;
+  static constexpr int PER_WAVE = (CHUNKS + 3) / 4;        // every wavefront sends as many (the surplus: zeros)
+  static constexpr int PATCH = PER_WAVE * 4 * 64;
   static constexpr int LDS_FLOATS = WL + 2 * PATCH;
   // where tap k = (c, kh, kw) lies relative to a pixel's window origin
   static constexpr int off(int k) { return (k / (KH * KW)) * PLANE + ((k % (KH * KW)) / KW) * PW + k % KW; }
@@ -133,11 +133,9 @@ __global__ __launch_bounds__(256, 2) void stem_fwd_kernel(StemArgs a) {
     const int origin = (n * Cfg::C * a.IH + ih0) * a.IW + iw0;   // may be negative; valid elements are not
 #pragma unroll
     for (int j = 0; j < Cfg::PER_WAVE; ++j) {
-      if (w + 4 * j < Cfg::CHUNKS) {   // wave-uniform
-        const int ih = ih0 + (rq[j] & 0xffff), iw = iw0 + (rq[j] >> 16);
-        const bool ok = rq[j] >= 0 && (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
-        buf_load_lds4(rx, patch + (w + 4 * j) * 64, ok ? (uint32_t)(origin + rel[j]) * 4u : OOB, 0);
-      }
+      const int ih = ih0 + (rq[j] & 0xffff), iw = iw0 + (rq[j] >> 16);
+      const bool ok = rq[j] >= 0 && (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
+      buf_load_lds4(rx, patch + (w + 4 * j) * 64, ok ? (uint32_t)(origin + rel[j]) * 4u : OOB, 0);
     }
   };
 
@@ -236,6 +234,219 @@ int launch_stem_shape(DeviceCtx* ctx, StemArgs& a) {
   return LNN_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Weight gradient of the same geometries: dW[o][col] = sum over pixels of dY[o][pixel] * X[window of pixel][col],
+// col = (c, kh, kw).  The roles turn around: the K dimension is the pixels, two per MFMA; a lane of the B operand
+// owns a column, whose offset inside a pixel's window is fixed for the whole kernel, and the pixel's position in the
+// patch is the compile-time part of the address.  The A operand (dY) goes from global memory straight into registers,
+// sixteen consecutive pixels per lane and row block, a tile ahead.  One block of four wavefronts per compute unit, one
+// wavefront per SIMD: each keeps all 2 x NB accumulators (160 registers for 7x7) for its quarter of every tile's
+// pixels and for all the block's tiles; only at the end the four wavefronts' sums are added through LDS and the
+// block's partial result goes to scratch, where a small kernel adds the blocks up in a fixed order.
+template <int KH_, int KW_, int S_, int TW_>
+struct StemWCfg {
+  static constexpr int C = 3, KH = KH_, KW = KW_, S = S_, TW = TW_, TH = 128 / TW_;
+  static constexpr int K = C * KH * KW, NB = (K + 31) / 32;   // column blocks
+  static constexpr int R = (TH - 1) * S + KH, QN = (TW - 1) * S + KW;
+  static constexpr int PW = QN | 1, PLANE = R * PW;
+  static constexpr int CHUNKS = (C * PLANE + 63) / 64, PER_WAVE = (CHUNKS + 3) / 4, PATCH = PER_WAVE * 4 * 64;
+  static constexpr int LDS_FLOATS = 2 * PATCH > 4096 ? 2 * PATCH : 4096;   // the final sum needs 4 x 1024 floats
+  static constexpr int PART = 2 * NB * 1024;   // floats of a block's partial result: [row block][column block][r][lane]
+  // a wavefront's 32 pixels: one tile row (TW = 32: lane half h = columns 16h .. 16h+15) or two (TW = 16: h = row)
+  static constexpr int H_STEP = TW == 32 ? 16 * S : S * PW;
+  static constexpr int W_STEP = (TW == 32 ? 1 : 2) * S * PW;
+};
+
+struct StemWArgs {
+  const float* X;
+  const float* dY;
+  float* part;
+  int N, IH, IW, O, OH, OW, PADT, PADL, tiles_w, tiles_h, tiles;
+  FastDiv dTW, dTH;   // divide by tiles_w, tiles_h
+  uint32_t bytesX, bytesY;
+};
+
+template <class Cfg>
+__global__ __launch_bounds__(256, 1) void stem_wgrad_kernel(StemWArgs a) {
+  __shared__ __attribute__((aligned(16))) float smem[Cfg::LDS_FLOATS];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, i = lane & 31, h = lane >> 5;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const rsrc_t rx = make_rsrc(a.X, a.bytesX), ry = make_rsrc(a.dY, a.bytesY);
+  constexpr uint32_t OOB = 0x80000000u;
+  constexpr int NB = Cfg::NB;
+
+  int rel[Cfg::PER_WAVE], rq[Cfg::PER_WAVE];
+#pragma unroll
+  for (int j = 0; j < Cfg::PER_WAVE; ++j) {
+    const int e = (w + 4 * j) * 64 + lane;
+    const int c = e / Cfg::PLANE, rem = e - c * Cfg::PLANE, r = rem / Cfg::PW, q = rem - r * Cfg::PW;
+    const bool used = e < Cfg::C * Cfg::PLANE && q < Cfg::QN;
+    rel[j] = (c * a.IH + r) * a.IW + q;
+    rq[j] = used ? (r | (q << 16)) : -1;
+  }
+  auto request = [&](int tw, int th, int n, float* patch) {
+    const int ih0 = th * Cfg::TH * Cfg::S - a.PADT, iw0 = tw * Cfg::TW * Cfg::S - a.PADL;
+    const int origin = (n * Cfg::C * a.IH + ih0) * a.IW + iw0;
+#pragma unroll
+    for (int j = 0; j < Cfg::PER_WAVE; ++j) {
+      const int ih = ih0 + (rq[j] & 0xffff), iw = iw0 + (rq[j] >> 16);
+      const bool ok = rq[j] >= 0 && (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
+      buf_load_lds4(rx, patch + (w + 4 * j) * 64, ok ? (uint32_t)(origin + rel[j]) * 4u : OOB, 0);
+    }
+  };
+  // dY of a tile: this lane's sixteen pixels (row oh, columns ow .. ow + 15) of channels i and 32 + i.  Pixels past
+  // the row's end are read as whatever follows in memory (or zero past the tensor) and cleared afterwards.
+  f32x4 an[2][4];
+  auto load_a = [&](int tw, int th, int n) {
+    const int oh = th * Cfg::TH + (Cfg::TW == 32 ? w : 2 * w + h), ow = tw * Cfg::TW + (Cfg::TW == 32 ? 16 * h : 0);
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+      const int o = mb * 32 + i;
+      const bool ok = o < a.O && oh < a.OH && ow < a.OW;
+      const uint32_t voff = ok ? (uint32_t)(((n * a.O + o) * a.OH + oh) * a.OW + ow) * 4u : OOB;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) an[mb][q] = buf_load4_s(ry, voff, (uint32_t)(16 * q));
+    }
+    return ow;
+  };
+
+  // the column of lane i in each column block: where its tap lies inside a pixel's window; plus this wavefront's and
+  // this lane half's pixels
+  int bbase[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    int col = nb * 32 + i;
+    if (col >= Cfg::K) col = 0;   // padding columns compute something nobody stores
+    const int c = col / (Cfg::KH * Cfg::KW), r = col - c * (Cfg::KH * Cfg::KW), kh = r / Cfg::KW, kw = r - kh * Cfg::KW;
+    bbase[nb] = c * Cfg::PLANE + kh * Cfg::PW + kw + w * Cfg::W_STEP + h * Cfg::H_STEP;
+  }
+  f32x16 acc[2][NB];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.0f;
+
+  // a tile index into (column of tiles, row of tiles, image), in scalar registers
+  auto fetch = [&](int tile, float* patch) {
+    const uint32_t t = (uint32_t)__builtin_amdgcn_readfirstlane(tile);
+    const uint32_t rest = a.dTW.div(t), tw = t - rest * (uint32_t)a.tiles_w, n = a.dTH.div(rest), th = rest - n * (uint32_t)a.tiles_h;
+    request((int)tw, (int)th, (int)n, patch);
+    return load_a((int)tw, (int)th, (int)n);
+  };
+  int cur = 0;
+  int ow_next = fetch((int)blockIdx.x, smem);   // the grid never has more blocks than tiles
+  for (int tile = (int)blockIdx.x; tile < a.tiles; tile += (int)gridDim.x, cur ^= 1) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    // this tile's dY, pixels past the end of the row cleared
+    float av[2][16];
+    const int left = a.OW - ow_next;   // pixels of this lane's run that exist
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) av[mb][4 * q + e] = 4 * q + e < left ? an[mb][q][e] : 0.0f;
+    const float* patch = smem + cur * Cfg::PATCH;
+    // the next tile's operands (behind the last tile: that tile once more, into the buffer nobody reads again - no
+    // branch, so that these instructions can be spread among the MFMAs below)
+    const int nt = tile + (int)gridDim.x;
+    ow_next = fetch(nt < a.tiles ? nt : tile, smem + (cur ^ 1) * Cfg::PATCH);
+    // sixteen steps: the pixel t (lane half 0) and t + 16 or the pixel below (lane half 1)
+    float b[2][NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) b[0][nb] = patch[bbase[nb]];
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      if (t + 1 < 16) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) b[(t + 1) & 1][nb] = patch[bbase[nb] + (t + 1) * Cfg::S];
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        acc[0][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[0][t], b[t & 1][nb], acc[0][nb], 0, 0, 0);
+        acc[1][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[1][t], b[t & 1][nb], acc[1][nb], 0, 0, 0);
+      }
+    }
+  }
+
+  // the four wavefronts' sums, one accumulator at a time: [wave][r][lane] in LDS, thread (r4, lane) adds four values
+  // (wavefronts in order) for r = 4*r4 .. 4*r4 + 3
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  float* part = a.part + (size_t)blockIdx.x * Cfg::PART;
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) smem[w * 1024 + r * 64 + lane] = acc[mb][nb][r];
+      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int e = tid + 256 * q;
+        part[(mb * NB + nb) * 1024 + e] = ((smem[e] + smem[1024 + e]) + smem[2048 + e]) + smem[3072 + e];
+      }
+    }
+}
+
+// dW[o][col] (+)= sum over the blocks' partial results, blocks added in a fixed order: 32 consecutive elements per
+// block of 256 threads, eight lanes per element striding over the blocks.
+__global__ __launch_bounds__(256) void stem_wgrad_reduce(float* dW, const float* part, int nblocks, int per_block, int NB,
+                                                         int O, int K, int beta) {
+  __shared__ float red[8][33];
+  const int li = threadIdx.x & 31, ls = threadIdx.x >> 5;
+  const int e = blockIdx.x * 32 + li;
+  float s = 0.0f;
+  if (e < per_block) {
+#pragma unroll 8
+    for (int b = ls; b < nblocks; b += 8) s += part[(size_t)b * per_block + e];
+  }
+  red[ls][li] = s;
+  __syncthreads();
+  if (ls == 0 && e < per_block) {
+#pragma unroll
+    for (int k = 1; k < 8; ++k) s += red[k][li];
+    // element e of a partial result = (row block, column block, r, lane)
+    const int lane = e & 63, r = (e >> 6) & 15, pair = e >> 10, mb = pair / NB, nb = pair - mb * NB;
+    const int o = mb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), col = nb * 32 + (lane & 31);
+    if (o < O && col < K) {
+      float* dst = dW + (size_t)o * K + col;
+      *dst = beta ? *dst + s : s;
+    }
+  }
+}
+
+template <int KH, int KW, int S>
+int launch_stem_wgrad_shape(DeviceCtx* ctx, StemWArgs& a, float* dW, int beta) {
+  auto count = [&](int tw_) { return (long long)((a.OW + tw_ - 1) / tw_) * ((a.OH + 128 / tw_ - 1) / (128 / tw_)); };
+  const bool wide = count(32) <= count(16);
+  using Wide = StemWCfg<KH, KW, S, 32>;
+  using Square = StemWCfg<KH, KW, S, 16>;
+  const int tw_ = wide ? 32 : 16, th_ = 128 / tw_;
+  a.tiles_w = (a.OW + tw_ - 1) / tw_;
+  a.tiles_h = (a.OH + th_ - 1) / th_;
+  const long long tiles = (long long)a.N * a.tiles_w * a.tiles_h;
+  if (tiles > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
+  a.tiles = (int)tiles;
+  a.dTW = make_fastdiv((uint32_t)a.tiles_w);
+  a.dTH = make_fastdiv((uint32_t)a.tiles_h);
+  const int blocks = (int)(tiles < ctx->cus ? tiles : ctx->cus);   // one block per compute unit
+  int st = ensure_workspace(ctx, (size_t)blocks * Wide::PART * sizeof(float));
+  if (st != LNN_OK) return st;
+  a.part = static_cast<float*>(ctx->ws);
+  if (wide) hipLaunchKernelGGL((stem_wgrad_kernel<Wide>), dim3(blocks), dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((stem_wgrad_kernel<Square>), dim3(blocks), dim3(256), 0, ctx->stream, a);
+  LNN_HIP(hipGetLastError());
+  hipLaunchKernelGGL(stem_wgrad_reduce, dim3((Wide::PART + 31) / 32), dim3(256), 0, ctx->stream, dW, a.part, blocks,
+                     Wide::PART, Wide::NB, a.O, Wide::K, beta ? 1 : 0);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
+}
+
 }  // namespace
 
 // Geometries the patch kernel takes.  With fewer than four tiles per compute unit the implicit-GEMM pass, which cuts
@@ -262,6 +473,27 @@ int launch_stem_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   if (k == 3 && s == 1) return launch_stem_shape<3, 3, 1>(ctx, a);
   if (k == 3 && s == 2) return launch_stem_shape<3, 3, 2>(ctx, a);
   return set_error(LNN_ERR_INVALID, "conv2d_fwd: not a stem geometry");
+}
+
+// The weight gradient of the same geometries; rows of dY must be 16-byte aligned for the 128-bit loads.
+bool stem_wgrad_applies(const lnn_conv2d_desc* d, int compute_units, const float* dY) {
+  if (!stem_fwd_applies(d, compute_units)) return false;
+  return d->OW % 4 == 0 && (reinterpret_cast<uintptr_t>(dY) & 15) == 0;
+}
+
+// dW (+)= wgrad(X, dY) for the geometries stem_wgrad_applies() accepts
+int launch_stem_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta) {
+  StemWArgs a;
+  a.X = X; a.dY = dY; a.part = nullptr;
+  a.N = d->N; a.IH = d->IH; a.IW = d->IW; a.O = d->O; a.OH = d->OH; a.OW = d->OW; a.PADT = d->PADT; a.PADL = d->PADL;
+  a.bytesX = (uint32_t)((uint64_t)d->N * d->C * d->IH * d->IW * 4);
+  a.bytesY = (uint32_t)((uint64_t)d->N * d->O * d->OH * d->OW * 4);
+  const int k = d->KH, s = d->stride;
+  if (k == 7 && s == 2) return launch_stem_wgrad_shape<7, 7, 2>(ctx, a, dW, beta);
+  if (k == 5 && s == 2) return launch_stem_wgrad_shape<5, 5, 2>(ctx, a, dW, beta);
+  if (k == 3 && s == 1) return launch_stem_wgrad_shape<3, 3, 1>(ctx, a, dW, beta);
+  if (k == 3 && s == 2) return launch_stem_wgrad_shape<3, 3, 2>(ctx, a, dW, beta);
+  return set_error(LNN_ERR_INVALID, "conv2d_wgrad: not a stem geometry");
 }
 
 }  // namespace lnn

@@ -1,6 +1,10 @@
 // Convolution weight gradient (split over the output pixels, deterministic slice reduction).
 #include "conv_common.hpp"
 
+#ifndef LNN_STEM_WGRAD
+#define LNN_STEM_WGRAD 1
+#endif
+
 namespace lnn {
 
 int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta,
@@ -12,6 +16,7 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");
+  if (LNN_STEM_WGRAD && !w_iohw && stem_wgrad_applies(d, ctx->cus, dY)) return launch_stem_wgrad(ctx, d, X, dY, dW, beta);
   a.tab = nullptr;
   const ConvGeom& g = a.g;
   a.X = X; a.W = dY; a.Out = dW;

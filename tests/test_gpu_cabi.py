@@ -498,6 +498,25 @@ def test_conv_stem_forward_from_lds_patch_integer_exact(hip):
             hip.conv2d_fwd_bias_act(0, desc, X.ptr, W.ptr, B.ptr, hip.ACT_LEAKY_RELU, 0.25, Y.ptr)
             pre = ref + b[None, :, None, None]
             assert np.array_equal(Y.get(), np.where(pre >= 0, pre, 0.25 * pre).astype(np.float32)), (xs, ws, s, padding)
+            # weight gradient (the patch kernel where OW % 4 == 0): the whole batch in one call against the same
+            # batches accumulated with '+=' on the implicit-GEMM pass, whose first image is pinned to the oracle
+            dy = rs.randint(-3, 4, size=ref.shape).astype(np.float32)
+            dY = DevArr(hip, dy)
+            dWref = DevArr(hip, shape=ws, fill=0.0)
+            for i0 in range(0, n, step):
+                m = min(step, n - i0)
+                dpart, _ = _desc(hip, (m,) + xs[1:], ws, s, 1, padding)
+                Xp, dYp = DevArr(hip, x[i0:i0 + m]), DevArr(hip, dy[i0:i0 + m])
+                hip.conv2d_wgrad(0, dpart, Xp.ptr, dYp.ptr, dWref.ptr, 1)
+            done, _ = _desc(hip, (1,) + xs[1:], ws, s, 1, padding)
+            dW1 = DevArr(hip, shape=ws, fill=np.nan)
+            X1, dY1 = DevArr(hip, x[:1]), DevArr(hip, dy[:1])
+            hip.conv2d_wgrad(0, done, X1.ptr, dY1.ptr, dW1.ptr, 0)
+            assert np.array_equal(dW1.get(), conv2d_dw(x[:1], dy[:1], ws, s, 1, padding))
+            for beta, fill in ((0, np.nan), (1, 5.0)):
+                dW = DevArr(hip, shape=ws, fill=fill)
+                hip.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW.ptr, beta)
+                assert np.array_equal(dW.get() - (5.0 if beta else 0.0), dWref.get()), (xs, ws, s, padding, beta)
     # neighbours of the stem geometries stay on the other kernels
     for xs, ws, s, d in [((70, 3, 128, 128), (32, 3, 7, 7), 2, 1), ((70, 3, 64, 64), (96, 3, 3, 3), 1, 1),
                          ((70, 4, 128, 128), (64, 4, 5, 5), 2, 1), ((70, 3, 64, 64), (64, 3, 3, 3), 1, 2),
