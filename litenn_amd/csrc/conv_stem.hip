@@ -12,6 +12,10 @@
 
 #include "common.hpp"
 
+#ifndef LNN_STEM_MIN_TILES
+#define LNN_STEM_MIN_TILES 4   // tiles of 256 pixels per compute unit from which the patch kernels are used
+#endif
+
 namespace lnn {
 namespace {
 
@@ -449,13 +453,14 @@ int launch_stem_wgrad_shape(DeviceCtx* ctx, StemWArgs& a, float* dW, int beta) {
 
 }  // namespace
 
-// Geometries the patch kernel takes.  With fewer than four tiles per compute unit the implicit-GEMM pass, which cuts
-// the work more finely, is as fast or faster (16 x 3 x 128 x 128, 5x5 stride 2, 256 tiles: 23 against 18 us).
+// Geometries the patch kernels take.  With fewer than four tiles per compute unit the implicit-GEMM passes, which cut
+// the work more finely, are about as fast (16 x 3 x 128 x 128, 5x5 stride 2, one tile per compute unit: forward and
+// weight gradient together within 2 us either way).
 bool stem_fwd_applies(const lnn_conv2d_desc* d, int compute_units) {
   if (d->C != 3 || d->O <= 32 || d->O > 64 || d->dilation != 1 || d->KH != d->KW) return false;
   const int k = d->KH, s = d->stride;
   if (!((k == 7 && s == 2) || (k == 5 && s == 2) || (k == 3 && (s == 1 || s == 2)))) return false;
-  return (long long)d->N * (((long long)d->OH * d->OW + 255) / 256) >= 4ll * compute_units;
+  return (long long)d->N * (((long long)d->OH * d->OW + 255) / 256) >= (long long)LNN_STEM_MIN_TILES * compute_units;
 }
 
 // Y (+)= conv(X, W) with the bias / activation epilogue, for the geometries stem_fwd_applies() accepts
