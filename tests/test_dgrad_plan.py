@@ -66,3 +66,28 @@ def test_bad_arguments():
     bad = api.conv_desc(1, 1, 4, 4, 1, 3, 3, 4, 4, 1, 1, 0, 1)
     with pytest.raises(api.HipException):
         api.conv2d_dgrad_path(bad, 0, 256)
+
+
+def test_forward_path_selection():
+    """lnn_conv2d_fwd_path: the patch kernels take three input channels, 33-64 output channels, square 3x3
+    (stride 1 or 2), 5x5 and 7x7 (stride 2) kernels without dilation, from four 256-pixel tiles per compute unit."""
+    import pytest
+
+    def path(C=3, O=64, K=7, s=2, d=1, N=32, H=224, cus=256, KW=None):
+        KW = K if KW is None else KW
+        ci = info_conv2d(H, H, K, KW, s, d, 'same')
+        return api.conv2d_fwd_path(api.conv_desc(N, C, H, H, O, K, KW, ci.OH, ci.OW, ci.PADL, ci.PADT, s, d), cus)
+
+    assert path() == api.FWD_PATH_STEM_PATCH
+    for k, s in ((3, 1), (3, 2), (5, 2), (7, 2)):
+        assert path(K=k, s=s) == api.FWD_PATH_STEM_PATCH
+        assert path(K=k, s=s, O=33) == api.FWD_PATH_STEM_PATCH
+    for kw in (dict(C=4), dict(C=1), dict(O=32), dict(O=65), dict(K=5, s=1), dict(K=7, s=1), dict(K=3, s=3), dict(d=2),
+               dict(K=3, KW=5, s=1), dict(K=9)):
+        assert path(**kw) == api.FWD_PATH_IMPLICIT_GEMM, kw
+    # 112 x 112 output pixels = 49 tiles per image: 1024 tiles from 21 images on 256 compute units
+    assert path(N=21) == api.FWD_PATH_STEM_PATCH and path(N=20) == api.FWD_PATH_IMPLICIT_GEMM
+    assert path(N=20, cus=240) == api.FWD_PATH_STEM_PATCH
+    with pytest.raises(api.HipException) as e:
+        path(cus=0)
+    assert e.value.code == api.ERR_INVALID
