@@ -539,7 +539,7 @@ struct ConvFwdBDirect {
   __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
   template <int PART, int NPARTS>
   __device__ __forceinline__ int issue_part(int k0, float* lds, int ld, int off) {
-    const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
     for (int e = KR * PART / NPARTS; e < KR * (PART + 1) / NPARTS; ++e) {
 #pragma unroll
@@ -643,7 +643,7 @@ struct ConvFwdBTap {
   __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
   template <int PART, int NPARTS>
   __device__ __forceinline__ int issue_part(int, float* lds, int ld, int off) {
-    const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
     for (int e = KR * PART / NPARTS; e < KR * (PART + 1) / NPARTS; ++e) {
       const uint32_t soff = (uint32_t)((c0 + wave + 4 * e) * IHW) * 4u;
@@ -750,7 +750,7 @@ struct ConvDgradBTap {
   __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
   template <int PART, int NPARTS>
   __device__ __forceinline__ int issue_part(int, float* lds, int ld, int off) {
-    const int wave = __builtin_amdgcn_readfirstlane(gwave()), lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(gwave());
 #pragma unroll
     for (int e = KR * PART / NPARTS; e < KR * (PART + 1) / NPARTS; ++e) {
       const uint32_t soff = (uint32_t)((o0 + wave + 4 * e) * OHW) * 4u;
