@@ -128,6 +128,9 @@ int lnn_conv2d_dgrad_f32(int dev, const lnn_conv2d_desc* d, const float* dY, con
 #define LNN_DGRAD_PATH_MFMA_TABLE 0 /* implicit GEMM on the matrix cores, K = (o, tap) through a gather table */
 #define LNN_DGRAD_PATH_MFMA_TAP 1   /* implicit GEMM, tap-major K over channel-permuted weights (O % 32 == 0) */
 #define LNN_DGRAD_PATH_VECTOR 2     /* C <= 4: vector-ALU kernel, all pixel classes of a 32 x 32 tile per block */
+#define LNN_DGRAD_PATH_STEM_MFMA 3  /* C <= 4, stride 2, O a multiple of 8 from 32, kernels up to 8 x 8, at least two
+                                       32 x 32-pixel tiles per compute unit: the 2 x 2 pixel parities as rows of a
+                                       16-row GEMM over a dY patch in LDS */
 int lnn_conv2d_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* path, int32_t* tile_info);
 /* Which kernel family lnn_conv2d_fwd_f32 / lnn_conv2d_fwd_bias_act_f32 use for a geometry on a device with
  * `compute_units` compute units.  Host arithmetic only: works without a device.  No counterpart in the reference,

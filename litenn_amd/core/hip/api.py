@@ -277,7 +277,7 @@ def conv2d_fwd_path(desc, compute_units):
     return path.value
 
 
-DGRAD_PATH_MFMA_TABLE, DGRAD_PATH_MFMA_TAP, DGRAD_PATH_VECTOR = 0, 1, 2
+DGRAD_PATH_MFMA_TABLE, DGRAD_PATH_MFMA_TAP, DGRAD_PATH_VECTOR, DGRAD_PATH_STEM_MFMA = 0, 1, 2, 3
 
 
 def conv2d_dgrad_path(desc, beta, compute_units):

@@ -55,6 +55,8 @@ int launch_stem_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
                     const float* bias, int act, float slope);
 bool stem_wgrad_applies(const lnn_conv2d_desc* d, int compute_units, const float* dY);
 int launch_stem_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* dY, float* dW, int beta);
+bool stem_dgrad_applies(const lnn_conv2d_desc* d, int compute_units);
+int launch_stem_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta);
 int conv_fwd_path(const lnn_conv2d_desc* d, int compute_units, int* path);
 int conv_weights_plan(const lnn_conv2d_desc* d, int pass, int* yes);
 int launch_permute_weights(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* W, int w_layout, float* Wp);

@@ -1,6 +1,10 @@
 // Convolution data gradient: pixel classes on the MFMA engine, and the vector-ALU kernel for very few input channels.
 #include "conv_common.hpp"
 
+#ifndef LNN_STEM_DGRAD
+#define LNN_STEM_DGRAD 1
+#endif
+
 namespace lnn {
 namespace {
 
@@ -308,6 +312,10 @@ int conv_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* 
   *path = g.O % BK == 0 ? LNN_DGRAD_PATH_MFMA_TAP : LNN_DGRAD_PATH_MFMA_TABLE;
   if (tile_info)
     for (int i = 0; i < 7; ++i) tile_info[i] = 0;
+  if (LNN_STEM_DGRAD && stem_dgrad_applies(d, compute_units)) {
+    *path = LNN_DGRAD_PATH_STEM_MFMA;
+    return LNN_OK;
+  }
   if (small_dgrad_applies(compute_units, g)) {
     SmallDgradArgs a;
     int grid_x = 0;
@@ -346,6 +354,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   if (!dY || (!W && !Wp) || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
   const int S = full.S;
   if (S > 15) return set_error(LNN_ERR_UNSUPPORTED, "conv2d_dgrad: stride > 15");
+  if (LNN_STEM_DGRAD && !Wp && stem_dgrad_applies(d, ctx->cus)) return launch_stem_dgrad(ctx, d, dY, W, dX, beta);
   if (!tapw && small_dgrad_applies(ctx->cus, full)) {
     st = launch_small_dgrad(ctx, full, dY, W, dX, beta);
     if (st != kNotHere) return st;

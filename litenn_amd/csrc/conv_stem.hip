@@ -455,6 +455,139 @@ int launch_stem_wgrad_shape(DeviceCtx* ctx, StemWArgs& a, float* dW, int beta) {
   return LNN_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Data gradient of stride-2 convolutions with at most 4 input channels (the image gradient of a stem).  Seen from a
+// 2 x 2 block of input pixels (2i + a, 2j + b), every tap reads dY at (i + dh, j + dw) with dh, dw from a window of
+// at most four values each, and which tap that is depends only on (a, dh) and (b, dw).  So
+//     dX[(c, a, b)][i, j] = sum over o, sh, sw of dY[o][i + DH0 + sh][j + DW0 + sw] * Wt[(c, a, b)][o][sh][sw]
+// is a stride-1 4 x 4 convolution of dY with C * 4 <= 16 output rows and zeros where a (parity, slot) pair has no
+// tap: a GEMM with 16 rows, K = 16 * O, computed with v_mfma_f32_16x16x4_f32 (the four k of an instruction = the four
+// sw of one (o, sh)).  A block of four wavefronts computes 16 x 16 coarse pixels; dY travels global -> LDS eight
+// channels at a time (19 x 19 patch each, next chunk during the current one), the B operand is read from the patch at
+// lane base + immediate, the A operand from the rearranged weights of the same eight channels.
+constexpr int kDgTile = 16, kDgRows = kDgTile + 3, kDgPitch = 20, kDgPlane = kDgRows * kDgPitch, kDgChunk = 8;
+constexpr int kDgPatch = 3072;   // 8 planes of 380 floats, rounded up to whole transfers of 64 (48 = 12 per wavefront)
+constexpr int kDgWt = kDgChunk * 256;   // [o][sh][row][sw] of eight channels
+
+struct StemDArgs {
+  const float* dY;
+  const float* Wt;
+  float* dX;
+  int N, C, IH, IW, O, OH, OW, DH0, DW0, tiles_w, tiles_h, beta, pairs;
+  uint32_t bytesY, bytesWt, bytesX;
+};
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Wt[o][sh][row = c*4 + a*2 + b][sw] = W[o][c][kh][kw] with kh = a + PADT - 2*(DH0 + sh), kw likewise; 0 without a tap
+__global__ void stem_dgrad_weights_kernel(float* wt, const float* w, int O, int C, int KH, int KW, int PADT, int PADL,
+                                          int DH0, int DW0) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= O * 256) return;
+  const int sw = e & 3, row = (e >> 2) & 15, sh = (e >> 6) & 3, o = e >> 8;
+  const int c = row >> 2, a = (row >> 1) & 1, b = row & 1;
+  const int kh = a + PADT - 2 * (DH0 + sh), kw = b + PADL - 2 * (DW0 + sw);
+  wt[e] = (c < C && kh >= 0 && kh < KH && kw >= 0 && kw < KW) ? w[((size_t)(o * C + c) * KH + kh) * KW + kw] : 0.0f;
+}
+
+template <int OL, int SH>
+__device__ __forceinline__ void stem_dgrad_step(const float* wt, const float* patch, int abase, const int (&bbase)[4],
+                                                f32x4 (&acc)[4]) {
+  const float a = wt[abase + (OL * 4 + SH) * 64];
+  float b[4];
+#pragma unroll
+  for (int cb = 0; cb < 4; ++cb) b[cb] = patch[bbase[cb] + OL * kDgPlane + SH * kDgPitch];
+#pragma unroll
+  for (int cb = 0; cb < 4; ++cb) acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[cb], acc[cb], 0, 0, 0);
+}
+template <int... Is>
+__device__ __forceinline__ void stem_dgrad_chunk(std::integer_sequence<int, Is...>, const float* wt, const float* patch,
+                                                 int abase, const int (&bbase)[4], f32x4 (&acc)[4]) {
+  (stem_dgrad_step<Is / 4, Is % 4>(wt, patch, abase, bbase, acc), ...);
+}
+
+__global__ __launch_bounds__(256, 3) void stem_dgrad_kernel(StemDArgs a) {
+  __shared__ __attribute__((aligned(16))) float smem[2 * (kDgPatch + kDgWt)];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const rsrc_t ry = make_rsrc(a.dY, a.bytesY), rw = make_rsrc(a.Wt, a.bytesWt), rx = make_rsrc(a.dX, a.bytesX);
+  constexpr uint32_t OOB = 0x80000000u;
+  int bid = blockIdx.x;
+  const int tw = bid % a.tiles_w;
+  bid /= a.tiles_w;
+  const int th = bid % a.tiles_h, n = bid / a.tiles_h;
+  const int i0 = th * kDgTile, j0 = tw * kDgTile;   // coarse origin of the tile
+  const int ohw = a.OH * a.OW;
+
+  // dY patch transfers of one chunk: transfer t of this wavefront fills floats [(w + 4t)*64, +64) of the patch buffer,
+  // element (channel ol, row r, column q) of the chunk; the chunk's first channel travels in the scalar offset
+  uint32_t voff[12];
+#pragma unroll
+  for (int t = 0; t < 12; ++t) {
+    const int e = (w + 4 * t) * 64 + lane;
+    const int ol = e / kDgPlane, rem = e - ol * kDgPlane, r = rem / kDgPitch, q = rem - r * kDgPitch;
+    const int oh = i0 + a.DH0 + r, ow = j0 + a.DW0 + q;
+    const bool ok = ol < kDgChunk && q < kDgRows && (unsigned)oh < (unsigned)a.OH && (unsigned)ow < (unsigned)a.OW;
+    voff[t] = ok ? (uint32_t)(((n * a.O + ol) * a.OH + oh) * a.OW + ow) * 4u : OOB;
+  }
+  auto request = [&](int chunk, float* buf) {
+    const uint32_t sy = (uint32_t)(chunk * kDgChunk * ohw) * 4u, sw_ = (uint32_t)(chunk * kDgWt) * 4u;
+#pragma unroll
+    for (int t = 0; t < 12; ++t) buf_load_lds4(ry, buf + (w + 4 * t) * 64, voff[t], sy);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) buf_load_lds4(rw, buf + kDgPatch + (w + 4 * t) * 64, (uint32_t)((w + 4 * t) * 64 + lane) * 4u, sw_);
+  };
+
+  // lane (x = lane % 16, kq = lane / 16): row x of the A operand / column x of the B operand, k = kq (= sw)
+  const int x = lane & 15, kq = lane >> 4;
+  const int abase = x * 4 + kq;
+  int bbase[4];
+#pragma unroll
+  for (int cb = 0; cb < 4; ++cb) bbase[cb] = (4 * w + cb) * kDgPitch + x + kq;
+  f32x4 acc[4];
+#pragma unroll
+  for (int cb = 0; cb < 4; ++cb) acc[cb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  const int nch = a.O / kDgChunk;
+  request(0, smem);
+  for (int ch = 0, cur = 0; ch < nch; ++ch, cur ^= 1) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const float* buf = smem + cur * (kDgPatch + kDgWt);
+    if (ch + 1 < nch) request(ch + 1, smem + (cur ^ 1) * (kDgPatch + kDgWt));
+    stem_dgrad_chunk(std::make_integer_sequence<int, kDgChunk * 4>{}, buf + kDgPatch, buf, abase, bbase, acc);
+  }
+
+  // accumulator element r of lane (x, g = lane / 16): row 4g + r = channel g, pixel parity (a, b) = (r / 2, r % 2),
+  // coarse pixel (i0 + 4w + cb, j0 + x)
+  const int c = kq;
+  if (c < a.C) {
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) {
+      const int i = i0 + 4 * w + cb, j = j0 + x;
+      if (a.pairs) {   // even row length, 8-byte aligned tensor: the two pixels of a row in one 64-bit access
+#pragma unroll
+        for (int pa = 0; pa < 2; ++pa) {
+          const int ih = 2 * i + pa, iw = 2 * j;
+          const uint32_t off = (ih < a.IH && iw < a.IW) ? (uint32_t)(((n * a.C + c) * a.IH + ih) * a.IW + iw) * 4u : OOB;
+          f32x2 v = {acc[cb][2 * pa], acc[cb][2 * pa + 1]};
+          if (a.beta) v += __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(rx, (int)off, 0, 0));
+          __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), rx, (int)off, 0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int ih = 2 * i + (r >> 1), iw = 2 * j + (r & 1);
+          const uint32_t off = (ih < a.IH && iw < a.IW) ? (uint32_t)(((n * a.C + c) * a.IH + ih) * a.IW + iw) * 4u : OOB;
+          float v = acc[cb][r];
+          if (a.beta) v += buf_load(rx, off);
+          buf_store(rx, off, v);
+        }
+      }
+    }
+  }
+}
+
 }  // namespace
 
 // Geometries the patch kernels take.  With fewer than four tiles per compute unit the implicit-GEMM passes, which cut
@@ -503,6 +636,46 @@ int launch_stem_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   if (k == 3 && s == 1) return launch_stem_wgrad_shape<3, 3, 1>(ctx, a, dW, beta);
   if (k == 3 && s == 2) return launch_stem_wgrad_shape<3, 3, 2>(ctx, a, dW, beta);
   return set_error(LNN_ERR_INVALID, "conv2d_wgrad: not a stem geometry");
+}
+
+// floor(a / 2) for negative a too
+static int half_floor(int a) { return a >= 0 ? a / 2 : -((-a + 1) / 2); }
+
+// The data gradient above: stride 2, no dilation, at most 4 input channels, output channels a multiple of 8 (from 32),
+// at most four dY rows and columns per input pixel pair (kernels up to 8 x 8), at least two tiles per compute unit.
+bool stem_dgrad_applies(const lnn_conv2d_desc* d, int compute_units) {
+  if (d->C > 4 || d->stride != 2 || d->dilation != 1 || d->O % kDgChunk != 0 || d->O < 32) return false;
+  const int dh0 = -half_floor(d->KH - 1 - d->PADT), dw0 = -half_floor(d->KW - 1 - d->PADL);
+  if (half_floor(1 + d->PADT) - dh0 + 1 > 4 || half_floor(1 + d->PADL) - dw0 + 1 > 4) return false;
+  const long long tiles = (long long)d->N * (((d->IH + 1) / 2 + kDgTile - 1) / kDgTile) * (((d->IW + 1) / 2 + kDgTile - 1) / kDgTile);
+  return tiles >= 2ll * compute_units && tiles <= 0x7fffffffll;
+}
+
+// dX (+)= dgrad(dY, W) for the geometries stem_dgrad_applies() accepts
+int launch_stem_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY, const float* W, float* dX, int beta) {
+  StemDArgs a;
+  a.dY = dY; a.dX = dX;
+  a.N = d->N; a.C = d->C; a.IH = d->IH; a.IW = d->IW; a.O = d->O; a.OH = d->OH; a.OW = d->OW;
+  a.DH0 = -half_floor(d->KH - 1 - d->PADT);
+  a.DW0 = -half_floor(d->KW - 1 - d->PADL);
+  a.tiles_h = ((d->IH + 1) / 2 + kDgTile - 1) / kDgTile;
+  a.tiles_w = ((d->IW + 1) / 2 + kDgTile - 1) / kDgTile;
+  a.beta = beta ? 1 : 0;
+  a.pairs = d->IW % 2 == 0 && (reinterpret_cast<uintptr_t>(dX) & 7) == 0;
+  a.bytesY = (uint32_t)((uint64_t)d->N * d->O * d->OH * d->OW * 4);
+  a.bytesX = (uint32_t)((uint64_t)d->N * d->C * d->IH * d->IW * 4);
+  a.bytesWt = (uint32_t)((uint64_t)d->O * 256 * 4);
+  int st = ensure_workspace(ctx, a.bytesWt);
+  if (st != LNN_OK) return st;
+  float* wt = static_cast<float*>(ctx->ws);
+  hipLaunchKernelGGL(stem_dgrad_weights_kernel, dim3((d->O * 256 + 255) / 256), dim3(256), 0, ctx->stream, wt, W, d->O, d->C,
+                     d->KH, d->KW, d->PADT, d->PADL, a.DH0, a.DW0);
+  LNN_HIP(hipGetLastError());
+  a.Wt = wt;
+  const long long tiles = (long long)a.N * a.tiles_w * a.tiles_h;
+  hipLaunchKernelGGL(stem_dgrad_kernel, dim3((unsigned)tiles), dim3(256), 0, ctx->stream, a);
+  LNN_HIP(hipGetLastError());
+  return LNN_OK;
 }
 
 }  // namespace lnn

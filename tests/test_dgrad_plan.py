@@ -57,6 +57,25 @@ def test_selection_rules():
     assert path(3, 3, 1, N=1, cus=304) == api.DGRAD_PATH_MFMA_TABLE
 
 
+def test_stem_mfma_selection():
+    """LNN_DGRAD_PATH_STEM_MFMA: stride 2, no dilation, at most four input channels, 32 or more output channels in
+    multiples of 8, at most four dY rows and columns per pair of input pixels, two tiles of 32 x 32 pixels per compute
+    unit; everything else keeps its earlier path."""
+    def path(C=3, O=64, K=7, s=2, d=1, padding=3, N=32, H=224, cus=256):
+        return api.conv2d_dgrad_path(_desc(N, C, H, H, O, K, s, d, padding), 0, cus)[0]
+
+    assert path() == api.DGRAD_PATH_STEM_MFMA
+    for kw in (dict(C=4), dict(C=1), dict(O=32), dict(O=72), dict(K=5, padding=2), dict(K=3, padding=1), dict(K=2, padding=0),
+               dict(K=7, padding='valid'), dict(K=8, padding=2), dict(K=4, padding=1)):
+        assert path(**kw) == api.DGRAD_PATH_STEM_MFMA, kw
+    for kw in (dict(C=5), dict(O=24), dict(O=36), dict(s=1, K=3, padding=1), dict(d=2), dict(K=9, padding=4), dict(K=8, padding=3),
+               dict(s=3, K=5, padding=2)):
+        assert path(**kw) != api.DGRAD_PATH_STEM_MFMA, kw
+    # 224 x 224 pixels = 49 tiles per image: 512 tiles from 11 images on 256 compute units
+    assert path(N=11) == api.DGRAD_PATH_STEM_MFMA and path(N=10) == api.DGRAD_PATH_VECTOR
+    assert path(N=10, cus=240) == api.DGRAD_PATH_STEM_MFMA
+
+
 def test_bad_arguments():
     import pytest
     d = _desc(4, 3, 16, 16, 4, 3, 1, 1, 'same')

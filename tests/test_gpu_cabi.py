@@ -538,6 +538,54 @@ def test_conv_stem_forward_from_lds_patch_integer_exact(hip):
         assert rel_err(y[img:img + 1], conv2d_fwd(x[img:img + 1], w, 2, 1, 'same')) <= TOL
 
 
+def test_conv_stem_dgrad_parity_rows_integer_exact(hip):
+    """Stride 2, at most 4 input channels, 32 or more output channels (a multiple of 8), at least two tiles of 32 x 32
+    input pixels per compute unit: the data gradient computes the four pixel parities of each channel as rows of a
+    16-row GEMM over a dY patch in LDS (v_mfma_f32_16x16x4_f32).  Kernels from 2 x 2 to 8 x 8 (square and not), every
+    padding kind, image sizes that are not multiples of the tile and odd, '=' and '+='; lnn_conv2d_dgrad_path confirms
+    the path.  The first and the last image are checked against the oracle, all images against the same call on
+    batches too small for this kernel (the vector-ALU or the implicit-GEMM data gradient, pinned by the other tests).
+    Exact on small integers."""
+    rs = np.random.RandomState(65)
+    cus = hip.device_info(0)['compute_units']
+    cases = [(3, 64, 7, 7, 3, 70, 66), (3, 32, 5, 5, 'same', 70, 66), (4, 40, 3, 3, 'same', 64, 64), (1, 64, 7, 7, 'valid', 71, 67),
+             (3, 48, 4, 4, 1, 65, 33), (2, 32, 8, 8, (2, 2, 4, 3), 70, 66), (3, 64, 2, 2, 0, 70, 66), (3, 32, 6, 3, (1, 0, 0, 2), 33, 130),
+             (4, 64, 7, 5, (2, 3, 1, 0), 70, 66), (3, 72, 5, 5, 2, 37, 41)]
+    for C, O, kh, kw, padding, ih, iw in cases:
+        tiles_per_img = (((ih + 1) // 2 + 15) // 16) * (((iw + 1) // 2 + 15) // 16)
+        n = -(-2 * cus // tiles_per_img) + 1
+        xs, ws = (n, C, ih, iw), (O, C, kh, kw)
+        ci = info_conv2d(ih, iw, kh, kw, 2, 1, padding)
+        desc = hip.conv_desc(n, C, ih, iw, O, kh, kw, ci.OH, ci.OW, ci.PADL, ci.PADT, 2, 1)
+        assert hip.conv2d_dgrad_path(desc, 0, cus)[0] == hip.DGRAD_PATH_STEM_MFMA, (xs, ws, padding)
+        say(f'stem dgrad x={xs} w={ws} pad={padding} dy {ci.OH}x{ci.OW}')
+        w = rs.randint(-3, 4, size=ws).astype(np.float32)
+        dy = rs.randint(-3, 4, size=(n, O, ci.OH, ci.OW)).astype(np.float32)
+        W, dY = DevArr(hip, w), DevArr(hip, dy)
+        ref = np.empty(xs, np.float32)
+        step = max(1, (2 * cus - 1) // tiles_per_img)
+        for i0 in range(0, n, step):
+            m = min(step, n - i0)
+            dpart = hip.conv_desc(m, C, ih, iw, O, kh, kw, ci.OH, ci.OW, ci.PADL, ci.PADT, 2, 1)
+            assert hip.conv2d_dgrad_path(dpart, 0, cus)[0] != hip.DGRAD_PATH_STEM_MFMA
+            dYp, dXp = DevArr(hip, dy[i0:i0 + m]), DevArr(hip, shape=(m,) + xs[1:], fill=np.nan)
+            hip.conv2d_dgrad(0, dpart, dYp.ptr, W.ptr, dXp.ptr, 0)
+            ref[i0:i0 + m] = dXp.get()
+        for img in (0, n - 1):
+            assert np.array_equal(ref[img:img + 1], conv2d_dx(dy[img:img + 1], w, (1,) + xs[1:], 2, 1, padding)), (xs, ws, padding)
+        for beta, fill in ((0, np.nan), (1, 3.0)):
+            dX = DevArr(hip, shape=xs, fill=fill)
+            hip.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, beta)
+            assert np.array_equal(dX.get() - (3.0 if beta else 0.0), ref), (xs, ws, padding, beta)
+    # neighbours that stay on the other kernels: few output channels, not a multiple of 8, stride 1, dilation, five
+    # channels, a 9 x 9 kernel and an 8 x 8 one with odd padding (five dY rows per pixel pair), too few tiles
+    for (N, C, O, k, s, d) in [(64, 3, 16, 7, 2, 1), (64, 3, 36, 7, 2, 1), (64, 3, 64, 3, 1, 1), (64, 3, 64, 3, 2, 2),
+                               (64, 5, 64, 7, 2, 1), (64, 3, 64, 9, 2, 1), (64, 3, 64, 8, 2, 1), (8, 3, 64, 7, 2, 1)]:
+        ci = info_conv2d(70, 66, k, k, s, d, 'same')
+        desc = hip.conv_desc(N, C, 70, 66, O, k, k, ci.OH, ci.OW, ci.PADL, ci.PADT, s, d)
+        assert hip.conv2d_dgrad_path(desc, 0, 256)[0] != hip.DGRAD_PATH_STEM_MFMA, (N, C, O, k, s, d)
+
+
 def test_conv_passes_on_weights_with_swapped_channel_axes(hip):
     """A transposed convolution keeps its kernel as [C][O][KH][KW] relative to the convolution whose passes it
     borrows.  lnn_conv2d_permute_weights_f32(LNN_W_IOHW) makes Wp straight from that storage, the *_pw passes run
@@ -907,8 +955,8 @@ def test_conv_full_size_adjoint_and_linearity(hip, xs, ws, s, d, padding):
     dy = rs.normal(0, 1, (xs[0], ws[0], ci.OH, ci.OW)).astype(np.float32)
     say(f'full-size identities x={xs} w={ws}')
     if xs[1] == 3 and hip.device_info(0)['compute_units'] == 256:
-        # the image stem at full batch is the shape the vector-ALU data gradient exists for (four chunks of output channels per wavefront)
-        assert hip.conv2d_dgrad_path(desc, 0, 256)[0] == hip.DGRAD_PATH_VECTOR
+        # the image stem at full batch takes the 16-row MFMA data gradient over a dY patch in LDS
+        assert hip.conv2d_dgrad_path(desc, 0, 256)[0] == hip.DGRAD_PATH_STEM_MFMA
     X, W, W2, dY = DevArr(hip, x), DevArr(hip, w), DevArr(hip, w2), DevArr(hip, dy)
     Y, Y2, Y12 = (DevArr(hip, shape=dy.shape, fill=np.nan) for _ in range(3))
     dX, dW = DevArr(hip, shape=xs, fill=np.nan), DevArr(hip, shape=ws, fill=np.nan)
