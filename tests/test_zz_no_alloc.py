@@ -61,6 +61,10 @@ def test_noalloc_wgrad_matches_the_allocating_entry_point_twice_in_a_row(hip):
                  ((1, 1024, 8, 8), (1024, 1024, 3, 3), 1, 1, 'same')):
         say(f'noalloc wgrad {case}')
         _both(hip, *case, seed=4)
+    # an image stem at a batch that takes the patch kernel: its blocks' partial results (10 MiB) live in the same array
+    patch = ((24, 3, 224, 224), (64, 3, 7, 7), 2, 1, 3)
+    say(f'noalloc wgrad {patch}')
+    _both(hip, *patch, seed=7)
     # and the first, large shape again after the small ones
     _both(hip, *big, seed=5)
 
