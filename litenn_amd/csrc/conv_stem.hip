@@ -61,6 +61,7 @@ struct StemArgs {
   const float* W;
   float* Y;
   int N, IH, IW, O, OH, OW, PADT, PADL, tiles_w, tiles_h, tiles, beta;
+  FastDiv dTW, dTH;   // divide by tiles_w, tiles_h
   uint32_t bytesX;
   PostOp post;
 };
@@ -133,8 +134,17 @@ __global__ __launch_bounds__(256, 2) void stem_fwd_kernel(StemArgs a) {
     rel[j] = (c * a.IH + r) * a.IW + q;
     rq[j] = used ? (r | (q << 16)) : -1;
   }
+  // a tile index into (column of tiles, row of tiles, image), in scalar registers
+  auto decode = [&](int tile, int& tw, int& th, int& n) {
+    const uint32_t t = (uint32_t)__builtin_amdgcn_readfirstlane(tile);
+    const uint32_t rest = a.dTW.div(t), img = a.dTH.div(rest);
+    tw = (int)(t - rest * (uint32_t)a.tiles_w);
+    th = (int)(rest - img * (uint32_t)a.tiles_h);
+    n = (int)img;
+  };
   auto request = [&](int tile, float* patch) {
-    const int tw = tile % a.tiles_w, rest = tile / a.tiles_w, th = rest % a.tiles_h, n = rest / a.tiles_h;
+    int tw, th, n;
+    decode(tile, tw, th, n);
     const int ih0 = th * Cfg::TH * Cfg::S - a.PADT, iw0 = tw * Cfg::TW * Cfg::S - a.PADL;
     const int origin = (n * Cfg::C * a.IH + ih0) * a.IW + iw0;   // may be negative; valid elements are not
 #pragma unroll
@@ -194,7 +204,8 @@ __global__ __launch_bounds__(256, 2) void stem_fwd_kernel(StemArgs a) {
     // go through a descriptor of this image's O planes: the lane's part of the address (pixel, and 4*h channels) is
     // computed once per pixel block, the rest of the channel index travels in the scalar offset, and channels past O
     // fall outside the descriptor and are dropped - no vector arithmetic per store.
-    const int tw = tile % a.tiles_w, rest = tile / a.tiles_w, th = rest % a.tiles_h, n = rest / a.tiles_h;
+    int tw, th, n;
+    decode(tile, tw, th, n);
     const int ohw = a.OH * a.OW;
     const rsrc_t ry = make_rsrc(a.Y + (size_t)n * a.O * ohw, (uint32_t)(a.O * ohw) * 4u);
 #pragma unroll
@@ -233,6 +244,8 @@ int launch_stem_shape(DeviceCtx* ctx, StemArgs& a) {
   const long long tiles = (long long)a.N * a.tiles_w * a.tiles_h;
   if (tiles > 0x7fffffffll) return set_error(LNN_ERR_UNSUPPORTED, "conv2d: too many tiles");
   a.tiles = (int)tiles;
+  a.dTW = make_fastdiv((uint32_t)a.tiles_w);
+  a.dTH = make_fastdiv((uint32_t)a.tiles_h);
   const long long blocks = tiles < 2ll * ctx->cus ? tiles : 2ll * ctx->cus;   // two blocks per compute unit
   if (wide) hipLaunchKernelGGL((stem_fwd_kernel<Wide>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a);
   else hipLaunchKernelGGL((stem_fwd_kernel<Square>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a);
