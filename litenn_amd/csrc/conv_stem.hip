@@ -155,7 +155,10 @@ __global__ __launch_bounds__(256, 2) void stem_fwd_kernel(StemArgs a) {
     }
   };
 
-  request((int)blockIdx.x, smem + Cfg::WL);
+  // consecutive workgroups go to different XCDs (eight, each with its own L2) and neighbouring tiles share input
+  // columns and output lines: number the blocks so that an XCD's blocks take neighbouring tiles
+  const int bx = (gridDim.x & 7) == 0 ? (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  request(bx, smem + Cfg::WL);
   // weights: element (o, k) of W[O][K] goes to wl[k/2][o/32][k%2][o%32]; zeros for the rows past O and the padding k
   constexpr int KP = 2 * Cfg::T;
   constexpr int WITER = (64 * KP + 255) / 256;
@@ -183,7 +186,7 @@ __global__ __launch_bounds__(256, 2) void stem_fwd_kernel(StemArgs a) {
   }
 
   int cur = 0;
-  for (int tile = (int)blockIdx.x; tile < a.tiles; tile += (int)gridDim.x, cur ^= 1) {
+  for (int tile = bx; tile < a.tiles; tile += (int)gridDim.x, cur ^= 1) {
     // this tile's patch has landed (and this thread's stores of the last tile have left); behind the barrier every
     // wavefront is done reading the other buffer, which the next tile's patch may now overwrite
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -486,7 +489,7 @@ struct StemDArgs {
   const float* dY;
   const float* Wt;
   float* dX;
-  int N, C, IH, IW, O, OH, OW, DH0, DW0, tiles_w, tiles_h, beta, pairs;
+  int N, C, IH, IW, O, OH, OW, DH0, DW0, tiles_w, tiles_h, tiles, per_xcd, beta, pairs;
   uint32_t bytesY, bytesWt, bytesX;
 };
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -525,7 +528,10 @@ __global__ __launch_bounds__(256, 3) void stem_dgrad_kernel(StemDArgs a) {
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const rsrc_t ry = make_rsrc(a.dY, a.bytesY), rw = make_rsrc(a.Wt, a.bytesWt), rx = make_rsrc(a.dX, a.bytesX);
   constexpr uint32_t OOB = 0x80000000u;
-  int bid = blockIdx.x;
+  // Consecutive workgroups go to different XCDs (eight, each with its own L2), neighbouring tiles share lines of dY:
+  // workgroup b takes tile (b % 8) * per_xcd + b / 8, so that an XCD walks a contiguous run of tiles.
+  int bid = (int)(blockIdx.x & 7) * a.per_xcd + (int)(blockIdx.x >> 3);
+  if (bid >= a.tiles) return;   // the whole block leaves together
   const int tw = bid % a.tiles_w;
   bid /= a.tiles_w;
   const int th = bid % a.tiles_h, n = bid / a.tiles_h;
@@ -686,7 +692,9 @@ int launch_stem_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   LNN_HIP(hipGetLastError());
   a.Wt = wt;
   const long long tiles = (long long)a.N * a.tiles_w * a.tiles_h;
-  hipLaunchKernelGGL(stem_dgrad_kernel, dim3((unsigned)tiles), dim3(256), 0, ctx->stream, a);
+  a.tiles = (int)tiles;
+  a.per_xcd = (int)((tiles + 7) / 8);
+  hipLaunchKernelGGL(stem_dgrad_kernel, dim3((unsigned)(8 * a.per_xcd)), dim3(256), 0, ctx->stream, a);
   LNN_HIP(hipGetLastError());
   return LNN_OK;
 }
