@@ -24,6 +24,9 @@
 #ifndef LNN_KSPLIT_HALF
 #define LNN_KSPLIT_HALF 1
 #endif
+#ifndef LNN_DGRAD_PAIRS
+#define LNN_DGRAD_PAIRS 1
+#endif
 #ifndef LNN_STAGES_WGRAD
 #define LNN_STAGES_WGRAD 3
 #endif
@@ -897,7 +900,9 @@ template <int PASS, int WM, int NTMAX>
 static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_off) {
   const int n = (int)cls.size();
   const int per_batch = n < kMaxBatch ? n : kMaxBatch;
-  const long long equal = ctx->cus / per_batch > 0 ? ctx->cus / per_batch : 1;   // equal shares of the chip
+  // equal shares of the chip; the 64 x 128 tile's three LDS stages (72 KB) fit twice on a compute unit
+  const long long chip = (long long)ctx->cus * (WM == 2 && NTMAX == 1 ? 2 : 1);
+  const long long equal = chip / per_batch > 0 ? chip / per_batch : 1;
   // The classes of one launch differ in their number of taps (5x5 stride 2: 9, 6, 6 and 4): with the tap-major
   // kernels, whose time follows the multiply-adds, each gets workgroups in proportion to its work instead
   // (256 -> 512 channels at 16 x 16: 77 -> 63 us).
@@ -926,7 +931,7 @@ static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_
       for (;;) {
         int best = -1;
         for (int i = 0; i < n; ++i) {
-          if (used + chunks[i] > ctx->cus || ks[i] + 1 > nkt[i] / 8) continue;   // plan_tiles caps slices at nkt / 8
+          if (used + chunks[i] > chip || ks[i] + 1 > nkt[i] / 8) continue;   // plan_tiles caps slices at nkt / 8
           if (best < 0 || nkt[i] * ks[best] > nkt[best] * ks[i]) best = i;
         }
         if (best < 0) break;
@@ -1001,6 +1006,21 @@ template <int PASS>
 static int launch_classes_by_m(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_off) {
   const int M = cls[0].M;
   if (M > 64) return launch_classes<PASS, 4, 4>(ctx, cls, ws_off);
+  if (LNN_DGRAD_PAIRS && PASS == PASS_DGRAD_TAPW && M > 32 && cls.size() == 4) {
+    // Four classes with many tiles each and different K lengths (5x5 stride 2: 9, 6, 6 and 4 taps): on 64 x 128
+    // tiles two workgroups share a compute unit, and with the classes in the order longest, second, shortest, third
+    // workgroups b and b + (number of compute units) - which land on the same one - are a long and a short piece.
+    bool plain = true;
+    for (const ConvArgs& a : cls) {
+      const long long units = (a.Ncols + 63) / 64;
+      plain = plain && units >= 2ll * ctx->cus / 4 * 2;   // at least one full 2-unit sub-tile per workgroup: no K split
+    }
+    if (plain) {
+      std::sort(cls.begin(), cls.end(), [](const ConvArgs& x, const ConvArgs& y) { return x.K > y.K; });
+      std::swap(cls[2], cls[3]);
+      return launch_classes<PASS, 2, 1>(ctx, cls, ws_off);
+    }
+  }
   if (M > 32) return launch_classes<PASS, 2, 2>(ctx, cls, ws_off);
   return launch_classes<PASS, 1, 1>(ctx, cls, ws_off);
 }

@@ -217,6 +217,43 @@ def test_conv_strided_dgrad_pixel_classes_integer_exact(hip):
     assert cnt > 300
 
 
+def test_conv_strided_dgrad_paired_classes_integer_exact(hip):
+    """Stride 2 with 33-64 input channels (a multiple of 4) and class planes of at least 512 sub-tiles of 64 x 128 each:
+    the four pixel classes run on 64 x 128 tiles, two workgroups per compute unit, ordered so that a class with many
+    taps shares its compute units with one with few.  Whole and ragged tiles, 5x5 and 3x3, '=' and '+='; the data
+    gradient through lnn_conv2d_dgrad_f32 and, on one permuted copy, lnn_conv2d_dgrad_pw_f32.  The first image is
+    checked against the oracle, all images against the same call on half the batch at a time (class planes too small
+    for this plan: the wider tiles, one workgroup per compute unit, which the other tests pin).  Exact on small
+    integers."""
+    rs = np.random.RandomState(66)
+    for xs, ws, padding in [((16, 64, 64, 64), (32, 64, 5, 5), 2), ((17, 48, 62, 66), (32, 48, 3, 3), 'same'),
+                            ((9, 36, 91, 90), (64, 36, 5, 5), (1, 2, 2, 1))]:
+        desc, ci = _desc(hip, xs, ws, 2, 1, padding)
+        say(f'paired classes x={xs} w={ws} pad={padding}')
+        n, O = xs[0], ws[0]
+        w = rs.randint(-2, 3, size=ws).astype(np.float32)
+        dy = rs.randint(-2, 3, size=(n, O, ci.OH, ci.OW)).astype(np.float32)
+        W, dY = DevArr(hip, w), DevArr(hip, dy)
+        ref = np.empty(xs, np.float32)
+        half = (n + 1) // 2
+        for i0 in range(0, n, half):
+            m = min(half, n - i0)
+            dpart, _ = _desc(hip, (m,) + xs[1:], ws, 2, 1, padding)
+            dYp, dXp = DevArr(hip, dy[i0:i0 + m]), DevArr(hip, shape=(m,) + xs[1:], fill=np.nan)
+            hip.conv2d_dgrad(0, dpart, dYp.ptr, W.ptr, dXp.ptr, 0)
+            ref[i0:i0 + m] = dXp.get()
+        assert np.array_equal(ref[:1], conv2d_dx(dy[:1], w, (1,) + xs[1:], 2, 1, padding)), (xs, ws, padding)
+        Wp = DevArr(hip, shape=(O, ws[2] * ws[3], ws[1]), fill=np.nan)
+        hip.conv2d_permute_weights(0, desc, W.ptr, hip.W_OIHW, Wp.ptr)
+        for beta, fill in ((0, np.nan), (1, -1.0)):
+            dX = DevArr(hip, shape=xs, fill=fill)
+            hip.conv2d_dgrad(0, desc, dY.ptr, W.ptr, dX.ptr, beta)
+            assert np.array_equal(dX.get() - (-1.0 if beta else 0.0), ref), (xs, ws, padding, beta)
+            dX = DevArr(hip, shape=xs, fill=fill)
+            hip.conv2d_dgrad_pw(0, desc, dY.ptr, Wp.ptr, dX.ptr, beta)
+            assert np.array_equal(dX.get() - (-1.0 if beta else 0.0), ref), (xs, ws, padding, beta, 'pw')
+
+
 def test_conv_channel_multiples_of_32_integer_exact(hip):
     """Channel counts that are multiples of 32 take the tap-major kernels
     (forward / dgrad: permuted weights, address arithmetic in the scalar
