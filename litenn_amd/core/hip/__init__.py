@@ -41,6 +41,37 @@ def launch(fn, *args):
                     raise
 
 
+def cached_permuted_copies(tensors):
+    """For an optimizer step over `tensors`: per tensor None, or (key, copies, C, KH*KW) when every device buffer of
+    the tensor holds exactly one permuted copy Wp[o][tap][c] made from OIHW storage (permuted_weights below) - the
+    update kernels can then store the new values in the copy too.  copies is a launch() argument."""
+    out = []
+    for t in tensors:
+        key, copies = None, []
+        for buf in t._get_buffers():
+            keys = [k for k in (buf._derived or {}) if k[0] == 'wp']
+            if len(keys) != 1 or keys[0][1] != int(api.W_OIHW) or (key is not None and keys[0] != key):
+                key = None
+                break
+            key = keys[0]
+            copies.append(buf._derived[key][1])
+        if key is None or key[2] * key[3] * key[4] * key[5] != t.shape.size:
+            out.append(None)
+        else:
+            out.append((key, _BufferList(copies), key[3], key[4] * key[5]))
+    return out
+
+
+def keep_permuted_copies(tensors, cached):
+    """After an update that wrote the copies of cached_permuted_copies(): they are valid for the tensors' new contents."""
+    if ShallowMode.active():
+        return
+    for t, c in zip(tensors, cached):
+        if c is not None:
+            for buf, copy in zip(t._get_buffers(), c[1]._get_buffers()):
+                buf._derived[c[0]] = (buf._version, copy)
+
+
 class _BufferList(HipDevicesBuffers):
     """Per-device buffers that already exist, in the shape launch() takes."""
 

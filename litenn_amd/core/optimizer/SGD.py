@@ -1,5 +1,5 @@
 import litenn_amd as nn
-from ..hip import api, launch
+from ..hip import api, launch, cached_permuted_copies, keep_permuted_copies
 from .Optimizer import Optimizer
 
 
@@ -24,5 +24,15 @@ class SGD(Optimizer):
             return
         k, ns = len(ts), [t.shape.size for t in ts]
         # every tensor's update in one launch per device: pointers arrive as (values, gradients, accumulators)
-        launch(lambda dev, *p: api.sgd_update_multi(dev, ns, p[:k], p[k:2 * k], p[2 * k:], self.momentum, lr, self.nesterov),
-               *ts, *[t.get_grad() for t in ts], *[self._accs[t.get_name()] for t in ts])
+        grads, accs = [t.get_grad() for t in ts], [self._accs[t.get_name()] for t in ts]
+        cached = cached_permuted_copies(ts)
+        if any(c is not None for c in cached):
+            # convolution kernels whose permuted copy is cached: the update refreshes the copy in the same pass
+            cs, kks = [c[2] if c else 0 for c in cached], [c[3] if c else 0 for c in cached]
+            launch(lambda dev, *p: api.sgd_update_multi_wp(dev, ns, p[:k], p[k:2 * k], p[2 * k:3 * k], self.momentum, lr,
+                                                           self.nesterov, p[3 * k:], cs, kks),
+                   *ts, *grads, *accs, *[c[1] if c else None for c in cached])
+            keep_permuted_copies(ts, cached)
+        else:
+            launch(lambda dev, *p: api.sgd_update_multi(dev, ns, p[:k], p[k:2 * k], p[2 * k:], self.momentum, lr, self.nesterov),
+                   *ts, *grads, *accs)

@@ -85,6 +85,7 @@ struct RedPlan {
   int kshape[kMaxRank], rshape[kMaxRank];
   long long kstride[kMaxRank], rstride[kMaxRank];
   uint64_t outs, red;
+  int flat;   // the reduced axes are the trailing ones: element r of a reduction lies r floats behind its first
 };
 
 __device__ __forceinline__ long long offset_of(uint32_t idx, int n, const int* shape, const long long* stride) {
@@ -106,7 +107,11 @@ __global__ void reduce_sum_kernel(RedPlan p, const float* in, float* dst, int pa
   const long long base = offset_of((uint32_t)o, p.nk, p.kshape, p.kstride);
   const uint64_t r0 = p.red * part / parts, r1 = p.red * (part + 1) / parts;
   float s = 0.0f;
-  for (uint64_t r = r0 + threadIdx.x; r < r1; r += 256) s += in[base + offset_of((uint32_t)r, p.nr, p.rshape, p.rstride)];
+  if (p.flat) {   // same elements in the same order, without the index arithmetic
+    for (uint64_t r = r0 + threadIdx.x; r < r1; r += 256) s += in[base + (long long)r];
+  } else {
+    for (uint64_t r = r0 + threadIdx.x; r < r1; r += 256) s += in[base + offset_of((uint32_t)r, p.nr, p.rshape, p.rstride)];
+  }
   sh[threadIdx.x] = s;
   __syncthreads();
   for (int w = 128; w > 0; w >>= 1) {
@@ -238,7 +243,17 @@ struct MultiArgs {
   const float* g[kMultiMax];    // its gradient
   float* s0[kMultiMax];         // optimizer state (SGD: accumulator; Adam: m)
   float* s1[kMultiMax];         // Adam: v
+  // a convolution kernel's copy in the layout the tap-major passes read, Wp[o][tap][c] (or null): the update writes
+  // the new value there too, so that the copy need not be made again before the next forward pass
+  float* wp[kMultiMax];
+  FastDiv dKK[kMultiMax], dC[kMultiMax];
 };
+// parameter element i = (o*C + c)*KK + tap goes to Wp[(o*KK + tap)*C + c]
+__device__ __forceinline__ void store_permuted(const MultiArgs& a, int k, uint64_t i, float value) {
+  const uint32_t oc = a.dKK[k].div((uint32_t)i), tap = (uint32_t)i - oc * a.dKK[k].d;
+  const uint32_t o = a.dC[k].div(oc), c = oc - o * a.dC[k].d;
+  a.wp[k][((size_t)o * a.dKK[k].d + tap) * a.dC[k].d + c] = value;
+}
 __global__ void sgd_multi_kernel(MultiArgs a, float momentum, float lr, int nesterov) {
   const int k = blockIdx.y;
   const uint64_t n = a.n[k];
@@ -248,7 +263,9 @@ __global__ void sgd_multi_kernel(MultiArgs a, float momentum, float lr, int nest
   for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
     const float x = momentum * acc[i] - lr * g[i];
     acc[i] = x;
-    v[i] += nesterov ? momentum * x - lr * g[i] : x;
+    const float nv = v[i] + (nesterov ? momentum * x - lr * g[i] : x);
+    v[i] = nv;
+    if (a.wp[k]) store_permuted(a, k, i, nv);
   }
 }
 __global__ void adam_multi_kernel(MultiArgs a, float beta1, float beta2, float lr) {
@@ -264,7 +281,9 @@ __global__ void adam_multi_kernel(MultiArgs a, float beta1, float beta2, float l
     const float vi = beta2 * v2[i] + (1.0f - beta2) * gi * gi;
     m[i] = mi;
     v2[i] = vi;
-    t[i] += -lr * mi / (sqrtf(vi) + 1e-7f);
+    const float nt = t[i] + -lr * mi / (sqrtf(vi) + 1e-7f);
+    t[i] = nt;
+    if (a.wp[k]) store_permuted(a, k, i, nt);
   }
 }
 
@@ -353,6 +372,8 @@ int launch_reduce_sum(DeviceCtx* ctx, int rank, const int32_t* shape, uint32_t m
     }
   }
   if (p.outs > 0x7fffffffull) return set_error(LNN_ERR_UNSUPPORTED, "reduce_sum: too many outputs");
+  p.flat = p.nr > 0 && p.rstride[p.nr - 1] == 1;
+  for (int i = 0; i + 1 < p.nr; ++i) p.flat = p.flat && p.rstride[i] == p.rstride[i + 1] * p.rshape[i + 1];
   // long reductions with few outputs are split so the whole chip takes part
   int parts = 1;
   if (p.red >= 8192) {
@@ -608,8 +629,10 @@ int launch_random_normal(DeviceCtx* ctx, float* out, uint64_t n, uint32_t seed, 
 }
 
 // kind 0: SGD (p0 momentum, p1 unused, flag nesterov), kind 1: Adam (p0 beta1, p1 beta2)
+// wp / wp_c / wp_kk (all null, or arrays of count): tensor i's permuted copy Wp[o][tap][c] or null, its C and KH*KW
 int launch_update_multi(DeviceCtx* ctx, int kind, int count, const uint64_t* n, float* const* t, const float* const* g,
-                        float* const* s0, float* const* s1, float p0, float p1, float lr, int flag) {
+                        float* const* s0, float* const* s1, float p0, float p1, float lr, int flag, float* const* wp,
+                        const int32_t* wp_c, const int32_t* wp_kk) {
   const char* who = kind ? "adam_update_multi" : "sgd_update_multi";
   if (count < 0) return set_error(LNN_ERR_INVALID, std::string(who) + ": negative count");
   if (count == 0) return LNN_OK;
@@ -624,6 +647,15 @@ int launch_update_multi(DeviceCtx* ctx, int kind, int count, const uint64_t* n, 
       if (a.n[i] && (!a.t[i] || !a.g[i] || !a.s0[i] || (kind && !a.s1[i])))
         return set_error(LNN_ERR_INVALID, std::string(who) + ": null pointer");
       most = a.n[i] > most ? a.n[i] : most;
+      a.dKK[i] = a.dC[i] = FastDiv{0, 0, 1};
+      if (wp && wp[i0 + i] && a.n[i]) {
+        if (!wp_c || !wp_kk || wp_c[i0 + i] <= 0 || wp_kk[i0 + i] <= 0 || a.n[i] % ((uint64_t)wp_c[i0 + i] * wp_kk[i0 + i]) != 0 ||
+            a.n[i] > 0x7fffffffull)
+          return set_error(LNN_ERR_INVALID, std::string(who) + ": a permuted copy whose channel and tap counts do not divide the tensor");
+        a.wp[i] = wp[i0 + i];
+        a.dKK[i] = make_fastdiv((uint32_t)wp_kk[i0 + i]);
+        a.dC[i] = make_fastdiv((uint32_t)wp_c[i0 + i]);
+      }
     }
     if (most == 0) continue;
     const dim3 grid(grid_for(most, ctx->cus / 2).x, (unsigned)nb);

@@ -13,7 +13,7 @@ from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
          'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'conv2d_permute_weights', 'conv2d_fwd_pw', 'conv2d_dgrad_pw', 'conv2d_wgrad_iohw', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
-         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal', 'bias_act_bwd', 'sgd_update_multi', 'adam_update_multi']
+         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal', 'bias_act_bwd', 'sgd_update_multi', 'sgd_update_multi_wp', 'adam_update_multi_wp', 'adam_update_multi']
 
 
 class FakeHip:
@@ -238,6 +238,20 @@ class FakeHip:
         for n, v, g, a in zip(ns, vs, gs, accs):
             self.sgd_update(dev, n, v, g, a, momentum, lr, nesterov)
         self.launches -= len(ns) - 1
+
+    def _refresh_copies(self, ns, vs, wps, cs, kks):
+        for n, v, wp, c, kk in zip(ns, vs, wps, cs, kks):
+            if wp is not None and n:
+                o = n // (c * kk)
+                self.f(wp, (o, kk, c))[...] = self.f(v, (o, c, kk)).transpose(0, 2, 1)
+
+    def sgd_update_multi_wp(self, dev, ns, vs, gs, accs, momentum, lr, nesterov, wps, cs, kks):
+        self.sgd_update_multi(dev, ns, vs, gs, accs, momentum, lr, nesterov)
+        self._refresh_copies(ns, vs, wps, cs, kks)
+
+    def adam_update_multi_wp(self, dev, ns, ts, gs, ms, vs, beta1, beta2, lr, wps, cs, kks):
+        self.adam_update_multi(dev, ns, ts, gs, ms, vs, beta1, beta2, lr)
+        self._refresh_copies(ns, ts, wps, cs, kks)
 
     def adam_update_multi(self, dev, ns, ts, gs, ms, vs, beta1, beta2, lr):
         for n, t, g, m, v in zip(ns, ts, gs, ms, vs):

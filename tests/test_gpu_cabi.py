@@ -849,6 +849,44 @@ def test_multi_tensor_updates_equal_single_launches(hip):
         hip.sgd_update_multi(0, [4], [None], [many[1][0].ptr], [many[2][0].ptr], 0.9, 1e-2, False)
 
 
+def test_multi_tensor_updates_refresh_permuted_copies(hip):
+    """lnn_sgd_update_multi_wp_f32 / lnn_adam_update_multi_wp_f32: the same new values and optimizer state as the
+    plain multi-tensor calls, bit for bit, and for every tensor that brings a permuted copy the copy equals
+    Wp[o][tap][c] of the new values; tensors without a copy, an empty tensor and more tensors than one launch holds
+    among them.  A copy whose channel and tap counts do not divide the tensor is refused."""
+    rs = np.random.RandomState(78)
+    shapes = [(32, 32, 9), None, (64, 3, 49), (5, 7, 1), None, (40, 24, 25), (8, 130, 4)] + [None] * 12 + [(3, 5, 6)]
+    sizes = [int(np.prod(sh)) if sh else 37 + i for i, sh in enumerate(shapes)]
+    sizes[4] = 0
+    mk = lambda: [rs.standard_normal(max(n, 1)).astype(np.float32) for n in sizes]
+    v0, g0, a0, b0 = mk(), mk(), mk(), [np.abs(x) for x in mk()]
+    cs = [sh[1] if sh else 0 for sh in shapes]
+    kks = [sh[2] if sh else 0 for sh in shapes]
+    for kind in ('sgd', 'sgd_nesterov', 'adam'):
+        say(f'multi-tensor update with permuted copies {kind}')
+        plain = [[DevArr(hip, x) for x in arrs] for arrs in (v0, g0, a0, b0)]
+        fused = [[DevArr(hip, x) for x in arrs] for arrs in (v0, g0, a0, b0)]
+        wps = [DevArr(hip, shape=(n,), fill=np.nan) if sh else None for sh, n in zip(shapes, sizes)]
+        pp, pf = [[d.ptr for d in col] for col in plain], [[d.ptr for d in col] for col in fused]
+        wptrs = [w.ptr if w is not None else None for w in wps]
+        if kind == 'adam':
+            hip.adam_update_multi(0, sizes, pp[0], pp[1], pp[2], pp[3], 0.9, 0.999, 1e-2)
+            hip.adam_update_multi_wp(0, sizes, pf[0], pf[1], pf[2], pf[3], 0.9, 0.999, 1e-2, wptrs, cs, kks)
+        else:
+            hip.sgd_update_multi(0, sizes, pp[0], pp[1], pp[2], 0.9, 1e-2, kind == 'sgd_nesterov')
+            hip.sgd_update_multi_wp(0, sizes, pf[0], pf[1], pf[2], 0.9, 1e-2, kind == 'sgd_nesterov', wptrs, cs, kks)
+        for col_p, col_f in zip(plain, fused):
+            for x, y in zip(col_p, col_f):
+                assert np.array_equal(x.get(), y.get())
+        for sh, w, v in zip(shapes, wps, fused[0]):
+            if sh:
+                assert np.array_equal(w.get().reshape(sh[0], sh[2], sh[1]), v.get().reshape(sh).transpose(0, 2, 1)), (kind, sh)
+    with pytest.raises(hip.HipException) as e:
+        hip.sgd_update_multi_wp(0, [10], [fused[0][0].ptr], [fused[1][0].ptr], [fused[2][0].ptr], 0.9, 1e-2, False,
+                                [wps[0].ptr], [3], [3])
+    assert e.value.code == hip.ERR_INVALID
+
+
 def test_bias_act_bwd_one_pass(hip):
     """dpre = dy * f'(y) and dbias[o] (+)= sum dpre: exact on small integers with a power-of-two slope, <= 1e-5 of
     the largest |dbias| on floats (fp32 sums against fp64)."""
