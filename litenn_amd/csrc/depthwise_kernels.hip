@@ -132,7 +132,7 @@ __device__ __forceinline__ void dw_unit_rows(const float* lds, int lo, int srcH,
       for (int j = 0; j + 1 < KS; ++j)
 #pragma unroll
         for (int b = 0; b < KS; ++b) win[j][b] = win[j + 1][b];
-      col.load_row(lds, lo, srcH, srcW, r - pt + KS - 1, win[KS - 1]);
+      col.load_row(lds, lo, srcH, srcW, r - pt + KS - 1, win[T - 1]);   // T = KS in every instantiation that runs
       float v = 0.0f;
 #pragma unroll
       for (int a = 0; a < KS; ++a)
