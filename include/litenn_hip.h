@@ -257,17 +257,19 @@ int lnn_sgd_update_multi_f32(int dev, int count, const uint64_t* n, float* const
                              float* const* acc, float momentum, float lr, int nesterov);
 int lnn_adam_update_multi_f32(int dev, int count, const uint64_t* n, float* const* t, const float* const* g,
                               float* const* m, float* const* v, float beta1, float beta2, float lr);
-/* The same, for a caller that keeps permuted copies of its convolution kernels (lnn_conv2d_permute_weights_f32,
- * layout LNN_W_OIHW): wp[i] is tensor i's copy Wp[o][tap][c] or NULL, wp_c[i] / wp_kk[i] its C and KH*KW.  The
- * update stores every new value in the copy as well, so the copy stays valid across the optimizer step and the next
- * forward pass needs no permutation launch.  No counterpart in the reference (Optimizer.py:117-147 updates tensor
- * by tensor and conv2D_dI_gradfn re-transposes the kernel in every backward pass, conv2D.py:48). */
+/* The same, for a caller that keeps permuted copies of its convolution kernels (lnn_conv2d_permute_weights_f32):
+ * wp[i] is tensor i's copy Wp[o][tap][c] or NULL, wp_c[i] / wp_kk[i] its C and KH*KW, wp_layout[i] how the tensor
+ * itself is stored (LNN_W_OIHW, or LNN_W_IOHW for the kernel of a transposed convolution; wp_layout NULL = all
+ * LNN_W_OIHW).  The update stores every new value in the copy as well, so the copy stays valid across the optimizer
+ * step and the next forward pass needs no permutation launch.  No counterpart in the reference
+ * (Optimizer.py:117-147 updates tensor by tensor; conv2D_dI_gradfn re-transposes the kernel in every backward pass,
+ * conv2D.py:48, conv2DTranspose swaps its channel axes in every pass, conv2DTranspose.py:33-47). */
 int lnn_sgd_update_multi_wp_f32(int dev, int count, const uint64_t* n, float* const* v, const float* const* g,
                                 float* const* acc, float momentum, float lr, int nesterov, float* const* wp,
-                                const int32_t* wp_c, const int32_t* wp_kk);
+                                const int32_t* wp_c, const int32_t* wp_kk, const int32_t* wp_layout);
 int lnn_adam_update_multi_wp_f32(int dev, int count, const uint64_t* n, float* const* t, const float* const* g,
                                  float* const* m, float* const* v, float beta1, float beta2, float lr, float* const* wp,
-                                 const int32_t* wp_c, const int32_t* wp_kk);
+                                 const int32_t* wp_c, const int32_t* wp_kk, const int32_t* wp_layout);
 
 /* On-device random initialisers: element i is drawn from a counter hash of (uint32)(i + seed), so a tensor
  * is filled in place without host staging (initializer/RandomUniform.py:13-27, RandomNormal.py:10-30; the PCG

@@ -42,15 +42,16 @@ def launch(fn, *args):
 
 
 def cached_permuted_copies(tensors):
-    """For an optimizer step over `tensors`: per tensor None, or (key, copies, C, KH*KW) when every device buffer of
-    the tensor holds exactly one permuted copy Wp[o][tap][c] made from OIHW storage (permuted_weights below) - the
-    update kernels can then store the new values in the copy too.  copies is a launch() argument."""
+    """For an optimizer step over `tensors`: per tensor None, or (key, copies, C, KH*KW, layout) when every device
+    buffer of the tensor holds exactly one permuted copy Wp[o][tap][c] (permuted_weights below; layout = how the
+    tensor itself is stored, W_OIHW or W_IOHW) - the update kernels can then store the new values in the copy too.
+    copies is a launch() argument."""
     out = []
     for t in tensors:
         key, copies = None, []
         for buf in t._get_buffers():
             keys = [k for k in (buf._derived or {}) if k[0] == 'wp']
-            if len(keys) != 1 or keys[0][1] != int(api.W_OIHW) or (key is not None and keys[0] != key):
+            if len(keys) != 1 or (key is not None and keys[0] != key):
                 key = None
                 break
             key = keys[0]
@@ -58,7 +59,7 @@ def cached_permuted_copies(tensors):
         if key is None or key[2] * key[3] * key[4] * key[5] != t.shape.size:
             out.append(None)
         else:
-            out.append((key, _BufferList(copies), key[3], key[4] * key[5]))
+            out.append((key, _BufferList(copies), key[3], key[4] * key[5], key[1]))
     return out
 
 

@@ -89,8 +89,8 @@ SIGNATURES = {
     'lnn_adam_update_f32': [_c_int, _c_u64, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32],
     'lnn_sgd_update_multi_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int],
     'lnn_adam_update_multi_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32],
-    'lnn_sgd_update_multi_wp_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int, _ptr, _ptr, _ptr],
-    'lnn_adam_update_multi_wp_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32, _ptr, _ptr, _ptr],
+    'lnn_sgd_update_multi_wp_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int, _ptr, _ptr, _ptr, _ptr],
+    'lnn_adam_update_multi_wp_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32, _ptr, _ptr, _ptr, _ptr],
     'lnn_bias_act_bwd_f32': [_c_int, _c_int, _c_int, _c_int, _ptr, _ptr, _c_int, _c_f32, _ptr, _ptr, _c_int],
     'lnn_random_uniform_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
     'lnn_random_normal_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
@@ -375,21 +375,23 @@ def sgd_update_multi(dev, ns, vs, gs, accs, momentum, lr, nesterov):
                                        _ptr_array(accs), float(momentum), float(lr), 1 if nesterov else 0))
 
 
-def sgd_update_multi_wp(dev, ns, vs, gs, accs, momentum, lr, nesterov, wps, cs, kks):
+def sgd_update_multi_wp(dev, ns, vs, gs, accs, momentum, lr, nesterov, wps, cs, kks, layouts=None):
     """sgd_update_multi that also stores the new values in the tensors' permuted copies Wp[o][tap][c] (wps[i] a device
-    pointer or None, cs[i] / kks[i] the copy's C and KH*KW)."""
+    pointer or None, cs[i] / kks[i] the copy's C and KH*KW, layouts[i] W_OIHW / W_IOHW: how tensor i is stored)."""
     count = len(ns)
+    lay = (ctypes.c_int32 * count)(*layouts) if layouts is not None else None
     check(lib.lnn_sgd_update_multi_wp_f32(dev, count, (ctypes.c_uint64 * count)(*ns), _ptr_array(vs), _ptr_array(gs),
                                           _ptr_array(accs), float(momentum), float(lr), 1 if nesterov else 0,
-                                          _ptr_array(wps), (ctypes.c_int32 * count)(*cs), (ctypes.c_int32 * count)(*kks)))
+                                          _ptr_array(wps), (ctypes.c_int32 * count)(*cs), (ctypes.c_int32 * count)(*kks), lay))
 
 
-def adam_update_multi_wp(dev, ns, ts, gs, ms, vs, beta1, beta2, lr, wps, cs, kks):
+def adam_update_multi_wp(dev, ns, ts, gs, ms, vs, beta1, beta2, lr, wps, cs, kks, layouts=None):
     """adam_update_multi that also stores the new values in the tensors' permuted copies (see sgd_update_multi_wp)."""
     count = len(ns)
+    lay = (ctypes.c_int32 * count)(*layouts) if layouts is not None else None
     check(lib.lnn_adam_update_multi_wp_f32(dev, count, (ctypes.c_uint64 * count)(*ns), _ptr_array(ts), _ptr_array(gs),
                                            _ptr_array(ms), _ptr_array(vs), float(beta1), float(beta2), float(lr),
-                                           _ptr_array(wps), (ctypes.c_int32 * count)(*cs), (ctypes.c_int32 * count)(*kks)))
+                                           _ptr_array(wps), (ctypes.c_int32 * count)(*cs), (ctypes.c_int32 * count)(*kks), lay))
 
 
 def adam_update_multi(dev, ns, ts, gs, ms, vs, beta1, beta2, lr):

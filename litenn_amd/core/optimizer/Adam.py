@@ -28,8 +28,9 @@ class Adam(Optimizer):
         if any(c is not None for c in cached):
             # convolution kernels whose permuted copy is cached: the update refreshes the copy in the same pass
             cs, kks = [c[2] if c else 0 for c in cached], [c[3] if c else 0 for c in cached]
+            lays = [c[4] if c else 0 for c in cached]
             launch(lambda dev, *p: api.adam_update_multi_wp(dev, ns, p[:k], p[k:2 * k], p[2 * k:3 * k], p[3 * k:4 * k],
-                                                            self.beta_1, self.beta_2, lr, p[4 * k:], cs, kks),
+                                                            self.beta_1, self.beta_2, lr, p[4 * k:], cs, kks, lays),
                    *ts, *grads, *ms, *vs, *[c[1] if c else None for c in cached])
             keep_permuted_copies(ts, cached)
         else:

@@ -19,7 +19,7 @@ int launch_sgd(DeviceCtx*, uint64_t, float*, const float*, float*, float, float,
 int launch_adam(DeviceCtx*, uint64_t, float*, const float*, float*, float*, float, float, float);
 int launch_random_uniform(DeviceCtx*, float*, uint64_t, uint32_t, double, double);
 int launch_update_multi(DeviceCtx*, int, int, const uint64_t*, float* const*, const float* const*, float* const*, float* const*,
-                        float, float, float, int, float* const*, const int32_t*, const int32_t*);
+                        float, float, float, int, float* const*, const int32_t*, const int32_t*, const int32_t*);
 int launch_bias_act_bwd(DeviceCtx*, int, int, int, const float*, const float*, int, float, float*, float*, int);
 int launch_random_normal(DeviceCtx*, float*, uint64_t, uint32_t, double, double);
 
@@ -478,27 +478,27 @@ int lnn_adam_update_f32(int dev, uint64_t n, float* t, const float* g, float* m,
 int lnn_sgd_update_multi_f32(int dev, int count, const uint64_t* n, float* const* v, const float* const* g, float* const* acc,
                              float momentum, float lr, int nesterov) {
   CTX(dev);
-  return launch_update_multi(ctx, 0, count, n, v, g, acc, nullptr, momentum, 0.0f, lr, nesterov, nullptr, nullptr, nullptr);
+  return launch_update_multi(ctx, 0, count, n, v, g, acc, nullptr, momentum, 0.0f, lr, nesterov, nullptr, nullptr, nullptr, nullptr);
 }
 
 int lnn_sgd_update_multi_wp_f32(int dev, int count, const uint64_t* n, float* const* v, const float* const* g,
                                 float* const* acc, float momentum, float lr, int nesterov, float* const* wp,
-                                const int32_t* wp_c, const int32_t* wp_kk) {
+                                const int32_t* wp_c, const int32_t* wp_kk, const int32_t* wp_layout) {
   CTX(dev);
-  return launch_update_multi(ctx, 0, count, n, v, g, acc, nullptr, momentum, 0.0f, lr, nesterov, wp, wp_c, wp_kk);
+  return launch_update_multi(ctx, 0, count, n, v, g, acc, nullptr, momentum, 0.0f, lr, nesterov, wp, wp_c, wp_kk, wp_layout);
 }
 
 int lnn_adam_update_multi_f32(int dev, int count, const uint64_t* n, float* const* t, const float* const* g, float* const* m,
                               float* const* v, float beta1, float beta2, float lr) {
   CTX(dev);
-  return launch_update_multi(ctx, 1, count, n, t, g, m, v, beta1, beta2, lr, 0, nullptr, nullptr, nullptr);
+  return launch_update_multi(ctx, 1, count, n, t, g, m, v, beta1, beta2, lr, 0, nullptr, nullptr, nullptr, nullptr);
 }
 
 int lnn_adam_update_multi_wp_f32(int dev, int count, const uint64_t* n, float* const* t, const float* const* g,
                                  float* const* m, float* const* v, float beta1, float beta2, float lr, float* const* wp,
-                                 const int32_t* wp_c, const int32_t* wp_kk) {
+                                 const int32_t* wp_c, const int32_t* wp_kk, const int32_t* wp_layout) {
   CTX(dev);
-  return launch_update_multi(ctx, 1, count, n, t, g, m, v, beta1, beta2, lr, 0, wp, wp_c, wp_kk);
+  return launch_update_multi(ctx, 1, count, n, t, g, m, v, beta1, beta2, lr, 0, wp, wp_c, wp_kk, wp_layout);
 }
 
 int lnn_bias_act_bwd_f32(int dev, int N, int O, int HW, const float* y, const float* dy, int act, float slope,

@@ -246,13 +246,17 @@ struct MultiArgs {
   // a convolution kernel's copy in the layout the tap-major passes read, Wp[o][tap][c] (or null): the update writes
   // the new value there too, so that the copy need not be made again before the next forward pass
   float* wp[kMultiMax];
-  FastDiv dKK[kMultiMax], dC[kMultiMax];
+  FastDiv dKK[kMultiMax], dIn[kMultiMax];   // divide by KH*KW, by the inner of the tensor's two channel axes
+  int wp_c[kMultiMax];                      // C of the copy; negative: the tensor is stored [C][O][tap]
 };
-// parameter element i = (o*C + c)*KK + tap goes to Wp[(o*KK + tap)*C + c]
+// parameter element i = (o*C + c)*KK + tap (or (c*O + o)*KK + tap for a tensor stored with swapped channel axes, as
+// a transposed convolution keeps its kernel) goes to Wp[(o*KK + tap)*C + c]
 __device__ __forceinline__ void store_permuted(const MultiArgs& a, int k, uint64_t i, float value) {
   const uint32_t oc = a.dKK[k].div((uint32_t)i), tap = (uint32_t)i - oc * a.dKK[k].d;
-  const uint32_t o = a.dC[k].div(oc), c = oc - o * a.dC[k].d;
-  a.wp[k][((size_t)o * a.dKK[k].d + tap) * a.dC[k].d + c] = value;
+  const uint32_t hi = a.dIn[k].div(oc), lo = oc - hi * a.dIn[k].d;
+  const bool swapped = a.wp_c[k] < 0;
+  const uint32_t C = (uint32_t)(swapped ? -a.wp_c[k] : a.wp_c[k]), o = swapped ? lo : hi, c = swapped ? hi : lo;
+  a.wp[k][((size_t)o * a.dKK[k].d + tap) * C + c] = value;
 }
 __global__ void sgd_multi_kernel(MultiArgs a, float momentum, float lr, int nesterov) {
   const int k = blockIdx.y;
@@ -629,10 +633,11 @@ int launch_random_normal(DeviceCtx* ctx, float* out, uint64_t n, uint32_t seed, 
 }
 
 // kind 0: SGD (p0 momentum, p1 unused, flag nesterov), kind 1: Adam (p0 beta1, p1 beta2)
-// wp / wp_c / wp_kk (all null, or arrays of count): tensor i's permuted copy Wp[o][tap][c] or null, its C and KH*KW
+// wp / wp_c / wp_kk / wp_layout (all null, or arrays of count; wp_layout may be null = all LNN_W_OIHW): tensor i's
+// permuted copy Wp[o][tap][c] or null, its C and KH*KW, and how the tensor itself is stored
 int launch_update_multi(DeviceCtx* ctx, int kind, int count, const uint64_t* n, float* const* t, const float* const* g,
                         float* const* s0, float* const* s1, float p0, float p1, float lr, int flag, float* const* wp,
-                        const int32_t* wp_c, const int32_t* wp_kk) {
+                        const int32_t* wp_c, const int32_t* wp_kk, const int32_t* wp_layout) {
   const char* who = kind ? "adam_update_multi" : "sgd_update_multi";
   if (count < 0) return set_error(LNN_ERR_INVALID, std::string(who) + ": negative count");
   if (count == 0) return LNN_OK;
@@ -647,14 +652,19 @@ int launch_update_multi(DeviceCtx* ctx, int kind, int count, const uint64_t* n, 
       if (a.n[i] && (!a.t[i] || !a.g[i] || !a.s0[i] || (kind && !a.s1[i])))
         return set_error(LNN_ERR_INVALID, std::string(who) + ": null pointer");
       most = a.n[i] > most ? a.n[i] : most;
-      a.dKK[i] = a.dC[i] = FastDiv{0, 0, 1};
+      a.dKK[i] = a.dIn[i] = FastDiv{0, 0, 1};
+      a.wp_c[i] = 0;
       if (wp && wp[i0 + i] && a.n[i]) {
         if (!wp_c || !wp_kk || wp_c[i0 + i] <= 0 || wp_kk[i0 + i] <= 0 || a.n[i] % ((uint64_t)wp_c[i0 + i] * wp_kk[i0 + i]) != 0 ||
             a.n[i] > 0x7fffffffull)
           return set_error(LNN_ERR_INVALID, std::string(who) + ": a permuted copy whose channel and tap counts do not divide the tensor");
+        const int layout = wp_layout ? wp_layout[i0 + i] : LNN_W_OIHW;
+        if (layout != LNN_W_OIHW && layout != LNN_W_IOHW) return set_error(LNN_ERR_INVALID, std::string(who) + ": unknown weight layout");
+        const uint32_t C = (uint32_t)wp_c[i0 + i], O = (uint32_t)(a.n[i] / ((uint64_t)C * wp_kk[i0 + i]));
         a.wp[i] = wp[i0 + i];
         a.dKK[i] = make_fastdiv((uint32_t)wp_kk[i0 + i]);
-        a.dC[i] = make_fastdiv((uint32_t)wp_c[i0 + i]);
+        a.dIn[i] = make_fastdiv(layout == LNN_W_OIHW ? C : O);
+        a.wp_c[i] = layout == LNN_W_OIHW ? (int)C : -(int)C;
       }
     }
     if (most == 0) continue;

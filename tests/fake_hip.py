@@ -239,19 +239,22 @@ class FakeHip:
             self.sgd_update(dev, n, v, g, a, momentum, lr, nesterov)
         self.launches -= len(ns) - 1
 
-    def _refresh_copies(self, ns, vs, wps, cs, kks):
-        for n, v, wp, c, kk in zip(ns, vs, wps, cs, kks):
+    def _refresh_copies(self, ns, vs, wps, cs, kks, layouts):
+        for i, (n, v, wp, c, kk) in enumerate(zip(ns, vs, wps, cs, kks)):
             if wp is not None and n:
                 o = n // (c * kk)
-                self.f(wp, (o, kk, c))[...] = self.f(v, (o, c, kk)).transpose(0, 2, 1)
+                if layouts is not None and layouts[i] == real_api.W_IOHW:
+                    self.f(wp, (o, kk, c))[...] = self.f(v, (c, o, kk)).transpose(1, 2, 0)
+                else:
+                    self.f(wp, (o, kk, c))[...] = self.f(v, (o, c, kk)).transpose(0, 2, 1)
 
-    def sgd_update_multi_wp(self, dev, ns, vs, gs, accs, momentum, lr, nesterov, wps, cs, kks):
+    def sgd_update_multi_wp(self, dev, ns, vs, gs, accs, momentum, lr, nesterov, wps, cs, kks, layouts=None):
         self.sgd_update_multi(dev, ns, vs, gs, accs, momentum, lr, nesterov)
-        self._refresh_copies(ns, vs, wps, cs, kks)
+        self._refresh_copies(ns, vs, wps, cs, kks, layouts)
 
-    def adam_update_multi_wp(self, dev, ns, ts, gs, ms, vs, beta1, beta2, lr, wps, cs, kks):
+    def adam_update_multi_wp(self, dev, ns, ts, gs, ms, vs, beta1, beta2, lr, wps, cs, kks, layouts=None):
         self.adam_update_multi(dev, ns, ts, gs, ms, vs, beta1, beta2, lr)
-        self._refresh_copies(ns, ts, wps, cs, kks)
+        self._refresh_copies(ns, ts, wps, cs, kks, layouts)
 
     def adam_update_multi(self, dev, ns, ts, gs, ms, vs, beta1, beta2, lr):
         for n, t, g, m, v in zip(ns, ts, gs, ms, vs):

@@ -137,6 +137,52 @@ def test_permuted_weight_copy_is_shared_and_follows_the_weights(nn_backend, monk
     assert len(made) == 3
 
 
+def test_transposed_convolution_copy_survives_optimizer_steps(nn_backend, monkeypatch):
+    """The kernel of a transposed convolution is stored with swapped channel axes relative to the convolution whose
+    passes it borrows; its permuted copy is made straight from that storage once, and SGD and Adam steps write the
+    new values into it: no further permutation launch, and forward, input gradient and kernel gradient stay exact
+    on the updated kernel."""
+    nn = nn_backend
+    from litenn_amd.core.hip import api
+    made = []
+    real = api.conv2d_permute_weights
+    monkeypatch.setattr(api, 'conv2d_permute_weights', lambda *a: (made.append(1), real(*a))[1])
+    rs = np.random.RandomState(12)
+    for opt_name in ('sgd', 'adam'):
+        made.clear()
+        x_n = rs.randint(-2, 3, size=(2, 32, 5, 6)).astype(np.float32)
+        k_n = rs.randint(-2, 3, size=(32, 32, 3, 3)).astype(np.float32)
+        x_t, k_t = nn.Tensor_from_value(x_n), nn.Tensor_from_value(k_n)
+        opt = nn.optimizer.SGD([k_t], lr=0.5) if opt_name == 'sgd' else nn.optimizer.Adam([k_t], lr=0.25)
+
+        def step(expect_k, exact):
+            y = nn.conv2DTranspose(x_t, k_t, stride=2)
+            g_n = np.ones(tuple(y.shape), np.float32)
+            ry, rdi, rdk = conv2d_transpose_all(x_n, expect_k, g_n, 2, 1, 'same')
+            opt.zero_grad()
+            nn.backward({y: g_n}, grad_for_non_trainables=True)
+            if exact:
+                assert np.array_equal(y.np(), ry) and np.array_equal(x_t.get_grad().np(), rdi)
+                assert np.array_equal(k_t.get_grad().np(), rdk)
+            else:
+                # Adam's quotient m / (sqrt(v) + eps) is rounded differently on host and device; a copy that had
+                # missed the step would be off by 0.25 per weight, i.e. by units in every output
+                assert np.allclose(y.np(), ry, rtol=1e-3, atol=2e-2) and np.allclose(x_t.get_grad().np(), rdi, rtol=1e-3, atol=2e-2)
+            x_t.free_grad()
+            return rdk
+
+        dk = step(k_n, True)
+        assert len(made) == 1
+        opt.step()
+        if opt_name == 'sgd':
+            k2 = (k_n - 0.5 * dk).astype(np.float32)
+        else:   # first Adam step from zero moments: m = 0.1 g, v = 0.001 g^2
+            m, v = np.float32(0.1) * dk, np.float32(0.001) * dk * dk
+            k2 = (k_n - np.float32(0.25) * m / (np.sqrt(v) + np.float32(1e-7))).astype(np.float32)
+        step(k2, opt_name == 'sgd')
+        assert len(made) == 1, opt_name
+
+
 def test_conv2d_transpose_module_and_errors(nn_backend):
     nn = nn_backend
     rs = np.random.RandomState(2)

@@ -852,10 +852,11 @@ def test_multi_tensor_updates_equal_single_launches(hip):
 def test_multi_tensor_updates_refresh_permuted_copies(hip):
     """lnn_sgd_update_multi_wp_f32 / lnn_adam_update_multi_wp_f32: the same new values and optimizer state as the
     plain multi-tensor calls, bit for bit, and for every tensor that brings a permuted copy the copy equals
-    Wp[o][tap][c] of the new values; tensors without a copy, an empty tensor and more tensors than one launch holds
+    Wp[o][tap][c] of the new values, for tensors stored [O][C][taps] and [C][O][taps]; tensors without a copy, an empty tensor and more tensors than one launch holds
     among them.  A copy whose channel and tap counts do not divide the tensor is refused."""
     rs = np.random.RandomState(78)
     shapes = [(32, 32, 9), None, (64, 3, 49), (5, 7, 1), None, (40, 24, 25), (8, 130, 4)] + [None] * 12 + [(3, 5, 6)]
+    lays = [hip.W_OIHW, 0, hip.W_IOHW, hip.W_IOHW, 0, hip.W_OIHW, hip.W_IOHW] + [0] * 12 + [hip.W_IOHW]   # (O, C, KK) above
     sizes = [int(np.prod(sh)) if sh else 37 + i for i, sh in enumerate(shapes)]
     sizes[4] = 0
     mk = lambda: [rs.standard_normal(max(n, 1)).astype(np.float32) for n in sizes]
@@ -871,16 +872,18 @@ def test_multi_tensor_updates_refresh_permuted_copies(hip):
         wptrs = [w.ptr if w is not None else None for w in wps]
         if kind == 'adam':
             hip.adam_update_multi(0, sizes, pp[0], pp[1], pp[2], pp[3], 0.9, 0.999, 1e-2)
-            hip.adam_update_multi_wp(0, sizes, pf[0], pf[1], pf[2], pf[3], 0.9, 0.999, 1e-2, wptrs, cs, kks)
+            hip.adam_update_multi_wp(0, sizes, pf[0], pf[1], pf[2], pf[3], 0.9, 0.999, 1e-2, wptrs, cs, kks, lays)
         else:
             hip.sgd_update_multi(0, sizes, pp[0], pp[1], pp[2], 0.9, 1e-2, kind == 'sgd_nesterov')
-            hip.sgd_update_multi_wp(0, sizes, pf[0], pf[1], pf[2], 0.9, 1e-2, kind == 'sgd_nesterov', wptrs, cs, kks)
+            hip.sgd_update_multi_wp(0, sizes, pf[0], pf[1], pf[2], 0.9, 1e-2, kind == 'sgd_nesterov', wptrs, cs, kks, lays)
         for col_p, col_f in zip(plain, fused):
             for x, y in zip(col_p, col_f):
                 assert np.array_equal(x.get(), y.get())
-        for sh, w, v in zip(shapes, wps, fused[0]):
-            if sh:
-                assert np.array_equal(w.get().reshape(sh[0], sh[2], sh[1]), v.get().reshape(sh).transpose(0, 2, 1)), (kind, sh)
+        for sh, lay, w, v in zip(shapes, lays, wps, fused[0]):
+            if sh:   # the tensor is stored [O][C][KK], or [C][O][KK] with swapped channel axes
+                O, C, KK = sh
+                want = v.get().reshape(O, C, KK).transpose(0, 2, 1) if lay == hip.W_OIHW else v.get().reshape(C, O, KK).transpose(1, 2, 0)
+                assert np.array_equal(w.get().reshape(O, KK, C), want), (kind, sh, lay)
     with pytest.raises(hip.HipException) as e:
         hip.sgd_update_multi_wp(0, [10], [fused[0][0].ptr], [fused[1][0].ptr], [fused[2][0].ptr], 0.9, 1e-2, False,
                                 [wps[0].ptr], [3], [3])
