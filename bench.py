@@ -333,6 +333,91 @@ def bench_matmul(api, steps, warmup, n=4096, cpu=True):
     return res
 
 
+def bench_dense(api, steps, warmup, batch=32, n_in=4096, n_out=4096, cpu=True):
+    """Dense layer x[batch, in] @ w[in, out] + bias and its backward (module/Dense.py:44-48, matmul.py:64-72): at small
+    batch every pass streams the weight matrix (or its gradient) once, so HBM and the matrix cores bound it about
+    equally; each pass is reported against the larger of its two minimum times."""
+    rs = np.random.RandomState(0)
+    x = rs.uniform(-1, 1, (batch, n_in)).astype(np.float32)
+    w = rs.normal(0, np.sqrt(2.0 / n_in), (n_in, n_out)).astype(np.float32)
+    b = rs.normal(0, 0.1, n_out).astype(np.float32)
+    dy = rs.normal(0, 1, (batch, n_out)).astype(np.float32)
+    X, W, Bi, dY = Dev(api, x), Dev(api, w), Dev(api, b), Dev(api, dy)
+    Y, dX, dW, dB = Dev(api, shape=(batch, n_out)), Dev(api, shape=(batch, n_in)), Dev(api, shape=(n_in, n_out)), Dev(api, shape=(n_out,))
+    flops = 2.0 * batch * n_in * n_out
+    nx, nw, ny = x.size, w.size, dy.size
+    bytes_pass = {'fwd': 4.0 * (nx + nw + n_out + ny), 'dX': 4.0 * (ny + nw + 2 * nx), 'dW': 4.0 * (nx + ny + 2 * nw),
+                  'dBias': 4.0 * (ny + 2 * n_out)}
+    flops_pass = {'fwd': flops, 'dX': flops, 'dW': flops, 'dBias': 0.0}
+    passes = {
+        'fwd': lambda: api.gemm_bias_act(0, 0, 0, 1, batch, n_out, n_in, X.ptr, n_in, 0, W.ptr, n_out, 0, Bi.ptr,
+                                         api.ACT_NONE, 0.0, Y.ptr, n_out, 0),
+        'dX': lambda: api.gemm(0, 0, 1, 1, batch, n_in, n_out, dY.ptr, n_out, 0, W.ptr, n_out, 0, dX.ptr, n_in, 0, 1),
+        'dW': lambda: api.gemm(0, 1, 0, 1, n_in, n_out, batch, X.ptr, n_in, 0, dY.ptr, n_out, 0, dW.ptr, n_out, 0, 1),
+        'dBias': lambda: api.bias_act_bwd(0, batch, n_out, 1, None, dY.ptr, api.ACT_NONE, 0.0, None, dB.ptr, 1),
+    }
+
+    def step():
+        for fn in passes.values():
+            fn()
+
+    wall_ms, cold_ms = timed_steps(step, lambda: api.synchronize(0), steps, warmup)
+    per_pass = {}
+    for k, fn in passes.items():
+        ms = time_events(api, fn, max(steps, 20))
+        t_mfma = flops_pass[k] / (PEAK_FP32_MFMA_TFLOPS * 1e9)    # ms
+        t_hbm = bytes_pass[k] / (PEAK_HBM_GBS * 1e6)
+        per_pass[k] = {'ms': ms, 'tflops': flops_pass[k] / ms / 1e9, 'frac_mfma': t_mfma / ms,
+                       'alg_gbs': bytes_pass[k] / ms / 1e6, 'frac_hbm': t_hbm / ms,
+                       'bound': 'mfma' if t_mfma >= t_hbm else 'hbm', 'frac_roofline': max(t_mfma, t_hbm) / ms}
+    # the dominant kernel: the pass furthest below its roofline among the three products
+    dom = min(('fwd', 'dX', 'dW'), key=lambda k: per_pass[k]['frac_roofline'])
+    pp = per_pass[dom]
+    if pp['bound'] == 'mfma':
+        roof = {'bound': 'mfma', 'kernel': dom, 'achieved': pp['tflops'], 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
+                'frac': pp['frac_mfma']}
+    else:
+        roof = {'bound': 'hbm', 'kernel': dom, 'achieved': pp['alg_gbs'], 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                'frac': pp['frac_hbm']}
+    name = f'cfgM_dense_b{batch}'
+    roof['traffic'] = MEASURED_TRAFFIC_BYTES.get(name, {}).get(dom)
+    dX.zero()
+    dW.zero()
+    dB.zero()
+    step()
+    res = {'metric': 'dense layer fwd+bwd fp32 TFLOP/s', 'value': 3 * flops / wall_ms / 1e9, 'unit': 'TFLOP/s',
+           'ms_per_step_cold': cold_ms, 'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S,
+           'ms_per_step': wall_ms, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32',
+           'data': 'synthetic',
+           'config': {'workload': f'{name}: x[{batch}, {n_in}] @ w[{n_in}, {n_out}] + bias, '
+                                  'step = fwd(+bias) + dX(+=) + dW(+=) + dBias(+=)'},
+           'samples_per_s': batch / wall_ms * 1e3, 'roofline': roof, 'passes': per_pass}
+    if cpu:
+        from oracle import refpath
+        times = []
+        ref = None
+        for i in range(3):
+            t0 = time.perf_counter()
+            ry = refpath.matmul(x, w) + b
+            rdx, rdw = refpath.matmul_bwd(x, w, dy)
+            if i > 0:
+                times.append(time.perf_counter() - t0)
+            ref = (ry, rdx, rdw)
+        cpu_s = float(np.median(times))
+        res['cpu_baseline'] = {'value': 3 * flops / cpu_s / 1e12, 'unit': 'TFLOP/s', 'cores': refpath.num_threads(),
+                               'kind': 'port', 'ms_per_step': cpu_s * 1e3,
+                               'sample': 'the full step (register-tiled GeMM forward, materialised transposes + GeMM for '
+                                         'both gradients, numpy bias add), median of 2 after 1 warm-up',
+                               'cpu_opencl': CPU_OPENCL}
+        got = (Y.get(), dX.get(), dW.get())
+        res['parity'] = {'checked_against': 'cpu_baseline outputs (fp32 reference data flow)',
+                         'max_rel_err': max(rel_err(g, r) for g, r in zip(got, ref)),
+                         'dbias_rel_err': rel_err(dB.get(), dy.astype(np.float64).sum(0)), 'tolerance': 1e-4}
+    for t in (X, W, Bi, dY, Y, dX, dW, dB):
+        t.free()
+    return res
+
+
 def bench_conv_transpose(api, steps, warmup, cpu=True):
     """Decoder layer: conv2DTranspose 256 -> 128, 5x5, stride 2, 'same', 16x16 -> 32x32, batch 16.  The three
     passes run on the convolution kernels with the roles swapped (forward = dgrad, dI = forward, dK = wgrad)."""
@@ -525,7 +610,7 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='run only a plain device copy of 256 MiB (three launches of the element-wise kernel) and exit: '
                          'the reference reading for the FETCH_SIZE / WRITE_SIZE counters')
-    ap.add_argument('--config', default='cfg3_vgg3x3', choices=list(CONV_CONFIGS) + ['cfg2_matmul', 'cfg5_encoder', 'cfgT_decoder', 'cfgD_depthwise'],
+    ap.add_argument('--config', default='cfg3_vgg3x3', choices=list(CONV_CONFIGS) + ['cfg2_matmul', 'cfg5_encoder', 'cfgT_decoder', 'cfgD_depthwise', 'cfgM_dense', 'cfgM_dense_b32', 'cfgM_dense_b256'],
                     help='workload of the JSON line (default: the headline configuration)')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -566,11 +651,22 @@ def main():
             r = bench_depthwise(api, args.steps, args.warmup, cpu=not args.no_cpu)
             f.write(json.dumps(r) + '\n')
             print(f'[bench] cfgD depthwise: {r["value"]:.0f} GB/s', file=sys.stderr, flush=True)
+            for bsz in (32, 256):
+                r = bench_dense(api, args.steps, args.warmup, batch=bsz, cpu=not args.no_cpu)
+                f.write(json.dumps(r) + '\n')
+                print(f'[bench] cfgM dense batch {bsz}: ' + ', '.join(f'{k} {v["ms"] * 1e3:.1f} us' for k, v in r['passes'].items()),
+                      file=sys.stderr, flush=True)
             r = bench_encoder(args.steps, args.warmup)
             f.write(json.dumps(r) + '\n')
             print(f'[bench] cfg5 encoder: {r["value"]:.0f} images/s, {r["ms_per_step"]:.3f} ms/step', file=sys.stderr,
                   flush=True)
-    if args.config == 'cfg2_matmul':
+    if args.config in ('cfgM_dense', 'cfgM_dense_b32'):
+        res = bench_dense(api, args.steps, args.warmup, batch=32, cpu=not args.no_cpu)
+        if args.config == 'cfgM_dense':   # the same layer at a batch where the matrix cores bound every pass
+            res['batch256'] = bench_dense(api, args.steps, args.warmup, batch=256, cpu=not args.no_cpu)
+    elif args.config == 'cfgM_dense_b256':
+        res = bench_dense(api, args.steps, args.warmup, batch=256, cpu=not args.no_cpu)
+    elif args.config == 'cfg2_matmul':
         res = bench_matmul(api, args.steps, args.warmup, cpu=not args.no_cpu)
     elif args.config == 'cfg5_encoder':
         res = bench_encoder(args.steps, args.warmup)

@@ -83,6 +83,16 @@ int lnn_gemm_f32(int dev, int trans_a, int trans_b, int batch, int M, int N, int
                  const float* A, int lda, int64_t stride_a,
                  const float* B, int ldb, int64_t stride_b,
                  float* C, int ldc, int64_t stride_c, int beta);
+/* C[b] = act(op(A[b]) * op(B[b]) + bias[n])   the product and the broadcast bias add that follows it in a dense
+ * layer (module/Dense.py:44-48: nn.matmul(x, weight) + bias; dual_wise_op.py:110-130 for the broadcast operand),
+ * and optionally the activation users put behind it (element_wise_op.py:208-222), in the product's only store:
+ * bit-identical to the separate kernels.  bias holds N values, one per column of C (the same for every batch
+ * item), or is NULL; act / slope as for lnn_conv2d_fwd_bias_act_f32 (declared below). */
+int lnn_gemm_bias_act_f32(int dev, int trans_a, int trans_b, int batch, int M, int N, int K,
+                          const float* A, int lda, int64_t stride_a,
+                          const float* B, int ldb, int64_t stride_b,
+                          const float* bias, int act, float slope,
+                          float* C, int ldc, int64_t stride_c);
 
 /* ---- convolution: replaces unfold2D + GeMM + transpose of conv2D.py:39-54.
  * Geometry as computed by InfoConv2D (InfoConv2D.py:41-77); only the left/top

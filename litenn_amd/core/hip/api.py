@@ -63,6 +63,8 @@ SIGNATURES = {
     'lnn_event_destroy': [_c_int, _ptr],
     'lnn_gemm_f32': [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _ptr, _c_int, _c_i64,
                      _ptr, _c_int, _c_i64, _ptr, _c_int, _c_i64, _c_int],
+    'lnn_gemm_bias_act_f32': [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _ptr, _c_int, _c_i64,
+                              _ptr, _c_int, _c_i64, _ptr, _c_int, _c_f32, _ptr, _c_int, _c_i64],
     'lnn_conv2d_fwd_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_fwd_bias_act_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int, ctypes.c_float, _ptr],
     'lnn_depthwise_conv2d_fwd_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
@@ -209,6 +211,13 @@ class Event:
 def gemm(dev, trans_a, trans_b, batch, M, N, K, A, lda, sa, B, ldb, sb, C, ldc, sc, beta):
     check(lib.lnn_gemm_f32(dev, int(trans_a), int(trans_b), batch, M, N, K, A, lda, sa, B, ldb, sb, C, ldc, sc,
                            int(beta)))
+
+
+def gemm_bias_act(dev, trans_a, trans_b, batch, M, N, K, A, lda, sa, B, ldb, sb, bias, act, slope, C, ldc, sc):
+    """C = act(op(A) . op(B) + bias[n]); bias (N values, one per column of C) may be None; act as for
+    conv2d_fwd_bias_act (ACT_NONE / ACT_LEAKY_RELU)."""
+    check(lib.lnn_gemm_bias_act_f32(dev, int(trans_a), int(trans_b), batch, M, N, K, A, lda, sa, B, ldb, sb, bias,
+                                    int(act), float(slope), C, ldc, sc))
 
 
 def conv_desc(N, C, IH, IW, O, KH, KW, OH, OW, PADL, PADT, stride, dilation):

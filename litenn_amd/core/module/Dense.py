@@ -26,6 +26,9 @@ class Dense(nn.Module):
         super().__init__(saveables=['weight', 'bias'])
 
     def forward(self, x, **kwargs):
+        # nn.matmul(x, weight) + bias (module/Dense.py:44-48) with the bias added in the product's epilogue
+        if self.use_bias and x.shape.rank == 2:
+            return nc.op.matmul_bias_act(x, self.weight, self.bias)
         x = nn.matmul(x, self.weight)
         if self.use_bias:
             x = x + self.bias

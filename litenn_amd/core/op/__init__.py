@@ -27,7 +27,8 @@ from .dual_wise_op import (dual_wise_op,
                            sub_op as sub,
                            mul_op as mul)
 from .matmul import (matmul_op as matmul,
-                     matmulc_op as matmulc)
+                     matmulc_op as matmulc,
+                     matmul_bias_act)
 from .reduce import (reduce_mean_op as reduce_mean,
                      reduce_sum_op as reduce_sum)
 from .reshape import reshape

@@ -80,8 +80,11 @@ class _EpilogueGrad:
     operand) - in the same launch as pre() when it runs first, which it does whenever the bias gradient is
     wanted at all."""
 
-    def __init__(self, act, alpha):
+    def __init__(self, act, alpha, dims=None):
         self.act, self.alpha = act, alpha
+        # (batch, channels, elements per channel plane) of the output: NCHW by default; a dense layer's (rows, out_ch)
+        # is the same with planes of one element
+        self.dims = dims if dims is not None else (lambda shape: (shape[0], shape[1], shape[2] * shape[3]))
         self.key, self.value = None, None      # key: (backward sweep, the dO tensor the value was formed from)
 
     def _drop(self):
@@ -92,7 +95,7 @@ class _EpilogueGrad:
         return (sweep is not None and self.key is not None and self.key[0] == sweep and self.key[1] is dO_t)
 
     def _run(self, O_t, dO_t, want_pre, bias_grad):
-        N, O, H, W = tuple(dO_t.shape)
+        N, O, HW = self.dims(tuple(dO_t.shape))
         pre = None
         if want_pre:
             pre = nn.Tensor(dO_t.shape)
@@ -114,7 +117,7 @@ class _EpilogueGrad:
             outs = list(outs)
             dpre = outs.pop(0) if pre is not None else None
             dbias = outs.pop(0) if bias_grad is not None else None
-            api.bias_act_bwd(dev, N, O, H * W, y, dy, self.act, self.alpha, dpre, dbias, beta)
+            api.bias_act_bwd(dev, N, O, HW, y, dy, self.act, self.alpha, dpre, dbias, beta)
         launch(run, *args)
 
     def pre(self, O_t, dO_t):

@@ -45,7 +45,8 @@ constexpr uint64_t kMaxTensorBytes = 0x7fffffffull;   // raw buffer descriptors 
 
 // launchers implemented in the kernel translation units
 int launch_gemm(DeviceCtx* ctx, int ta, int tb, int batch, int M, int N, int K, const float* A, int lda,
-                long long sA, const float* B, int ldb, long long sB, float* C, int ldc, long long sC, int beta);
+                long long sA, const float* B, int ldb, long long sB, float* C, int ldc, long long sC, int beta,
+                const float* bias = nullptr, int act = 0, float slope = 0.0f);   // bias: one value per column of C
 // Wp: the weights in the permuted layout (made by launch_permute_weights), or null; W may be null when Wp is given
 int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta,
                     const float* bias, int act, float slope, const float* Wp = nullptr);

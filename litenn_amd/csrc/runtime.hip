@@ -308,6 +308,15 @@ int lnn_gemm_f32(int dev, int trans_a, int trans_b, int batch, int M, int N, int
   return launch_gemm(ctx, trans_a, trans_b, batch, M, N, K, A, lda, stride_a, B, ldb, stride_b, C, ldc, stride_c, beta);
 }
 
+int lnn_gemm_bias_act_f32(int dev, int trans_a, int trans_b, int batch, int M, int N, int K, const float* A, int lda,
+                          int64_t stride_a, const float* B, int ldb, int64_t stride_b, const float* bias, int act,
+                          float slope, float* C, int ldc, int64_t stride_c) {
+  CTX(dev);
+  if (act != LNN_ACT_NONE && act != LNN_ACT_LEAKY_RELU) return set_error(LNN_ERR_INVALID, "gemm_bias_act: unknown activation");
+  return launch_gemm(ctx, trans_a, trans_b, batch, M, N, K, A, lda, stride_a, B, ldb, stride_b, C, ldc, stride_c, 0, bias,
+                     act, slope);
+}
+
 int lnn_conv2d_fwd_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* W, float* Y, int beta) {
   CTX(dev);
   return launch_conv_fwd(ctx, d, X, W, Y, beta, nullptr, 0, 0.0f);

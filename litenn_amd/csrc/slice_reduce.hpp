@@ -1,0 +1,155 @@
+// Sum of the K slices of a split-K pass: the partial sums part[slice][m][col] of a GEMM-shaped result, added in a
+// fixed order into the final tensor, with the output mapping, '+=' and the bias / activation epilogue applied there.
+// Shared by the convolution passes and the plain GEMM; everything has internal linkage (each translation unit that
+// includes this carries its own copy of these small kernels).
+#pragma once
+#include "common.hpp"
+
+namespace lnn {
+namespace {
+
+// out[map(m, col)] (+)= sum over slices of part[slice][m][col], slices added in a
+// fixed order.  A block covers 32 consecutive elements (one 128-byte line per
+// slice row) with 8 lanes per element striding over the slices.  Elements of
+// units >= last_unit0 (unit = (m >> bm_log) * per_mt + (col >> uw_log)) have
+// only slices_last slices.
+struct ReduceArgs {
+  int n, slices, slices_last, beta, ncols;
+  int bm_log, uw_log, per_mt, last_unit0;
+  FastDiv dN;
+  OutMap om;
+  PostOp post;
+};
+__device__ __forceinline__ void reduce_body(float* out, const float* part, const ReduceArgs& a) {
+  __shared__ float red[8][33];
+  const int li = threadIdx.x & 31, ls = threadIdx.x >> 5;
+  const int i = blockIdx.x * 32 + li;
+  float s = 0.0f;
+  uint32_t m = 0, col = 0;
+  if (i < a.n) {
+    m = a.dN.div((uint32_t)i);
+    col = (uint32_t)i - m * (uint32_t)a.ncols;
+    const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
+    const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+    // the additions stay in slice order; unrolled so that several slices' loads are in flight together (many
+    // slices over a tiny output, the weight gradient of an image stem, would otherwise pay one latency per slice)
+#pragma unroll 8
+    for (int k = ls; k < ns; k += 8) s += part[(size_t)k * a.n + i];
+  }
+  red[ls][li] = s;
+  __syncthreads();
+  if (ls == 0 && i < a.n) {
+#pragma unroll
+    for (int k = 1; k < 8; ++k) s += red[k][li];
+    const uint32_t o = a.om.col(col) + m * (uint32_t)a.om.ld;
+    if (a.post.any()) s = a.post.apply(s, a.post.bias != nullptr ? a.post.bias[a.post.bias_col ? col : m] : 0.0f);
+    out[o] = a.beta ? out[o] + s : s;
+  }
+}
+__global__ __launch_bounds__(256) void reduce_partials(float* out, const float* part, ReduceArgs a) {
+  reduce_body(out, part, a);
+}
+
+// The same for ncols % 4 == 0 with 128-bit reads: a block covers 128 consecutive
+// elements, 8 lanes per group of 4 striding over the slices.
+__device__ __forceinline__ void reduce_body4(float* out, const float* part, const ReduceArgs& a) {
+  __shared__ float red[8][128];
+  const int q = threadIdx.x & 31, ls = threadIdx.x >> 5;
+  const int i4 = (blockIdx.x * 32 + q) * 4;
+  f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (i4 < a.n) {
+    const uint32_t m = a.dN.div((uint32_t)i4), col = (uint32_t)i4 - m * (uint32_t)a.ncols;
+    const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
+    const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+#pragma unroll 4
+    for (int k = ls; k < ns; k += 8) s += *reinterpret_cast<const f32x4*>(&part[(size_t)k * a.n + i4]);
+  }
+  *reinterpret_cast<f32x4*>(&red[ls][4 * q]) = s;
+  __syncthreads();
+  const int e = threadIdx.x, i = blockIdx.x * 128 + e;
+  if (e < 128 && i < a.n) {
+    float t = red[0][e];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) t += red[k][e];
+    const uint32_t m = a.dN.div((uint32_t)i), col = (uint32_t)i - m * (uint32_t)a.ncols;
+    const uint32_t o = a.om.col(col) + m * (uint32_t)a.om.ld;
+    if (a.post.any()) t = a.post.apply(t, a.post.bias != nullptr ? a.post.bias[a.post.bias_col ? col : m] : 0.0f);
+    out[o] = a.beta ? out[o] + t : t;
+  }
+}
+// ... and with at most kFewSlices slices: nothing to gain from lanes striding over the slices (most of them would
+// idle), so every thread adds up the slices of four consecutive elements itself, all its loads in flight together,
+// and a block covers 1024 elements, which leave through LDS so that consecutive lanes store consecutive elements.
+// The additions are the ones reduce_body4 makes, in the same order.
+constexpr int kFewSlices = 8;
+template <int NS>
+__device__ __forceinline__ f32x4 sum_slices(const float* part, size_t n, int i4, int ns) {
+  f32x4 v[NS];
+#pragma unroll
+  for (int k = 0; k < NS; ++k) v[k] = *reinterpret_cast<const f32x4*>(&part[(size_t)(k < ns ? k : 0) * n + i4]);
+  f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+  const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int k = 0; k < NS; ++k) s += k < ns ? v[k] : zero;
+  return s;
+}
+__device__ __forceinline__ void reduce_body4_few(float* out, const float* part, const ReduceArgs& a) {
+  __shared__ float red[1024];
+  const int i4 = ((int)blockIdx.x * 256 + (int)threadIdx.x) * 4;
+  f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (i4 < a.n) {
+    const uint32_t m = a.dN.div((uint32_t)i4), col = (uint32_t)i4 - m * (uint32_t)a.ncols;
+    const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
+    const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+    // the slice count of the problem is uniform: one straight run of loads per count; a unit of the last chunk,
+    // which may have fewer slices, reads slice 0 again in their place and adds zeros
+    switch (a.slices) {
+      case 2: s = sum_slices<2>(part, (size_t)a.n, i4, ns); break;
+      case 3: s = sum_slices<3>(part, (size_t)a.n, i4, ns); break;
+      case 4: s = sum_slices<4>(part, (size_t)a.n, i4, ns); break;
+      case 5: s = sum_slices<5>(part, (size_t)a.n, i4, ns); break;
+      case 6: s = sum_slices<6>(part, (size_t)a.n, i4, ns); break;
+      case 7: s = sum_slices<7>(part, (size_t)a.n, i4, ns); break;
+      default: s = sum_slices<8>(part, (size_t)a.n, i4, ns); break;
+    }
+  }
+  *reinterpret_cast<f32x4*>(&red[4 * threadIdx.x]) = s;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = (int)threadIdx.x + 256 * j, i = (int)blockIdx.x * 1024 + e;
+    if (i < a.n) {
+      float t = red[e];
+      const uint32_t m = a.dN.div((uint32_t)i), col = (uint32_t)i - m * (uint32_t)a.ncols;
+      const uint32_t o = a.om.col(col) + m * (uint32_t)a.om.ld;
+      if (a.post.any()) t = a.post.apply(t, a.post.bias != nullptr ? a.post.bias[a.post.bias_col ? col : m] : 0.0f);
+      out[o] = a.beta ? out[o] + t : t;
+    }
+  }
+}
+// elements per block of the 128-bit reductions
+__host__ __device__ inline int reduce4_block(const ReduceArgs& a) { return a.slices <= kFewSlices ? 1024 : 128; }
+__global__ __launch_bounds__(256) void reduce_partials4(float* out, const float* part, ReduceArgs a) {
+  if (a.slices <= kFewSlices) reduce_body4_few(out, part, a);
+  else reduce_body4(out, part, a);
+}
+
+// The reductions of the pixel classes of one strided dgrad in one launch: blockIdx.y = class.
+constexpr int kMaxReduceBatch = 4;
+struct ReduceBatch {
+  ReduceArgs r[kMaxReduceBatch];
+  float* out[kMaxReduceBatch];
+  const float* part[kMaxReduceBatch];
+  int vec[kMaxReduceBatch];
+};
+__global__ __launch_bounds__(256) void reduce_partials_batch(ReduceBatch b) {
+  const int c = blockIdx.y;
+  const int per_block = b.vec[c] ? reduce4_block(b.r[c]) : 32;
+  if ((long long)blockIdx.x * per_block >= b.r[c].n) return;   // the whole block leaves together
+  if (b.vec[c] && b.r[c].slices <= kFewSlices) reduce_body4_few(b.out[c], b.part[c], b.r[c]);
+  else if (b.vec[c]) reduce_body4(b.out[c], b.part[c], b.r[c]);
+  else reduce_body(b.out[c], b.part[c], b.r[c]);
+}
+
+}  // namespace
+}  // namespace lnn

@@ -528,6 +528,25 @@ __global__ __launch_bounds__(256) void bias_act_bwd_kernel(int N, int O, int HW,
   if (threadIdx.x == 0) part[(size_t)o * slices + sl] = (red[0] + red[1]) + (red[2] + red[3]);
 }
 
+// The same for planes of one element, a dense layer's y[rows][O]: a thread owns a feature and walks down its
+// slice of the rows (consecutive threads read consecutive floats of a row).
+__global__ __launch_bounds__(256) void bias_act_bwd_rows_kernel(int N, int O, int slices, const float* __restrict__ y,
+                                                                const float* dy, int act, float slope, float* dpre,
+                                                                float* __restrict__ part) {
+  const int o = blockIdx.x * 256 + threadIdx.x, sl = blockIdx.y;
+  if (o >= O) return;
+  const int r0 = (int)((long long)N * sl / slices), r1 = (int)((long long)N * (sl + 1) / slices);
+  float acc = 0.0f;
+  for (int r = r0; r < r1; ++r) {
+    const size_t e = (size_t)r * O + o;
+    float g = dy[e];
+    if (act == LNN_ACT_LEAKY_RELU) g *= y[e] >= 0.0f ? 1.0f : slope;
+    if (dpre) dpre[e] = g;
+    acc += g;
+  }
+  if (part) part[(size_t)o * slices + sl] = acc;
+}
+
 __global__ void bias_act_bwd_finish_kernel(int O, int slices, const float* __restrict__ part, float* __restrict__ dbias,
                                            int beta) {
   const int o = blockIdx.x * blockDim.x + threadIdx.x;
@@ -544,6 +563,27 @@ int launch_bias_act_bwd(DeviceCtx* ctx, int N, int O, int HW, const float* y, co
   if (!dy || (act != LNN_ACT_NONE && !y)) return set_error(LNN_ERR_INVALID, "bias_act_bwd: null pointer");
   if (!dpre && !dbias) return set_error(LNN_ERR_INVALID, "bias_act_bwd: nothing to compute");
   if ((uint64_t)N * O * HW * 4 > kMaxTensorBytes) return set_error(LNN_ERR_UNSUPPORTED, "bias_act_bwd: a tensor of 2 GiB or more");
+  if (HW == 1) {
+    const int blocks = (O + 255) / 256;
+    long long sl = ((long long)ctx->cus * 4 + blocks - 1) / blocks;
+    if (sl > N) sl = N;
+    if (sl > 64) sl = 64;
+    float* part1 = nullptr;
+    if (dbias) {
+      int st = ensure_workspace(ctx, (size_t)O * sl * sizeof(float));
+      if (st != LNN_OK) return st;
+      part1 = static_cast<float*>(ctx->ws);
+    }
+    hipLaunchKernelGGL(bias_act_bwd_rows_kernel, dim3((unsigned)blocks, (unsigned)sl), dim3(256), 0, ctx->stream, N, O, (int)sl, y,
+                       dy, act, slope, dpre, part1);
+    LNN_HIP(hipGetLastError());
+    if (dbias) {
+      hipLaunchKernelGGL(bias_act_bwd_finish_kernel, dim3((O + 255) / 256), dim3(256), 0, ctx->stream, O, (int)sl, part1,
+                         dbias, beta ? 1 : 0);
+      LNN_HIP(hipGetLastError());
+    }
+    return LNN_OK;
+  }
   if (O > 65535) return set_error(LNN_ERR_UNSUPPORTED, "bias_act_bwd: more than 65535 channels");
   const int ppp = (HW + kEpiPiece - 1) / kEpiPiece;
   const long long total = (long long)N * ppp;

@@ -1458,9 +1458,10 @@ struct ConvWgradBAnyC {
 // it is stored ('=' only): y = f(acc + bias[m]), f = identity or leaky ReLU
 // (x >= 0 ? x : slope * x, the same selection the pointwise kernel makes).
 struct PostOp {
-  const float* bias;   // one value per output row m, or null
+  const float* bias;   // one value per output row m (per column n with bias_col), or null
   int act;             // 0 none, 1 leaky ReLU
   float slope;
+  int bias_col;        // 0: bias[m] (a convolution's output channel), 1: bias[n] (a dense layer's output feature)
   __host__ __device__ bool any() const { return bias != nullptr || act != 0; }
   __device__ __forceinline__ float apply(float v, float b) const {
     v += b;
@@ -1982,6 +1983,15 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
 #pragma unroll
         for (int r = 0; r < 16; ++r) buf_store(p.rc, elem(cb, roff[r]), acc[j][r] + old[j & 1][r]);
         cb = cbn;
+      }
+    } else if (p.post.any() && p.post.bias_col) {
+#pragma unroll
+      for (int j = 0; j < NTC; ++j) {
+        const uint32_t cb = col_off(j);
+        const int n = ng + (wn * NT + j) * 32 + i;
+        const float b = (p.post.bias != nullptr && n < p.Ncols) ? p.post.bias[n] : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) buf_store(p.rc, elem(cb, roff[r]), p.post.apply(acc[j][r], b));
       }
     } else if (p.post.any()) {
       float bv[16];

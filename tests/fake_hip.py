@@ -12,7 +12,7 @@ from oracle import (conv2d_fwd, conv2d_dx, conv2d_dw, unfold_index_map, unfold_T
 from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
-         'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'conv2d_permute_weights', 'conv2d_fwd_pw', 'conv2d_dgrad_pw', 'conv2d_wgrad_iohw', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
+         'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'gemm_bias_act', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'conv2d_permute_weights', 'conv2d_fwd_pw', 'conv2d_dgrad_pw', 'conv2d_wgrad_iohw', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
          'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal', 'bias_act_bwd', 'sgd_update_multi', 'sgd_update_multi_wp', 'adam_update_multi_wp', 'adam_update_multi']
 
 
@@ -79,6 +79,18 @@ class FakeHip:
         b = self.f(B, (batch, N, K) if tb else (batch, K, N)).astype(np.float64)
         r = np.matmul(a.transpose(0, 2, 1) if ta else a, b.transpose(0, 2, 1) if tb else b)
         self._put(self.f(C, (batch, M, N)), r, beta)
+
+    def gemm_bias_act(self, dev, ta, tb, batch, M, N, K, A, lda, sa, B, ldb, sb, bias, act, slope, C, ldc, sc):
+        self.launches += 1
+        assert lda == (M if ta else K) and ldb == (K if tb else N) and ldc == N, 'fake gemm: dense operands only'
+        a = self.f(A, (batch, K, M) if ta else (batch, M, K)).astype(np.float64)
+        b = self.f(B, (batch, N, K) if tb else (batch, K, N)).astype(np.float64)
+        r = np.matmul(a.transpose(0, 2, 1) if ta else a, b.transpose(0, 2, 1) if tb else b).astype(np.float32)
+        if bias is not None:
+            r = r + self.f(bias, (N,)).reshape(1, 1, -1)
+        if act == 1:
+            r = np.where(r >= 0, r, np.float32(slope) * r)
+        self._put(self.f(C, (batch, M, N)), r, 0)
 
     @staticmethod
     def _geom(d):

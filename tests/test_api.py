@@ -511,6 +511,50 @@ def test_conv2d_and_dense_modules(nn_backend):
     assert np.array_equal(conv.bias.get_grad().np(), gy.sum((0, 2, 3)))
 
 
+def test_dense_bias_in_the_product_epilogue(nn_backend):
+    """Dense.forward = nn.matmul(x, weight) + bias (module/Dense.py:44-48) with the bias added by the product's
+    epilogue: same values and same gradients as the two separate ops, also behind an activation and when the
+    gradients already hold something."""
+    import litenn_amd.core as nc
+    nn = nn_backend
+    rs = np.random.RandomState(8)
+    for rows, n_in, n_out in ((5, 12, 20), (32, 64, 256), (70, 16, 8)):
+        w = rs.randint(-4, 5, size=(n_in, n_out)).astype(np.float32)
+        b = rs.randint(-4, 5, size=(n_out,)).astype(np.float32)
+        xv = rs.randint(-4, 5, size=(rows, n_in)).astype(np.float32)
+        gy = rs.randint(-4, 5, size=(rows, n_out)).astype(np.float32)
+        dense = nn.Dense(n_in, n_out, weight_initializer=nn.initializer.NumpyArray(w),
+                         bias_initializer=nn.initializer.NumpyArray(b))
+        x = nn.Tensor_from_value(xv)
+        y = dense(x)
+        assert y.shape == (rows, n_out)
+        want = xv.astype(np.float64) @ w + b
+        assert np.array_equal(y.np(), want)
+        nn.backward({y: gy}, grad_for_non_trainables=True)
+        assert np.array_equal(x.get_grad().np(), gy.astype(np.float64) @ w.T)
+        assert np.array_equal(dense.weight.get_grad().np(), xv.T.astype(np.float64) @ gy)
+        assert np.array_equal(dense.bias.get_grad().np(), gy.sum(0))
+        # a second sweep accumulates into the same gradients
+        y = dense(x)
+        nn.backward({y: gy}, grad_for_non_trainables=True)
+        assert np.array_equal(dense.bias.get_grad().np(), 2 * gy.sum(0))
+        assert np.array_equal(dense.weight.get_grad().np(), 2 * (xv.T.astype(np.float64) @ gy))
+        # the fused activation: leaky_relu(x @ w + b)
+        x2, w2, b2 = nn.Tensor_from_value(xv), nn.Tensor_from_value(w), nn.Tensor_from_value(b)
+        z = nc.op.matmul_bias_act(x2, w2, b2, leaky_relu_alpha=0.5)
+        pre = want
+        assert np.array_equal(z.np(), np.where(pre >= 0, pre, 0.5 * pre))
+        nn.backward({z: gy}, grad_for_non_trainables=True)
+        dpre = gy * np.where(pre >= 0, 1.0, 0.5)
+        assert np.array_equal(b2.get_grad().np(), dpre.sum(0))
+        assert np.array_equal(w2.get_grad().np(), xv.T.astype(np.float64) @ dpre)
+        assert np.array_equal(x2.get_grad().np(), dpre @ w.T.astype(np.float64))
+    with pytest.raises(ValueError):
+        nc.op.matmul_bias_act(nn.Tensor((4, 6)), nn.Tensor((6, 8)), nn.Tensor((7,)))
+    with pytest.raises(ValueError):
+        nc.op.matmul_bias_act(nn.Tensor((4, 6)), nn.Tensor((6, 8)), None, leaky_relu_alpha=0.0)
+
+
 def test_shallow_mode_allocates_nothing(nn_backend):
     nn = nn_backend
 
