@@ -281,6 +281,21 @@ int lnn_adam_update_multi_wp_f32(int dev, int count, const uint64_t* n, float* c
                                  float* const* m, float* const* v, float beta1, float beta2, float lr, float* const* wp,
                                  const int32_t* wp_c, const int32_t* wp_kk, const int32_t* wp_layout);
 
+/* The same two multi-tensor updates with learning-rate dropout (Optimizer.py:186-203): inside each of the reference's
+ * update kernels element gid of a tensor takes lr = 0 where hash_float_uint(gid + seed) <= lr_dropout, the seed a
+ * fresh np.random.randint(2^31) per kernel launch (Optimizer.py:178-182), the hash the counter hash of the device
+ * initialisers below.  seeds: SGD two per tensor - {accumulator kernel, value kernel} (SGD.py:42-74; the second
+ * matters with nesterov only) - Adam one per tensor (Adam.py:61-72); lr_dropout == 0 ignores them (may be NULL).
+ * wp .. wp_layout as above, all NULL for tensors without permuted copies. */
+int lnn_sgd_update_multi_lrd_f32(int dev, int count, const uint64_t* n, float* const* v, const float* const* g,
+                                 float* const* acc, float momentum, float lr, int nesterov, float lr_dropout,
+                                 const uint32_t* seeds, float* const* wp, const int32_t* wp_c, const int32_t* wp_kk,
+                                 const int32_t* wp_layout);
+int lnn_adam_update_multi_lrd_f32(int dev, int count, const uint64_t* n, float* const* t, const float* const* g,
+                                  float* const* m, float* const* v, float beta1, float beta2, float lr, float lr_dropout,
+                                  const uint32_t* seeds, float* const* wp, const int32_t* wp_c, const int32_t* wp_kk,
+                                  const int32_t* wp_layout);
+
 /* On-device random initialisers: element i is drawn from a counter hash of (uint32)(i + seed), so a tensor
  * is filled in place without host staging (initializer/RandomUniform.py:13-27, RandomNormal.py:10-30; the PCG
  * hashes of CLKernelHelper.py:210-228).  The reference draws seed = np.random.randint(2^31) on the host.

@@ -93,6 +93,8 @@ SIGNATURES = {
     'lnn_adam_update_multi_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32],
     'lnn_sgd_update_multi_wp_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int, _ptr, _ptr, _ptr, _ptr],
     'lnn_adam_update_multi_wp_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32, _ptr, _ptr, _ptr, _ptr],
+    'lnn_sgd_update_multi_lrd_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_int, _c_f32, _ptr, _ptr, _ptr, _ptr, _ptr],
+    'lnn_adam_update_multi_lrd_f32': [_c_int, _c_int, _ptr, _ptr, _ptr, _ptr, _ptr, _c_f32, _c_f32, _c_f32, _c_f32, _ptr, _ptr, _ptr, _ptr, _ptr],
     'lnn_bias_act_bwd_f32': [_c_int, _c_int, _c_int, _c_int, _ptr, _ptr, _c_int, _c_f32, _ptr, _ptr, _c_int],
     'lnn_random_uniform_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
     'lnn_random_normal_f32': [_c_int, _ptr, _c_u64, _c_u32, _c_f64, _c_f64],
@@ -401,6 +403,34 @@ def adam_update_multi_wp(dev, ns, ts, gs, ms, vs, beta1, beta2, lr, wps, cs, kks
     check(lib.lnn_adam_update_multi_wp_f32(dev, count, (ctypes.c_uint64 * count)(*ns), _ptr_array(ts), _ptr_array(gs),
                                            _ptr_array(ms), _ptr_array(vs), float(beta1), float(beta2), float(lr),
                                            _ptr_array(wps), (ctypes.c_int32 * count)(*cs), (ctypes.c_int32 * count)(*kks), lay))
+
+
+def _wp_arrays(count, wps, cs, kks, layouts):
+    if wps is None:
+        return None, None, None, None
+    lay = (ctypes.c_int32 * count)(*layouts) if layouts is not None else None
+    return _ptr_array(wps), (ctypes.c_int32 * count)(*cs), (ctypes.c_int32 * count)(*kks), lay
+
+
+def sgd_update_multi_lrd(dev, ns, vs, gs, accs, momentum, lr, nesterov, lr_dropout, seeds, wps=None, cs=None, kks=None,
+                         layouts=None):
+    """sgd_update_multi(_wp) with learning-rate dropout: seeds holds two uint32 per tensor (accumulator kernel, value
+    kernel), as the reference draws them (Optimizer.py:178-182)."""
+    count = len(ns)
+    check(lib.lnn_sgd_update_multi_lrd_f32(dev, count, (ctypes.c_uint64 * count)(*ns), _ptr_array(vs), _ptr_array(gs),
+                                           _ptr_array(accs), float(momentum), float(lr), 1 if nesterov else 0,
+                                           float(lr_dropout), (ctypes.c_uint32 * (2 * count))(*seeds),
+                                           *_wp_arrays(count, wps, cs, kks, layouts)))
+
+
+def adam_update_multi_lrd(dev, ns, ts, gs, ms, vs, beta1, beta2, lr, lr_dropout, seeds, wps=None, cs=None, kks=None,
+                          layouts=None):
+    """adam_update_multi(_wp) with learning-rate dropout: one uint32 seed per tensor."""
+    count = len(ns)
+    check(lib.lnn_adam_update_multi_lrd_f32(dev, count, (ctypes.c_uint64 * count)(*ns), _ptr_array(ts), _ptr_array(gs),
+                                            _ptr_array(ms), _ptr_array(vs), float(beta1), float(beta2), float(lr),
+                                            float(lr_dropout), (ctypes.c_uint32 * count)(*seeds),
+                                            *_wp_arrays(count, wps, cs, kks, layouts)))
 
 
 def adam_update_multi(dev, ns, ts, gs, ms, vs, beta1, beta2, lr):

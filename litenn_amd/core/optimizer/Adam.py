@@ -25,7 +25,20 @@ class Adam(Optimizer):
         k, ns = len(ts), [t.shape.size for t in ts]
         grads, ms, vs = [t.get_grad() for t in ts], [self._ms[t.get_name()] for t in ts], [self._vs[t.get_name()] for t in ts]
         cached = cached_permuted_copies(ts)
-        if any(c is not None for c in cached):
+        seeds = self._kernel_seeds(k)     # one per tensor: the value kernel (Adam.py:76-86)
+        if self.lr_dropout != 0.0:
+            any_copy = any(c is not None for c in cached)
+            cs, kks = [c[2] if c else 0 for c in cached], [c[3] if c else 0 for c in cached]
+            lays = [c[4] if c else 0 for c in cached]
+
+            def run(dev, *p):
+                wps = p[4 * k:] if any_copy else None
+                api.adam_update_multi_lrd(dev, ns, p[:k], p[k:2 * k], p[2 * k:3 * k], p[3 * k:4 * k], self.beta_1, self.beta_2,
+                                          lr, self.lr_dropout, seeds, wps, cs if any_copy else None,
+                                          kks if any_copy else None, lays if any_copy else None)
+            launch(run, *ts, *grads, *ms, *vs, *([c[1] if c else None for c in cached] if any_copy else []))
+            keep_permuted_copies(ts, cached)
+        elif any(c is not None for c in cached):
             # convolution kernels whose permuted copy is cached: the update refreshes the copy in the same pass
             cs, kks = [c[2] if c else 0 for c in cached], [c[3] if c else 0 for c in cached]
             lays = [c[4] if c else 0 for c in cached]

@@ -11,15 +11,16 @@ class Optimizer(nc.ModuleBase):
 
      tensors_list   tensors to optimise (no references, gradients or op results)
      lr(0.001) lr_decay(0.0) clipnorm(0.0)
-     lr_dropout     must stay 0.0 here: it needs the reference's device-side
-                    hash generator, which is outside this package's scope
+     lr_dropout(0.0)  fraction of elements whose learning rate is zero in a step: element gid of a tensor is
+                      dropped where the counter hash of gid + seed, scaled to [0, 1], does not exceed it, with
+                      a fresh host-drawn seed per update kernel (Optimizer.py:178-203)
     """
 
     def __init__(self, _tensors_list, lr=0.001, lr_decay=0.0, lr_dropout=0.0, clipnorm=0.0, saveables=None):
         if _tensors_list is None:
             raise ValueError('_tensors_list must be specified.')
-        if lr_dropout != 0.0:
-            raise NotImplementedError('lr_dropout is not provided by this package')
+        if not 0.0 <= lr_dropout <= 1.0:
+            raise ValueError('lr_dropout must lie in [0, 1]')
         seen_ids, seen_names = set(), set()
         for t in _tensors_list:
             if id(t) in seen_ids:
@@ -77,6 +78,12 @@ class Optimizer(nc.ModuleBase):
 
     def _on_step(self):
         raise NotImplementedError()
+
+    def _kernel_seeds(self, count):
+        """One seed per update kernel the reference would launch, drawn from numpy's global generator exactly as
+        it does (Optimizer.py:178-182: np.random.randint(2147483648) per kernel.run, whether or not lr_dropout is on,
+        so the generator's state stays in step with the reference's)."""
+        return [int(np.random.randint(2147483648)) for _ in range(count)]
 
     def _current_lr(self):
         """lr / (1 + lr_decay * iteration)   (Optimizer.py:191-197)."""

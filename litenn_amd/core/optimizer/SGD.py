@@ -26,7 +26,20 @@ class SGD(Optimizer):
         # every tensor's update in one launch per device: pointers arrive as (values, gradients, accumulators)
         grads, accs = [t.get_grad() for t in ts], [self._accs[t.get_name()] for t in ts]
         cached = cached_permuted_copies(ts)
-        if any(c is not None for c in cached):
+        seeds = self._kernel_seeds(2 * k)     # per tensor: accumulator kernel, value kernel (SGD.py:76-83)
+        if self.lr_dropout != 0.0:
+            any_copy = any(c is not None for c in cached)
+            cs, kks = [c[2] if c else 0 for c in cached], [c[3] if c else 0 for c in cached]
+            lays = [c[4] if c else 0 for c in cached]
+
+            def run(dev, *p):
+                wps = p[3 * k:] if any_copy else None
+                api.sgd_update_multi_lrd(dev, ns, p[:k], p[k:2 * k], p[2 * k:3 * k], self.momentum, lr, self.nesterov,
+                                         self.lr_dropout, seeds, wps, cs if any_copy else None, kks if any_copy else None,
+                                         lays if any_copy else None)
+            launch(run, *ts, *grads, *accs, *([c[1] if c else None for c in cached] if any_copy else []))
+            keep_permuted_copies(ts, cached)
+        elif any(c is not None for c in cached):
             # convolution kernels whose permuted copy is cached: the update refreshes the copy in the same pass
             cs, kks = [c[2] if c else 0 for c in cached], [c[3] if c else 0 for c in cached]
             lays = [c[4] if c else 0 for c in cached]

@@ -19,7 +19,8 @@ int launch_sgd(DeviceCtx*, uint64_t, float*, const float*, float*, float, float,
 int launch_adam(DeviceCtx*, uint64_t, float*, const float*, float*, float*, float, float, float);
 int launch_random_uniform(DeviceCtx*, float*, uint64_t, uint32_t, double, double);
 int launch_update_multi(DeviceCtx*, int, int, const uint64_t*, float* const*, const float* const*, float* const*, float* const*,
-                        float, float, float, int, float* const*, const int32_t*, const int32_t*, const int32_t*);
+                        float, float, float, int, float* const*, const int32_t*, const int32_t*, const int32_t*, float = 0.0f,
+                        const uint32_t* = nullptr);
 int launch_bias_act_bwd(DeviceCtx*, int, int, int, const float*, const float*, int, float, float*, float*, int);
 int launch_random_normal(DeviceCtx*, float*, uint64_t, uint32_t, double, double);
 
@@ -508,6 +509,23 @@ int lnn_adam_update_multi_wp_f32(int dev, int count, const uint64_t* n, float* c
                                  const int32_t* wp_c, const int32_t* wp_kk, const int32_t* wp_layout) {
   CTX(dev);
   return launch_update_multi(ctx, 1, count, n, t, g, m, v, beta1, beta2, lr, 0, wp, wp_c, wp_kk, wp_layout);
+}
+
+int lnn_sgd_update_multi_lrd_f32(int dev, int count, const uint64_t* n, float* const* v, const float* const* g,
+                                 float* const* acc, float momentum, float lr, int nesterov, float lr_dropout,
+                                 const uint32_t* seeds, float* const* wp, const int32_t* wp_c, const int32_t* wp_kk,
+                                 const int32_t* wp_layout) {
+  CTX(dev);
+  return launch_update_multi(ctx, 0, count, n, v, g, acc, nullptr, momentum, 0.0f, lr, nesterov, wp, wp_c, wp_kk, wp_layout,
+                             lr_dropout, seeds);
+}
+
+int lnn_adam_update_multi_lrd_f32(int dev, int count, const uint64_t* n, float* const* t, const float* const* g,
+                                  float* const* m, float* const* v, float beta1, float beta2, float lr, float lr_dropout,
+                                  const uint32_t* seeds, float* const* wp, const int32_t* wp_c, const int32_t* wp_kk,
+                                  const int32_t* wp_layout) {
+  CTX(dev);
+  return launch_update_multi(ctx, 1, count, n, t, g, m, v, beta1, beta2, lr, 0, wp, wp_c, wp_kk, wp_layout, lr_dropout, seeds);
 }
 
 int lnn_bias_act_bwd_f32(int dev, int N, int O, int HW, const float* y, const float* dy, int act, float slope,

@@ -248,7 +248,17 @@ struct MultiArgs {
   float* wp[kMultiMax];
   FastDiv dKK[kMultiMax], dIn[kMultiMax];   // divide by KH*KW, by the inner of the tensor's two channel axes
   int wp_c[kMultiMax];                      // C of the copy; negative: the tensor is stored [C][O][tap]
+  // learning-rate dropout (Optimizer.py:199-202): seeds of the tensor's state-update and value-update kernels
+  uint32_t seed0[kMultiMax], seed1[kMultiMax];
 };
+__device__ __forceinline__ uint32_t hash_u32(uint32_t v);
+// lr, or 0 where the counter hash of (element + seed), scaled to [0, 1], does not exceed `drop`
+// (Optimizer.py:199-202: if (hash_float_uint(gid + seed) <= lr_dropout) lr = 0; drop == 0 compiles the test out there)
+__device__ __forceinline__ float dropped_lr(float lr, float drop, uint64_t i, uint32_t seed) {
+  if (drop == 0.0f) return lr;
+  const float u = (float)hash_u32((uint32_t)(i + seed)) * (1.0f / 4294967296.0f);
+  return u <= drop ? 0.0f : lr;
+}
 // parameter element i = (o*C + c)*KK + tap (or (c*O + o)*KK + tap for a tensor stored with swapped channel axes, as
 // a transposed convolution keeps its kernel) goes to Wp[(o*KK + tap)*C + c]
 __device__ __forceinline__ void store_permuted(const MultiArgs& a, int k, uint64_t i, float value) {
@@ -258,21 +268,22 @@ __device__ __forceinline__ void store_permuted(const MultiArgs& a, int k, uint64
   const uint32_t C = (uint32_t)(swapped ? -a.wp_c[k] : a.wp_c[k]), o = swapped ? lo : hi, c = swapped ? hi : lo;
   a.wp[k][((size_t)o * a.dKK[k].d + tap) * C + c] = value;
 }
-__global__ void sgd_multi_kernel(MultiArgs a, float momentum, float lr, int nesterov) {
+__global__ void sgd_multi_kernel(MultiArgs a, float momentum, float lr, int nesterov, float drop) {
   const int k = blockIdx.y;
   const uint64_t n = a.n[k];
   float* v = a.t[k];
   const float* g = a.g[k];
   float* acc = a.s0[k];
   for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    const float x = momentum * acc[i] - lr * g[i];
+    // the reference's two kernels per tensor (SGD.py:42-74) draw their dropout masks from separate seeds
+    const float x = momentum * acc[i] - dropped_lr(lr, drop, i, a.seed0[k]) * g[i];
     acc[i] = x;
-    const float nv = v[i] + (nesterov ? momentum * x - lr * g[i] : x);
+    const float nv = v[i] + (nesterov ? momentum * x - dropped_lr(lr, drop, i, a.seed1[k]) * g[i] : x);
     v[i] = nv;
     if (a.wp[k]) store_permuted(a, k, i, nv);
   }
 }
-__global__ void adam_multi_kernel(MultiArgs a, float beta1, float beta2, float lr) {
+__global__ void adam_multi_kernel(MultiArgs a, float beta1, float beta2, float lr, float drop) {
   const int k = blockIdx.y;
   const uint64_t n = a.n[k];
   float* t = a.t[k];
@@ -285,7 +296,7 @@ __global__ void adam_multi_kernel(MultiArgs a, float beta1, float beta2, float l
     const float vi = beta2 * v2[i] + (1.0f - beta2) * gi * gi;
     m[i] = mi;
     v2[i] = vi;
-    const float nt = t[i] + -lr * mi / (sqrtf(vi) + 1e-7f);
+    const float nt = t[i] + -dropped_lr(lr, drop, i, a.seed0[k]) * mi / (sqrtf(vi) + 1e-7f);
     t[i] = nt;
     if (a.wp[k]) store_permuted(a, k, i, nt);
   }
@@ -677,11 +688,15 @@ int launch_random_normal(DeviceCtx* ctx, float* out, uint64_t n, uint32_t seed, 
 // permuted copy Wp[o][tap][c] or null, its C and KH*KW, and how the tensor itself is stored
 int launch_update_multi(DeviceCtx* ctx, int kind, int count, const uint64_t* n, float* const* t, const float* const* g,
                         float* const* s0, float* const* s1, float p0, float p1, float lr, int flag, float* const* wp,
-                        const int32_t* wp_c, const int32_t* wp_kk, const int32_t* wp_layout) {
+                        const int32_t* wp_c, const int32_t* wp_kk, const int32_t* wp_layout, float drop,
+                        const uint32_t* seeds) {
   const char* who = kind ? "adam_update_multi" : "sgd_update_multi";
   if (count < 0) return set_error(LNN_ERR_INVALID, std::string(who) + ": negative count");
   if (count == 0) return LNN_OK;
   if (!n || !t || !g || !s0 || (kind && !s1)) return set_error(LNN_ERR_INVALID, std::string(who) + ": null array");
+  if (!(drop >= 0.0f && drop <= 1.0f)) return set_error(LNN_ERR_INVALID, std::string(who) + ": lr_dropout outside [0, 1]");
+  if (drop != 0.0f && !seeds) return set_error(LNN_ERR_INVALID, std::string(who) + ": lr_dropout needs seeds");
+  const int per = kind ? 1 : 2;   // seeds per tensor: SGD's two kernels, Adam's one
   for (int i0 = 0; i0 < count; i0 += kMultiMax) {
     const int nb = count - i0 < kMultiMax ? count - i0 : kMultiMax;
     MultiArgs a = {};
@@ -694,6 +709,8 @@ int launch_update_multi(DeviceCtx* ctx, int kind, int count, const uint64_t* n, 
       most = a.n[i] > most ? a.n[i] : most;
       a.dKK[i] = a.dIn[i] = FastDiv{0, 0, 1};
       a.wp_c[i] = 0;
+      a.seed0[i] = seeds ? seeds[per * (i0 + i)] : 0u;
+      a.seed1[i] = (seeds && per == 2) ? seeds[per * (i0 + i) + 1] : 0u;
       if (wp && wp[i0 + i] && a.n[i]) {
         if (!wp_c || !wp_kk || wp_c[i0 + i] <= 0 || wp_kk[i0 + i] <= 0 || a.n[i] % ((uint64_t)wp_c[i0 + i] * wp_kk[i0 + i]) != 0 ||
             a.n[i] > 0x7fffffffull)
@@ -709,8 +726,8 @@ int launch_update_multi(DeviceCtx* ctx, int kind, int count, const uint64_t* n, 
     }
     if (most == 0) continue;
     const dim3 grid(grid_for(most, ctx->cus / 2).x, (unsigned)nb);
-    if (kind) hipLaunchKernelGGL(adam_multi_kernel, grid, dim3(256), 0, ctx->stream, a, p0, p1, lr);
-    else hipLaunchKernelGGL(sgd_multi_kernel, grid, dim3(256), 0, ctx->stream, a, p0, lr, flag ? 1 : 0);
+    if (kind) hipLaunchKernelGGL(adam_multi_kernel, grid, dim3(256), 0, ctx->stream, a, p0, p1, lr, drop);
+    else hipLaunchKernelGGL(sgd_multi_kernel, grid, dim3(256), 0, ctx->stream, a, p0, lr, flag ? 1 : 0, drop);
     LNN_HIP(hipGetLastError());
   }
   return LNN_OK;

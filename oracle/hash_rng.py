@@ -82,6 +82,12 @@ def random_uniform(n, seed, low=0.0, high=1.0):
     return fma32(u, span, np.float32(low))
 
 
+def lr_dropout_mask(n, seed, lr_dropout):
+    """True where an optimizer kernel sets lr = 0 for element gid: hash_float_uint(gid+seed) <= lr_dropout in single
+    precision (optimizer/Optimizer.py:199-202; the threshold is a float literal there, CLDevice.py:93)."""
+    return _unit(hash_u32(_counter(n, seed))) <= np.float32(lr_dropout)
+
+
 def random_normal(n, seed, mean=0.0, stddev=1.0):
     """Box-Muller on hash_float2_uint(gid+seed) (RandomNormal.py:14-24).  A zero first half gives inf, as there."""
     x, y = hash_u32x2(_counter(n, seed), np.ones(n, dtype=np.uint64))

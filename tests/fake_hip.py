@@ -13,7 +13,7 @@ from litenn_amd.core.hip import api as real_api
 
 NAMES = ['device_count', 'device_info', 'release_device', 'malloc', 'free', 'mem_info', 'memcpy_h2d', 'memcpy_d2h',
          'memcpy_d2d', 'fill_u32', 'fill_f32', 'synchronize', 'gemm', 'gemm_bias_act', 'conv2d_fwd', 'conv2d_fwd_bias_act', 'conv2d_dgrad', 'conv2d_wgrad', 'conv2d_permute_weights', 'conv2d_fwd_pw', 'conv2d_dgrad_pw', 'conv2d_wgrad_iohw', 'depthwise_conv2d_fwd', 'depthwise_conv2d_dgrad', 'depthwise_conv2d_wgrad',
-         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal', 'bias_act_bwd', 'sgd_update_multi', 'sgd_update_multi_wp', 'adam_update_multi_wp', 'adam_update_multi']
+         'unfold2d', 'transpose', 'ew_fwd', 'ew_bwd', 'binary_bcast', 'reduce_sum', 'reduce_sum_bwd', 'sgd_update', 'adam_update', 'random_uniform', 'random_normal', 'bias_act_bwd', 'sgd_update_multi', 'sgd_update_multi_wp', 'adam_update_multi_wp', 'adam_update_multi', 'sgd_update_multi_lrd', 'adam_update_multi_lrd']
 
 
 class FakeHip:
@@ -272,6 +272,35 @@ class FakeHip:
         for n, t, g, m, v in zip(ns, ts, gs, ms, vs):
             self.adam_update(dev, n, t, g, m, v, beta1, beta2, lr)
         self.launches -= len(ns) - 1
+
+    def sgd_update_multi_lrd(self, dev, ns, vs, gs, accs, momentum, lr, nesterov, lr_dropout, seeds, wps=None, cs=None,
+                             kks=None, layouts=None):
+        from oracle import hash_rng
+        self.launches += 1
+        mom, lr32 = np.float32(momentum), np.float32(lr)
+        for i, (n, v, g, acc) in enumerate(zip(ns, vs, gs, accs)):
+            V, G, A = self.f(v)[:n], self.f(g)[:n], self.f(acc)[:n]
+            lr_a = np.where(hash_rng.lr_dropout_mask(n, seeds[2 * i], lr_dropout), np.float32(0), lr32) if lr_dropout else lr32
+            lr_t = np.where(hash_rng.lr_dropout_mask(n, seeds[2 * i + 1], lr_dropout), np.float32(0), lr32) if lr_dropout else lr32
+            a = (mom * A - lr_a * G).astype(np.float32)
+            A[:] = a
+            V[:] = V + ((mom * a - lr_t * G) if nesterov else a)
+        if wps is not None:
+            self._refresh_copies(ns, vs, wps, cs, kks, layouts)
+
+    def adam_update_multi_lrd(self, dev, ns, ts, gs, ms, vs, beta1, beta2, lr, lr_dropout, seeds, wps=None, cs=None,
+                              kks=None, layouts=None):
+        from oracle import hash_rng
+        self.launches += 1
+        b1, b2, lr32 = np.float32(beta1), np.float32(beta2), np.float32(lr)
+        for i, (n, t, g, m, v) in enumerate(zip(ns, ts, gs, ms, vs)):
+            T, G, M, V = self.f(t)[:n], self.f(g)[:n], self.f(m)[:n], self.f(v)[:n]
+            lr_t = np.where(hash_rng.lr_dropout_mask(n, seeds[i], lr_dropout), np.float32(0), lr32) if lr_dropout else lr32
+            M[:] = b1 * M + (np.float32(1) - b1) * G
+            V[:] = b2 * V + (np.float32(1) - b2) * G * G
+            T[:] = T - lr_t * M / (np.sqrt(V) + np.float32(1e-7))
+        if wps is not None:
+            self._refresh_copies(ns, ts, wps, cs, kks, layouts)
 
     def bias_act_bwd(self, dev, N, O, HW, y, dy, act, slope, dpre, dbias, beta_bias):
         self.launches += 1

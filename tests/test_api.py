@@ -589,8 +589,58 @@ def test_sgd_closed_form(nn_backend):
             w = w + (momentum * acc - lr * g if nesterov else acc)
         np.testing.assert_allclose(w_t.np(), w, rtol=1e-5, atol=1e-6)
         w_t._set_trainable(False)
-    with pytest.raises(NotImplementedError):
-        nn.optimizer.SGD([nn.Tensor((4,))], lr_dropout=0.7)
+    with pytest.raises(ValueError):
+        nn.optimizer.SGD([nn.Tensor((4,))], lr_dropout=1.7)
+
+
+def test_lr_dropout_follows_the_counter_hash(nn_backend):
+    """Optimizer.py:178-203: every update kernel draws a seed from numpy's global generator and zeroes the learning
+    rate of element gid where hash_float_uint(gid + seed) <= lr_dropout.  With the generator seeded, the dropped
+    elements are those the oracle's hash names, for SGD (two kernels per tensor, SGD.py:42-83) and Adam (one,
+    Adam.py:61-86)."""
+    nn = nn_backend
+    n, p = 5000, 0.3
+    rs = np.random.RandomState(2)
+    w0 = rs.randint(-8, 9, size=n).astype(np.float32)
+    g = rs.randint(1, 9, size=n).astype(np.float32)
+    for nesterov in (False, True):
+        w_t = nn.Tensor_from_value(w0)
+        opt = nn.optimizer.SGD([w_t], momentum=0.5, nesterov=nesterov, lr=0.25, lr_dropout=p)
+        np.random.seed(77)
+        seeds = [int(np.random.randint(2147483648)) for _ in range(4)]
+        np.random.seed(77)
+        w, acc = w0.astype(np.float64), np.zeros(n)
+        for it in range(2):
+            w_t.get_grad().set(g)
+            opt.step()
+            lr_a = np.where(hash_rng.lr_dropout_mask(n, seeds[2 * it], p), 0.0, 0.25)
+            lr_t = np.where(hash_rng.lr_dropout_mask(n, seeds[2 * it + 1], p), 0.0, 0.25)
+            acc = 0.5 * acc - lr_a * g
+            w = w + (0.5 * acc - lr_t * g if nesterov else acc)
+        assert np.array_equal(w_t.np(), w)          # small integers and quarters: exact in fp32
+        assert 0.2 < hash_rng.lr_dropout_mask(n, seeds[0], p).mean() < 0.4
+        w_t._set_trainable(False)
+    w_t = nn.Tensor_from_value(w0)
+    opt = nn.optimizer.Adam([w_t], lr=0.5, lr_dropout=p)
+    np.random.seed(78)
+    seed = int(np.random.randint(2147483648))
+    np.random.seed(78)
+    w_t.get_grad().set(g)
+    opt.step()
+    dropped = hash_rng.lr_dropout_mask(n, seed, p)
+    got = w_t.np()
+    assert np.array_equal(got[dropped], w0[dropped]) and np.all(got[~dropped] != w0[~dropped])
+    w_t._set_trainable(False)
+    # the seeds are drawn whether or not dropout is on, as the reference does: the generator stays in step with it
+    w_t = nn.Tensor_from_value(w0)
+    opt = nn.optimizer.SGD([w_t], lr=0.25)
+    np.random.seed(79)
+    expect = np.random.RandomState(79)
+    w_t.get_grad().set(g)
+    opt.step()
+    expect.randint(2147483648), expect.randint(2147483648)
+    assert np.random.randint(1 << 30) == expect.randint(1 << 30)
+    w_t._set_trainable(False)
 
 
 def test_adam_closed_form(nn_backend):

@@ -131,3 +131,45 @@ def test_bias_act_bwd_rows_layout(hip):
             pre = dy * np.where(y >= 0, 1.0, 0.5).astype(np.float32)
             assert np.array_equal(dP.get(), pre)
             assert np.array_equal(dB.get(), pre.sum(0) + (db0 if beta else 0))
+
+
+def test_lr_dropout_updates_match_the_hash_oracle(hip):
+    """lnn_*_update_multi_lrd_f32 against the oracle's counter hash, bit for bit: two tensors per launch, every seed
+    position, with and without nesterov (Optimizer.py:186-203, SGD.py:42-74, Adam.py:61-72)."""
+    from oracle import hash_rng
+    rs = np.random.RandomState(9)
+    ns = [70001, 333]
+    p, lr, mom = 0.4, 0.5, 0.5
+    w0 = [rs.randint(-8, 9, size=n).astype(np.float32) for n in ns]
+    g = [rs.randint(1, 9, size=n).astype(np.float32) for n in ns]
+    a0 = [rs.randint(-4, 5, size=n).astype(np.float32) for n in ns]
+    seeds = [12345, 2147483647, 4294967295 - 100, 7]     # the third wraps the 32-bit counter inside the tensor
+    for nesterov in (0, 1):
+        say(f'sgd_update_multi_lrd nesterov={nesterov}')
+        W, G, A = [DevArr(hip, x) for x in w0], [DevArr(hip, x) for x in g], [DevArr(hip, x) for x in a0]
+        hip.sgd_update_multi_lrd(0, ns, [x.ptr for x in W], [x.ptr for x in G], [x.ptr for x in A], mom, lr, nesterov, p, seeds)
+        for i, n in enumerate(ns):
+            lr_a = np.where(hash_rng.lr_dropout_mask(n, seeds[2 * i], p), 0.0, lr)
+            lr_t = np.where(hash_rng.lr_dropout_mask(n, seeds[2 * i + 1], p), 0.0, lr)
+            acc = mom * a0[i].astype(np.float64) - lr_a * g[i]
+            w = w0[i] + (mom * acc - lr_t * g[i] if nesterov else acc)
+            assert np.array_equal(A[i].get(), acc) and np.array_equal(W[i].get(), w)
+    say('adam_update_multi_lrd')
+    W, G = [DevArr(hip, x) for x in w0], [DevArr(hip, x) for x in g]
+    M, V = [DevArr(hip, np.zeros(n, np.float32)) for n in ns], [DevArr(hip, np.zeros(n, np.float32)) for n in ns]
+    hip.adam_update_multi_lrd(0, ns, [x.ptr for x in W], [x.ptr for x in G], [x.ptr for x in M], [x.ptr for x in V],
+                              0.9, 0.999, lr, p, seeds[:2])
+    for i, n in enumerate(ns):
+        dropped = hash_rng.lr_dropout_mask(n, seeds[i], p)
+        got = W[i].get()
+        assert np.array_equal(got[dropped], w0[i][dropped]) and np.all(got[~dropped] != w0[i][~dropped])
+        assert 0.3 < dropped.mean() < 0.5
+    # lr_dropout == 0 is the plain update and needs no seeds
+    W, G, A = [DevArr(hip, x) for x in w0], [DevArr(hip, x) for x in g], [DevArr(hip, x) for x in a0]
+    W2, G2, A2 = [DevArr(hip, x) for x in w0], [DevArr(hip, x) for x in g], [DevArr(hip, x) for x in a0]
+    hip.sgd_update_multi_lrd(0, ns, [x.ptr for x in W], [x.ptr for x in G], [x.ptr for x in A], mom, lr, 1, 0.0, seeds)
+    hip.sgd_update_multi(0, ns, [x.ptr for x in W2], [x.ptr for x in G2], [x.ptr for x in A2], mom, lr, 1)
+    for i in range(2):
+        assert np.array_equal(W[i].get(), W2[i].get())
+    with pytest.raises(hip.HipException):
+        hip.sgd_update_multi_lrd(0, ns, [x.ptr for x in W], [x.ptr for x in G], [x.ptr for x in A], mom, lr, 1, 1.5, seeds)

@@ -133,3 +133,16 @@ def test_fma32_rounds_once():
     for x, y, z, g in zip(a.tolist(), b.tolist(), c.tolist(), got.tolist()):
         assert np.float32(g) == nearest_f32(Fraction(x) * Fraction(y) + Fraction(z)), (x, y, z)
     assert got[-4] != got[-3]      # the 2^-60 addends break the tie in opposite directions
+
+
+def test_lr_dropout_mask_is_the_uniform_stream_against_a_threshold():
+    """Optimizer.py:199-202 compares hash_float_uint(gid + seed) with lr_dropout: the mask is the uniform initialiser's
+    unit stream (low 0, high 1) cut at the threshold, with the expected share of elements dropped; the counter wraps
+    modulo 2**32 like the initialisers'."""
+    n = 200000
+    for seed, p in ((3, 0.25), (2147483647, 0.5), (4294967295 - 50, 0.9)):
+        mask = hash_rng.lr_dropout_mask(n, seed, p)
+        assert np.array_equal(mask, hash_rng.random_uniform(n, seed, 0.0, 1.0) <= np.float32(p))
+        assert abs(mask.mean() - p) < 0.01
+    assert not hash_rng.lr_dropout_mask(1000, 1, 0.0).any() or hash_rng.random_uniform(1000, 1).min() == 0.0
+    assert hash_rng.lr_dropout_mask(1000, 1, 1.0).all()
