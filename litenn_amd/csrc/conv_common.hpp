@@ -15,44 +15,6 @@
 #include "common.hpp"
 #include "slice_reduce.hpp"
 
-// Forward / dgrad: remainder units cut along K (see plan_tiles).
-#ifndef LNN_TAIL_SPLIT
-#define LNN_TAIL_SPLIT 1
-#endif
-#ifndef LNN_WGRAD_UNROLL
-#define LNN_WGRAD_UNROLL 0
-#endif
-#ifndef LNN_KSPLIT_HALF
-#define LNN_KSPLIT_HALF 1
-#endif
-#ifndef LNN_DGRAD_PAIRS
-#define LNN_DGRAD_PAIRS 1
-#endif
-#ifndef LNN_STAGES_WGRAD
-#define LNN_STAGES_WGRAD 3
-#endif
-#ifndef LNN_STAGES_FD
-#define LNN_STAGES_FD 3
-#endif
-// B-side gathers: 1 = straight into LDS, 0 = through registers (needs three stages)
-#ifndef LNN_FD_B_DIRECT
-#define LNN_FD_B_DIRECT 1
-#endif
-#ifndef LNN_CLASS_SHARES
-#define LNN_CLASS_SHARES 1
-#endif
-#ifndef LNN_SMALL_DGRAD
-#define LNN_SMALL_DGRAD 1
-#endif
-#ifndef LNN_FWD_ANYC
-#define LNN_FWD_ANYC 1
-#endif
-#ifndef LNN_WGRAD_ANYC
-#define LNN_WGRAD_ANYC 1
-#endif
-#ifndef LNN_WGRAD_B_DIRECT
-#define LNN_WGRAD_B_DIRECT 1
-#endif
 
 namespace lnn {
 namespace {
@@ -133,10 +95,10 @@ __global__ void build_ktable(KEntry* tab, int K, int Kpad, int mode, ConvGeom g,
 
 // *_TAP: tap-major K order over channel-permuted weights (channels % BK == 0)
 // PASS_WGRAD_TAP4: PASS_WGRAD_TAP with 128-bit transfers of the pixel gather too (stride 1, OW % 4 == 0, no padded columns)
-// PASS_FWD_ANYC: PASS_FWD (any channel count, gather table) with both operands straight into LDS, three stages
+// PASS_FWD_ANYC: forward for any channel count (gather table), both operands straight into LDS, three stages
 // PASS_WGRAD_ANYC: wgrad for any channel count with transfers straight into LDS; a group's columns may span taps
 // PASS_DGRAD_TAPW: tap-major dgrad that reads the weights in the forward pass's permuted layout (C % 4 == 0)
-enum { PASS_FWD = 0, PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5, PASS_WGRAD_TAP4 = 6,
+enum { PASS_DGRAD = 1, PASS_WGRAD = 2, PASS_FWD_TAP = 3, PASS_DGRAD_TAP = 4, PASS_WGRAD_TAP = 5, PASS_WGRAD_TAP4 = 6,
        PASS_DGRAD_TAPW = 7, PASS_WGRAD_ANYC = 8, PASS_FWD_ANYC = 9 };
 // the weight-gradient passes whose GEMM columns are tap-major (column tap*C + c)
 constexpr bool wgrad_tap(int pass) { return pass == PASS_WGRAD_TAP || pass == PASS_WGRAD_TAP4 || pass == PASS_WGRAD_ANYC; }
@@ -204,11 +166,10 @@ struct ConvCfg {
   static constexpr int SA = DIRECT ? BM * BK : LdsSize<true, BM>::value;
   // B side: pixel-contiguous gathers (fwd, dgrad) or K-contiguous (wgrad).
   static constexpr int SB = DIRECT ? BNMAX * BK : LdsSize<PASS == PASS_WGRAD, BNMAX>::value;
-  static constexpr int STAGES = !DIRECT ? 2 : (wgrad_tap(PASS) ? LNN_STAGES_WGRAD : (PASS == PASS_FWD_ANYC ? 3 : LNN_STAGES_FD));
+  static constexpr int STAGES = DIRECT ? 3 : 2;
 };
 
 // Loader selection and initialisation per pass.  FLAG:
-//   PASS_FWD        128-bit loads of W rows (CKK % 4 == 0)
 //   PASS_WGRAD(_TAP) 128-bit loads of dY (OHW % 4 == 0)
 template <int PASS, bool FLAG, int ST>
 struct ConvProblem;
@@ -222,14 +183,6 @@ struct ConvProblemBase {
   PostOp post;
 };
 
-template <bool FLAG, int ST>
-struct ConvProblem<PASS_FWD, FLAG, ST> : ConvProblemBase {
-  static constexpr int STAGES = ST;
-  template <int R> using LA = PlainKC<R, FLAG>;
-  template <int R> using LB = ConvFwdB<R>;
-  template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
-  template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
-};
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_FWD_ANYC, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
@@ -245,7 +198,7 @@ template <bool FLAG, int ST>
 struct ConvProblem<PASS_FWD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = ConvFwdATap<R>;            // permuted weights [O][KK*C]
-  template <int R> using LB = ConvFwdBTap<R, LNN_FD_B_DIRECT != 0>;
+  template <int R> using LB = ConvFwdBTap<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, M, kbeg); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, col0, Ncols, kbeg); }
 };
@@ -261,7 +214,7 @@ template <bool FLAG, int ST>
 struct ConvProblem<PASS_DGRAD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = DirectKC<R>;               // permuted weights [C][taps*O]
-  template <int R> using LB = ConvDgradBTap<R, LNN_FD_B_DIRECT != 0>;
+  template <int R> using LB = ConvDgradBTap<R, false>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, K, row0, M, K); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg); }
 };
@@ -269,7 +222,7 @@ template <bool FLAG, int ST>
 struct ConvProblem<PASS_DGRAD_TAPW, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
   template <int R> using LA = ConvDgradATapMC<R>;        // the forward pass's permuted weights [O][KK*C]
-  template <int R> using LB = ConvDgradBTap<R, LNN_FD_B_DIRECT != 0, LNN_CB_MAJOR != 0>;
+  template <int R> using LB = ConvDgradBTap<R, true>;
   // K = O * (taps of the pixel class)
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, tab, row0, kbeg, K / g.O); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A&) const { l.init(rx, g, tab, col0, Ncols, kbeg, K / g.O); }
@@ -286,10 +239,10 @@ struct ConvProblem<PASS_WGRAD, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  static constexpr bool STREAM_UNROLL = LNN_WGRAD_UNROLL != 0;   // measured: slower with constant stages (config 3: 0.235 -> 0.247 ms)
+  static constexpr bool STREAM_UNROLL = false;   // measured: slower with constant stages (config 3: 0.235 -> 0.247 ms)
   static constexpr bool STREAM_REGIONS = true;
   template <int R> using LA = typename std::conditional<FLAG, ConvWgradTapA4Direct<R>, ConvWgradTapADirect<R>>::type;
-  template <int R> using LB = ConvWgradTapBDirect<R, LNN_WGRAD_B_DIRECT != 0>;
+  template <int R> using LB = ConvWgradTapBDirect<R>;
   template <int R> __device__ __forceinline__ void init_a(LA<R>& l, int row0) const { l.init(rw, g, row0, kend, kbeg); }
   template <int R, class A> __device__ __forceinline__ void init_b(LB<R>& l, int col0, A& la) const { l.init(rx, g, col0, la, kend, kbeg); }
 };
@@ -297,7 +250,7 @@ struct ConvProblem<PASS_WGRAD_TAP, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_ANYC, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  static constexpr bool STREAM_UNROLL = LNN_WGRAD_UNROLL != 0;   // measured: slower with constant stages (config 3: 0.235 -> 0.247 ms)
+  static constexpr bool STREAM_UNROLL = false;   // measured: slower with constant stages (config 3: 0.235 -> 0.247 ms)
   static constexpr bool STREAM_REGIONS = true;
   template <int R> using LA = typename std::conditional<FLAG, ConvWgradTapA4Direct<R>, ConvWgradTapADirect<R>>::type;
   template <int R> using LB = ConvWgradBAnyC<R>;
@@ -308,7 +261,7 @@ struct ConvProblem<PASS_WGRAD_ANYC, FLAG, ST> : ConvProblemBase {
 template <bool FLAG, int ST>
 struct ConvProblem<PASS_WGRAD_TAP4, FLAG, ST> : ConvProblemBase {
   static constexpr int STAGES = ST;
-  static constexpr bool STREAM_UNROLL = LNN_WGRAD_UNROLL != 0;   // measured: slower with constant stages (config 3: 0.235 -> 0.247 ms)
+  static constexpr bool STREAM_UNROLL = false;   // measured: slower with constant stages (config 3: 0.235 -> 0.247 ms)
   static constexpr bool STREAM_REGIONS = true;
   template <int R> using LA = ConvWgradTapA4Direct<R>;
   template <int R> using LB = ConvWgradTapB4Direct<R>;
@@ -326,7 +279,7 @@ __host__ __device__ inline OutMap plain_map(int ncols) {
 template <int PASS>
 __host__ __device__ inline OutMap final_map(const ConvArgs& a) {
   OutMap om = plain_map(a.Ncols);
-  if (PASS == PASS_FWD || PASS == PASS_FWD_TAP || PASS == PASS_FWD_ANYC) {
+  if (PASS == PASS_FWD_TAP || PASS == PASS_FWD_ANYC) {
     om.nchw = 1; om.ld = a.g.OHW; om.mtot = a.g.O; om.dHW = a.g.dOHW;
   } else if (PASS == PASS_DGRAD || dgrad_tap(PASS)) {
     om.nchw = 3; om.ld = a.full_IHW; om.mtot = a.g.C; om.dHW = a.g.dIHW;
@@ -617,7 +570,7 @@ static size_t plan_tiles(ConvArgs& a, long long slots, bool allow_tail = false) 
   // Few output tiles (small images, deep layers): a workgroup's share would be a sliver of a sub-tile and
   // most of its time data movement.  Cut the output into full sub-tiles instead and split K over the
   // workgroups that are left, as wgrad does.
-  const int chunk = (2 * NTMAX) >> LNN_KSPLIT_HALF > 1 ? (2 * NTMAX) >> LNN_KSPLIT_HALF : 2;
+  const int chunk = NTMAX > 1 ? NTMAX : 2;
   const long long chunks = (total + chunk - 1) / chunk;
   const int nkt = (a.K + BK - 1) / BK;
   if (total < slots * (NTMAX + 1) && chunks * 2 <= slots && nkt >= 16) {
@@ -631,7 +584,7 @@ static size_t plan_tiles(ConvArgs& a, long long slots, bool allow_tail = false) 
   }
   // A few units per workgroup and a remainder: the workgroups that would take one unit more set the pace
   // (3136 units on 256 workgroups: 13 against 12.25).  Cut the remainder along K instead, one slice per workgroup.
-  if (allow_tail && LNN_TAIL_SPLIT && total > slots && total <= 64 * slots) {
+  if (allow_tail && total > slots && total <= 64 * slots) {
     const long long q = total / slots, r = total - q * slots;
     long long ts = r > 0 ? slots / r : 0;
     if (ts > nkt / 6) ts = nkt / 6;   // a slice should still hold a handful of K steps
@@ -729,7 +682,7 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     }
   }
   dim3 g(a.grid_x, grid_y, 1), b(512, 1, 1);
-  constexpr bool kUsesFlag = PASS == PASS_FWD || PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP || PASS == PASS_WGRAD_ANYC;   // the other passes have one variant
+  constexpr bool kUsesFlag = PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP || PASS == PASS_WGRAD_ANYC;   // the other passes have one variant
   if (flag || !kUsesFlag) {
     hipLaunchKernelGGL((conv_kernel<PASS, WM, NTMAX, true>), g, b, 0, ctx->stream, a);
   } else if constexpr (kUsesFlag) {
@@ -765,7 +718,7 @@ static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_
   // kernels, whose time follows the multiply-adds, each gets workgroups in proportion to its work instead
   // (256 -> 512 channels at 16 x 16: 77 -> 63 us).
   std::vector<long long> share(n, equal);
-  if (LNN_CLASS_SHARES && dgrad_tap(PASS) && n <= kMaxBatch) {
+  if (dgrad_tap(PASS) && n <= kMaxBatch) {
     // Only where every class is cut along K anyway (few output tiles: any share divides into whole sub-tiles times
     // K slices).  Classes with many tiles and no K split lose more to the narrow sub-tiles of an odd share than
     // they gain (64 -> 128 channels at 64 x 64: 82 -> 121 us).
@@ -864,7 +817,7 @@ template <int PASS>
 static int launch_classes_by_m(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_off) {
   const int M = cls[0].M;
   if (M > 64) return launch_classes<PASS, 4, 4>(ctx, cls, ws_off);
-  if (LNN_DGRAD_PAIRS && PASS == PASS_DGRAD_TAPW && M > 32 && cls.size() == 4) {
+  if (PASS == PASS_DGRAD_TAPW && M > 32 && cls.size() == 4) {
     // Four classes with many tiles each and different K lengths (5x5 stride 2: 9, 6, 6 and 4 taps): on 64 x 128
     // tiles two workgroups share a compute unit, and with the classes in the order longest, second, shortest, third
     // workgroups b and b + (number of compute units) - which land on the same one - are a long and a short piece.

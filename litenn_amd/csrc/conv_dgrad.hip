@@ -1,9 +1,6 @@
 // Convolution data gradient: pixel classes on the MFMA engine, and the vector-ALU kernel for very few input channels.
 #include "conv_common.hpp"
 
-#ifndef LNN_STEM_DGRAD
-#define LNN_STEM_DGRAD 1
-#endif
 
 namespace lnn {
 namespace {
@@ -226,7 +223,7 @@ __global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
 // The vector-ALU data gradient serves C <= 4, dilation 1, stride 1 (K = 1, 3, 5) or 2 (K = 3, 4, 5, 7), when there
 // are enough tiles to occupy the chip (a small problem is quicker on the MFMA path, whose tiles are finer).
 static bool small_dgrad_applies(int cus, const ConvGeom& g) {
-  if (!LNN_SMALL_DGRAD || g.C > 4 || g.D != 1 || g.KH != g.KW) return false;
+  if (g.C > 4 || g.D != 1 || g.KH != g.KW) return false;
   const int K = g.KH;
   const bool shape = (g.S == 1 && (K == 1 || K == 3 || K == 5)) || (g.S == 2 && (K == 3 || K == 4 || K == 5 || K == 7));
   if (!shape) return false;
@@ -312,7 +309,7 @@ int conv_dgrad_path(const lnn_conv2d_desc* d, int beta, int compute_units, int* 
   *path = g.O % BK == 0 ? LNN_DGRAD_PATH_MFMA_TAP : LNN_DGRAD_PATH_MFMA_TABLE;
   if (tile_info)
     for (int i = 0; i < 7; ++i) tile_info[i] = 0;
-  if (LNN_STEM_DGRAD && stem_dgrad_applies(d, compute_units)) {
+  if (stem_dgrad_applies(d, compute_units)) {
     *path = LNN_DGRAD_PATH_STEM_MFMA;
     return LNN_OK;
   }
@@ -354,7 +351,7 @@ int launch_conv_dgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* dY,
   if (!dY || (!W && !Wp) || !dX) return set_error(LNN_ERR_INVALID, "conv2d_dgrad: null pointer");
   const int S = full.S;
   if (S > 15) return set_error(LNN_ERR_UNSUPPORTED, "conv2d_dgrad: stride > 15");
-  if (LNN_STEM_DGRAD && !Wp && stem_dgrad_applies(d, ctx->cus)) return launch_stem_dgrad(ctx, d, dY, W, dX, beta);
+  if (!Wp && stem_dgrad_applies(d, ctx->cus)) return launch_stem_dgrad(ctx, d, dY, W, dX, beta);
   if (!tapw && small_dgrad_applies(ctx->cus, full)) {
     st = launch_small_dgrad(ctx, full, dY, W, dX, beta);
     if (st != kNotHere) return st;

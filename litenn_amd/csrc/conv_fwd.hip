@@ -1,9 +1,6 @@
 // Convolution forward pass (and its fused bias / activation epilogue).
 #include "conv_common.hpp"
 
-#ifndef LNN_STEM_FWD
-#define LNN_STEM_FWD 1
-#endif
 
 namespace lnn {
 
@@ -26,7 +23,7 @@ int conv_fwd_path(const lnn_conv2d_desc* d, int compute_units, int* path) {
   int st = fill_geom(d, g);
   if (st != LNN_OK) return st;
   if (!path || compute_units <= 0) return set_error(LNN_ERR_INVALID, "conv2d_fwd_path: null result pointer or no compute units");
-  *path = LNN_STEM_FWD && stem_fwd_applies(d, compute_units) ? LNN_FWD_PATH_STEM_PATCH : LNN_FWD_PATH_IMPLICIT_GEMM;
+  *path = stem_fwd_applies(d, compute_units) ? LNN_FWD_PATH_STEM_PATCH : LNN_FWD_PATH_IMPLICIT_GEMM;
   return LNN_OK;
 }
 
@@ -53,7 +50,7 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   if (Wp && a.g.C % BK != 0) return set_error(LNN_ERR_INVALID, "conv2d_fwd: this geometry does not read permuted weights");
   if (Wp && !aligned16(Wp)) return set_error(LNN_ERR_INVALID, "conv2d_fwd: permuted weights must be 16-byte aligned");
   if (!X || (!W && !Wp) || !Y) return set_error(LNN_ERR_INVALID, "conv2d_fwd: null pointer");
-  if (LNN_STEM_FWD && !Wp && stem_fwd_applies(d, ctx->cus)) return launch_stem_fwd(ctx, d, X, W, Y, beta, bias, act, slope);
+  if (!Wp && stem_fwd_applies(d, ctx->cus)) return launch_stem_fwd(ctx, d, X, W, Y, beta, bias, act, slope);
   st = reserve_tables(ctx, 1);
   if (st != LNN_OK) return st;
   a.tab = nullptr;
@@ -77,8 +74,7 @@ int launch_conv_fwd(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, co
   }
   st = get_table(ctx, a.g, 0, PixelClass{}, &a.tab);
   if (st != LNN_OK) return st;
-  if (LNN_FWD_ANYC) return launch_by_m<PASS_FWD_ANYC>(ctx, a, true);
-  return launch_by_m<PASS_FWD>(ctx, a, a.K % 4 == 0 && aligned16(W));
+  return launch_by_m<PASS_FWD_ANYC>(ctx, a, true);
 }
 
 }  // namespace lnn

@@ -12,9 +12,7 @@
 
 #include "common.hpp"
 
-#ifndef LNN_STEM_MIN_TILES
-#define LNN_STEM_MIN_TILES 4   // tiles of 256 pixels per compute unit from which the patch kernels are used
-#endif
+constexpr int kStemMinTiles = 4;   // tiles of 256 pixels per compute unit from which the patch kernels are used
 
 namespace lnn {
 namespace {
@@ -616,7 +614,7 @@ bool stem_fwd_applies(const lnn_conv2d_desc* d, int compute_units) {
   if (d->C != 3 || d->O <= 32 || d->O > 64 || d->dilation != 1 || d->KH != d->KW) return false;
   const int k = d->KH, s = d->stride;
   if (!((k == 7 && s == 2) || (k == 5 && s == 2) || (k == 3 && (s == 1 || s == 2)))) return false;
-  return (long long)d->N * (((long long)d->OH * d->OW + 255) / 256) >= (long long)LNN_STEM_MIN_TILES * compute_units;
+  return (long long)d->N * (((long long)d->OH * d->OW + 255) / 256) >= (long long)kStemMinTiles * compute_units;
 }
 
 // Y (+)= conv(X, W) with the bias / activation epilogue, for the geometries stem_fwd_applies() accepts

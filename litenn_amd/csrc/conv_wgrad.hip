@@ -1,9 +1,6 @@
 // Convolution weight gradient (split over the output pixels, deterministic slice reduction).
 #include "conv_common.hpp"
 
-#ifndef LNN_STEM_WGRAD
-#define LNN_STEM_WGRAD 1
-#endif
 
 namespace lnn {
 
@@ -16,7 +13,7 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");
-  if (LNN_STEM_WGRAD && !w_iohw && stem_wgrad_applies(d, ctx->cus, dY)) return launch_stem_wgrad(ctx, d, X, dY, dW, beta);
+  if (!w_iohw && stem_wgrad_applies(d, ctx->cus, dY)) return launch_stem_wgrad(ctx, d, X, dY, dW, beta);
   a.tab = nullptr;
   const ConvGeom& g = a.g;
   a.X = X; a.W = dY; a.Out = dW;
@@ -35,7 +32,7 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
     return launch_by_m<PASS_WGRAD_TAP>(ctx, a, vec);
   }
   // any other channel count: a group's columns may span taps
-  if (LNN_WGRAD_ANYC && wgrad_walkers_fit(g)) return launch_by_m<PASS_WGRAD_ANYC>(ctx, a, vec);
+  if (wgrad_walkers_fit(g)) return launch_by_m<PASS_WGRAD_ANYC>(ctx, a, vec);
   if (w_iohw) return set_error(LNN_ERR_UNSUPPORTED, "conv2d_wgrad: this geometry cannot write a gradient with swapped channel axes");
   // tiny images: the table-driven kernel with per-column gather entries
   st = reserve_tables(ctx, 1);

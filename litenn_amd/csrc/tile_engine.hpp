@@ -32,25 +32,6 @@
 
 namespace lnn {
 
-#ifndef LNN_CB_MAJOR
-#define LNN_CB_MAJOR 1
-#endif
-// Three-stage pipelines of two direct loaders run without phases: one barrier per K step, inside the MFMA stream.
-#ifndef LNN_STREAM
-#define LNN_STREAM 1
-#endif
-#ifndef LNN_GROUP_REGIONS
-#define LNN_GROUP_REGIONS 1
-#endif
-#ifndef LNN_VALU_FIRST
-#define LNN_VALU_FIRST 64
-#endif
-#ifndef LNN_STREAM_UNROLL
-#define LNN_STREAM_UNROLL 1
-#endif
-#ifndef LNN_REQUEST_FIRST
-#define LNN_REQUEST_FIRST 0
-#endif
 constexpr int BK = 32;            // K extent of one LDS stage
 constexpr int KG = BK / 4;        // float4 groups along K
 constexpr int KR = BK / 4;        // K rows fetched per wavefront of a group in the pixel-major gathers
@@ -362,67 +343,6 @@ __device__ __forceinline__ ktab_t as_ktab(const KEntry* p) {
   return reinterpret_cast<ktab_t>(reinterpret_cast<uintptr_t>(p));
 }
 
-// Forward im2col gather: element (pixel p, k) = X[n, c, oh*S-PT+kh*D, ow*S-PL+kw*D].
-// Each wavefront fetches 4 of the 16 k rows; lanes run over pixels so that
-// global reads follow the image rows and k stays wave-uniform.
-template <int R>
-struct ConvFwdB {
-  static constexpr bool KC = false;
-  static constexpr int CC = (R + 63) / 64;
-  rsrc_t rs;
-  ktab_t tab;
-  int IH, IW;
-  int base[CC], ih0[CC], iw0[CC];
-  int tx[KR], ty[KR], tz[KR];   // table entries of the next fetch (scalar registers)
-  float v[KR][CC];
-  __device__ __forceinline__ void load_entries(int k0) {
-    const int wave = __builtin_amdgcn_readfirstlane(gwave());
-#pragma unroll
-    for (int e = 0; e < KR; ++e) {
-      const ktab_t t = tab + (k0 + wave + 4 * e);
-      tx[e] = t->x; ty[e] = t->y; tz[e] = t->z;
-    }
-  }
-  __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P, int kbeg) {
-    rs = r;
-    tab = as_ktab(tab_);
-    load_entries(kbeg);
-    IH = g.IH;
-    IW = g.IW;
-    const int lane = threadIdx.x & 63;
-#pragma unroll
-    for (int c = 0; c < CC; ++c) {
-      const int col = lane + 64 * c, p = p0 + col;
-      const bool ok = col < R && p < P;
-      const uint32_t pp = ok ? (uint32_t)p : 0u;
-      const uint32_t img = g.dOHW.div(pp), rem = pp - img * g.OHW;
-      const uint32_t oh = g.dOW.div(rem), ow = rem - oh * g.OW;
-      ih0[c] = (int)oh * g.S - g.PADT;
-      iw0[c] = ok ? (int)ow * g.S - g.PADL : -BIG;
-      base[c] = ((int)img * g.C * g.IH + ih0[c]) * g.IW + ((int)ow * g.S - g.PADL);
-    }
-  }
-  __device__ __forceinline__ void fetch(int k0) {
-#pragma unroll
-    for (int e = 0; e < KR; ++e) {
-#pragma unroll
-      for (int c = 0; c < CC; ++c) {
-        const bool ok = (uint32_t)(ih0[c] + ty[e]) < (uint32_t)IH && (uint32_t)(iw0[c] + tz[e]) < (uint32_t)IW;
-        v[e][c] = buf_load(rs, ok ? (uint32_t)(base[c] + tx[e]) * 4u : OOB);
-      }
-    }
-    load_entries(k0 + BK);
-  }
-  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
-    const int wave = gwave(), lane = threadIdx.x & 63;
-#pragma unroll
-    for (int e = 0; e < KR; ++e)
-#pragma unroll
-      for (int c = 0; c < CC; ++c)
-        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
-  }
-};
-
 // The forward pass's weight operand Wp[o][tap][c], rows of K = KK*C floats, read in the K order of ConvFwdBTap
 // (see there): K step (channel block, tap) sits at row offset tap*C + block*BK.
 template <int R>
@@ -431,26 +351,16 @@ struct ConvFwdATap : DirectKC<R> {
   __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int row0, int M, int kbeg) {
     DirectKC<R>::init(r, g.C * g.KK, row0, M, 0);
     C = g.C; KK = g.KK;
-#if LNN_CB_MAJOR
     const int t0 = kbeg / BK, cb = t0 / g.KK;
     tap = t0 - cb * g.KK;
     c0 = cb * BK;
-#else
-    tap = kbeg / g.C;
-    c0 = kbeg - tap * g.C;
-#endif
   }
   __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
   template <int PART, int NPARTS>
   __device__ __forceinline__ int issue_part(int, float* lds, int ld, int off) {
     const int n = DirectKC<R>::template issue_part<PART, NPARTS>(tap * C + c0, lds, ld, off);
     if (PART == NPARTS - 1) {
-#if LNN_CB_MAJOR
       if (++tap == KK) { tap = 0; c0 += BK; }
-#else
-      c0 += BK;
-      if (c0 >= C) { c0 = 0; ++tap; }
-#endif
     }
     return n;
   }
@@ -559,23 +469,22 @@ struct ConvFwdBDirect {
 // step is BK consecutive channels of a single tap: the pixel part of the
 // address and its range test depend on the tap only and live in a VGPR, the
 // channel part is wave-uniform and rides in the scalar offset of the buffer
-// instruction.  No table, no per-element arithmetic.  fetch() must be called
+// instruction.  No table, no per-element arithmetic.  issue() must be called
 // with consecutive K steps starting at the kbeg given to init().
-// K order: with LNN_CB_MAJOR the channel block is the outer loop and the taps the inner one (k-step t = block * KK +
+// K order: the channel block is the outer loop and the taps the inner one (k-step t = block * KK +
 // tap), so that the KK consecutive steps of one block of BK channels re-read the same pixels, shifted, while they
 // are still in the L2 of the XCD; tap-major order (all channels of a tap, then the next tap) revisits a pixel only
 // after the whole channel range, by when a 4 MB L2 shared by 32 workgroups has dropped it.
-template <int R, bool DIR = false>
+template <int R>
 struct ConvFwdBTap {
-  static constexpr bool KC = false, DIRECT = DIR;
+  static constexpr bool KC = false, DIRECT = true;
   static constexpr int CC = (R + 63) / 64;
   static constexpr int NLD = KR * CC;
   rsrc_t rs;
   int IH, IW, IHW, C, D, KW, KH;
   int base[CC], ih0[CC], iw0[CC];
   uint32_t voff[CC];   // per-pixel byte offset for the current tap, or OOB
-  int c0, kh, kw;   // K position of the next fetch
-  float v[KR][CC];
+  int c0, kh, kw;   // K position of the next transfer
   __device__ __forceinline__ void set_tap() {
     const int dh = kh * D, dw = kw * D, tapoff = dh * IW + dw;
 #pragma unroll
@@ -587,13 +496,8 @@ struct ConvFwdBTap {
   __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, int p0, int P, int kbeg) {
     rs = r;
     IH = g.IH; IW = g.IW; IHW = g.IHW; C = g.C; D = g.D; KW = g.KW; KH = g.KH;
-#if LNN_CB_MAJOR
     const int t0 = kbeg / BK, cb = t0 / g.KK, tap = t0 - cb * g.KK;
     c0 = cb * BK;
-#else
-    const int tap = kbeg / g.C;
-    c0 = kbeg - tap * g.C;
-#endif
     kh = tap / g.KW;
     kw = tap - kh * g.KW;
     const int lane = threadIdx.x & 63;
@@ -610,18 +514,7 @@ struct ConvFwdBTap {
     }
     set_tap();
   }
-  __device__ __forceinline__ void fetch(int) {
-    const int wave = __builtin_amdgcn_readfirstlane(gwave());
-#pragma unroll
-    for (int e = 0; e < KR; ++e) {
-      const uint32_t soff = (uint32_t)((c0 + wave + 4 * e) * IHW) * 4u;
-#pragma unroll
-      for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
-    }
-    advance();
-  }
   __device__ __forceinline__ void advance() {
-#if LNN_CB_MAJOR
     ++kw;                                   // next tap of the same channel block ...
     if (kw == KW) {
       kw = 0;
@@ -629,15 +522,6 @@ struct ConvFwdBTap {
       if (kh == KH) { kh = 0; c0 += BK; }   // ... then the next block, from the first tap
     }
     set_tap();
-#else
-    c0 += BK;
-    if (c0 >= C) {   // wave-uniform: next tap
-      c0 = 0;
-      ++kw;
-      if (kw == KW) { kw = 0; ++kh; }
-      set_tap();
-    }
-#endif
   }
   // straight into the LDS stage: element (k = wave + 4e, column lane + 64c)
   __device__ __forceinline__ int issue(int k0, float* lds, int ld, int off) { return issue_part<0, 1>(k0, lds, ld, off); }
@@ -654,21 +538,13 @@ struct ConvFwdBTap {
     if (PART == NPARTS - 1) advance();
     return (KR * (PART + 1) / NPARTS - KR * PART / NPARTS) * CC;
   }
-  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
-    const int wave = gwave(), lane = threadIdx.x & 63;
-#pragma unroll
-    for (int e = 0; e < KR; ++e)
-#pragma unroll
-      for (int c = 0; c < CC; ++c)
-        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
-  }
 };
 
 // OBM: K order with the block of BK output channels as the outer loop and the class's taps as the inner one (the
-// counterpart of LNN_CB_MAJOR in ConvFwdBTap, for the same reason); otherwise tap-major.
-template <int R, bool DIR = false, bool OBM = false>
+// counterpart of the K order of ConvFwdBTap, for the same reason); otherwise tap-major.
+template <int R, bool OBM>
 struct ConvDgradBTap {
-  static constexpr bool KC = false, DIRECT = DIR;
+  static constexpr bool KC = false, DIRECT = true;
   static constexpr int CC = (R + 63) / 64;
   static constexpr int NLD = KR * CC;
   rsrc_t rs;
@@ -686,7 +562,6 @@ struct ConvDgradBTap {
       voff[c] = ok ? (uint32_t)(base[c] + oh * OW + ow) * 4u : OOB;
     }
   }
-  float v[KR][CC];
   __device__ __forceinline__ void init(rsrc_t r, const ConvGeom& g, const KEntry* tab_, int p0, int P, int kbeg, int nt_ = 0) {
     rs = r;
     tab = as_ktab(tab_);
@@ -717,16 +592,6 @@ struct ConvDgradBTap {
       base[c] = (int)img * g.O * g.OHW;
     }
     set_tap();
-  }
-  __device__ __forceinline__ void fetch(int) {
-    const int wave = __builtin_amdgcn_readfirstlane(gwave());
-#pragma unroll
-    for (int e = 0; e < KR; ++e) {
-      const uint32_t soff = (uint32_t)((o0 + wave + 4 * e) * OHW) * 4u;
-#pragma unroll
-      for (int c = 0; c < CC; ++c) v[e][c] = buf_load_s(rs, voff[c], soff);
-    }
-    advance();
   }
   __device__ __forceinline__ void advance() {
     if (OBM) {
@@ -761,14 +626,6 @@ struct ConvDgradBTap {
     if (PART == NPARTS - 1) advance();
     return (KR * (PART + 1) / NPARTS - KR * PART / NPARTS) * CC;
   }
-  __device__ __forceinline__ void commit(float* lds, int ld, int off) const {
-    const int wave = gwave(), lane = threadIdx.x & 63;
-#pragma unroll
-    for (int e = 0; e < KR; ++e)
-#pragma unroll
-      for (int c = 0; c < CC; ++c)
-        if (R % 64 == 0 || lane + 64 * c < R) lds[(wave + 4 * e) * ld + off + lane + 64 * c] = v[e][c];
-  }
 };
 
 // dgrad weight operand read from the weights in the layout the tap-major forward pass reads,
@@ -795,18 +652,11 @@ struct ConvDgradATapMC {
     rs = r;
     tab = as_ktab(tab_);
     ld = g.KK * g.C; O = g.O; C = g.C; nt = nt_;
-#if LNN_CB_MAJOR
     const int t0 = kbeg / BK, ob = nt > 0 ? t0 / nt : 0;
     tap = t0 - ob * nt;
     o0 = ob * BK;
     cw = (tab + tap)->w;
     nw = (tab + (tap + 1 == nt ? 0 : tap + 1))->w;
-#else
-    tap = kbeg / g.O;
-    o0 = kbeg - tap * g.O;
-    cw = (tab + tap)->w;
-    nw = (tab + tap + 1)->w;
-#endif
     const int wave = gwave(), lane = threadIdx.x & 63;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -826,19 +676,9 @@ struct ConvDgradATapMC {
       if (NI % 4 == 0 || q < NI) { buf_load_lds16(rs, lds + off * BK + q * 256, voff[e], soff); ++n; }
     }
     if (PART == NPARTS - 1) {
-#if LNN_CB_MAJOR
       if (++tap == nt) { tap = 0; o0 += BK; }
       cw = nw;
       nw = (tab + (tap + 1 == nt ? 0 : tap + 1))->w;
-#else
-      o0 += BK;
-      if (o0 >= O) {   // wave-uniform: next tap of the class
-        o0 = 0;
-        ++tap;
-        cw = nw;
-        nw = (tab + tap + 1)->w;
-      }
-#endif
     }
     return n;
   }
@@ -1257,14 +1097,11 @@ struct ConvWgradTapA4Direct {
   }
 };
 
-// DIR = false: the same gather through registers (cheaper to issue than
-// transfers into LDS), parked into the same swizzled layout one step later.
-template <int R, bool DIR = true>
+template <int R>
 struct ConvWgradTapBDirect {
-  static constexpr bool KC = true, DIRECT = DIR;
+  static constexpr bool KC = true, DIRECT = true;
   static constexpr int LAYOUT = LAY_KC_SWZ;
   static constexpr int E = R / 8, NLD = E;
-  float v[E];
   static_assert(R % 8 == 0, "whole row pairs for all four wavefronts");
   rsrc_t rs;
   int IH, IW, IHW, OH, OW, kend;
@@ -1294,30 +1131,20 @@ struct ConvWgradTapBDirect {
     iw = ow * g.S + kw * g.D - g.PADL;
     xoff = ((int)img * g.C + c0 + 2 * gwave() + (int)((threadIdx.x & 63) >> 5)) * g.IHW + ih * g.IW + iw;
   }
-  __device__ __forceinline__ int issue(int, float* lds, int, int off) { go<true, 0, 1>(lds, off); return E; }
+  __device__ __forceinline__ int issue(int, float* lds, int, int off) { go<0, 1>(lds, off); return E; }
   template <int PART, int NPARTS>
   __device__ __forceinline__ int issue_part(int, float* lds, int, int off) {
-    go<true, PART, NPARTS>(lds, off);
+    go<PART, NPARTS>(lds, off);
     return E * (PART + 1) / NPARTS - E * PART / NPARTS;
   }
-  __device__ __forceinline__ void fetch(int) { go<false, 0, 1>(nullptr, 0); }
-  __device__ __forceinline__ void commit(float* lds, int, int off) const {
-    const int wave = gwave(), lane = threadIdx.x & 63;
-#pragma unroll
-    for (int e = 0; e < E; ++e) lds[(off + 8 * e + 2 * wave) * BK + lane] = v[e];
-  }
-  template <bool TO_LDS, int PART, int NPARTS>
+  template <int PART, int NPARTS>
   __device__ __forceinline__ void go(float* lds, int off) {
     const int wave = __builtin_amdgcn_readfirstlane(gwave());
     const bool ok = p < kend && (uint32_t)ih < (uint32_t)IH && (uint32_t)iw < (uint32_t)IW;
     const uint32_t voff = ok ? (uint32_t)xoff * 4u : OOB;
 #pragma unroll
     for (int e = E * PART / NPARTS; e < E * (PART + 1) / NPARTS; ++e) {
-      const uint32_t soff = (uint32_t)(8 * e * IHW) * 4u;
-      if (TO_LDS)
-        buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, voff, soff);
-      else
-        v[e] = buf_load_s(rs, voff, soff);
+      buf_load_lds4(rs, lds + (off + 8 * e + 2 * wave) * BK, voff, (uint32_t)(8 * e * IHW) * 4u);
     }
     if (PART == NPARTS - 1) {
       p += BK; oh += qh; ow += rw; ih += s_q; iw += s_r; xoff += x_step;
@@ -1634,7 +1461,7 @@ __device__ __forceinline__ void mma_stage_stream(const float* __restrict__ As, c
       // REGIONS (the loops that keep a running stage index): each group is a scheduling region of its own.  With
       // the whole stage in one region their slots were honoured for the first share only and the other transfers
       // went out in one burst (config 3 wgrad 0.242 -> 0.235 ms); the unrolled loops schedule well as one region
-      if (LNN_GROUP_REGIONS && REGIONS) __builtin_amdgcn_sched_barrier(0);
+      if (REGIONS) __builtin_amdgcn_sched_barrier(0);
     } else {
       mfmas(ic<cur>(), ic<0>(), ic<FREE>());
       send(kkc);
@@ -1647,12 +1474,10 @@ __device__ __forceinline__ void mma_stage_stream(const float* __restrict__ As, c
       if (NEXT) read_slots(); else __builtin_amdgcn_sched_group_barrier(0x008, PAIRS, 0);
     }
   };
-#if LNN_VALU_FIRST
   if (REGIONS)
   // vector-ALU instructions of the step (fragment addresses, the loaders' address walks) in one batch at the start:
   // one alone between two MFMAs costs the matrix pipe 13-18 cycles, in a batch 5-9 each
-    __builtin_amdgcn_sched_group_barrier(0x002, LNN_VALU_FIRST, 0);
-#endif
+    __builtin_amdgcn_sched_group_barrier(0x002, 64, 0);
   group(ic<0>());
   group(ic<1>());
   group(ic<2>());
@@ -1745,9 +1570,9 @@ struct request_first<T, std::void_t<decltype(T::REQUEST_FIRST)>> : std::integral
 // A problem whose streaming loop should keep a running stage index (no threefold unrolling: register pressure or code
 // size cost it more than the address arithmetic) declares `static constexpr bool STREAM_UNROLL = false`.
 template <class T, class = void>
-struct stream_unroll : std::integral_constant<bool, LNN_STREAM_UNROLL != 0> {};
+struct stream_unroll : std::true_type {};
 template <class T>
-struct stream_unroll<T, std::void_t<decltype(T::STREAM_UNROLL)>> : std::integral_constant<bool, T::STREAM_UNROLL && LNN_STREAM_UNROLL> {};
+struct stream_unroll<T, std::void_t<decltype(T::STREAM_UNROLL)>> : std::integral_constant<bool, T::STREAM_UNROLL> {};
 
 // Whether the streaming stage makes each MFMA group a scheduling region of its own (see mma_stage_stream): by default
 // the loops that are not unrolled; a problem overrides it with `static constexpr bool STREAM_REGIONS`.
@@ -1836,7 +1661,7 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
         }
       }
     }
-  } else if constexpr (DA && DB && ST == 3 && LNN_STREAM) {
+  } else if constexpr (DA && DB && ST == 3) {
     // No phases: both groups run the same schedule side by side and share the matrix pipes as they come; whenever
     // one wavefront of a SIMD waits (for fragments, at the barrier) the other one's MFMAs fill the pipe.  During K
     // step t every wavefront sends the transfers of step t+2 off, in shares between its MFMAs, into the stage that
@@ -1932,7 +1757,7 @@ __device__ __forceinline__ void group_body(const P& p, float* ldsA, float* ldsB,
       for (int phase = 0; phase < 2; ++phase) {
         if (phase == G) {
           compute(cur);
-        } else if constexpr (DA && DB && (LNN_REQUEST_FIRST || request_first<P>::value)) {
+        } else if constexpr (DA && DB && request_first<P>::value) {
           // K step t+2 goes out first (into the stage last read for step t-1), then the wait for step t+1, which
           // has been in flight for a whole step, leaves those newest transfers outstanding: every transfer gets
           // close to two steps to land, which short steps (narrow tiles) need
