@@ -528,7 +528,9 @@ static ReduceArgs reduce_args(const ConvArgs& a, int final_beta) {
   r.n = a.M * a.Ncols; r.slices = a.ksplit; r.slices_last = a.ksplit; r.beta = final_beta; r.ncols = a.Ncols;
   r.bm_log = WM == 4 ? 7 : (WM == 2 ? 6 : 5); r.uw_log = WN == 4 ? 7 : (WN == 2 ? 6 : 5);
   r.per_mt = 0; r.last_unit0 = 0x7fffffff;
+  r.kk = 0;
   if (wgrad_tap(PASS)) {
+    r.kk = a.g.KK;
     r.slices_last = a.ks_last;
     r.per_mt = a.seg_units * a.segs_per_mt;
     r.last_unit0 = (a.n_chunks - 1) * a.chunk_units;
@@ -542,7 +544,10 @@ static ReduceArgs reduce_args(const ConvArgs& a, int final_beta) {
 template <int PASS, int WM>
 static int launch_reduce(DeviceCtx* ctx, const ConvArgs& a, float* final_out, int final_beta) {
   const ReduceArgs r = reduce_args<PASS, WM>(a, final_beta);
-  if (a.Ncols % 4 == 0)   // partial buffers start 256-byte aligned
+  if (wgrad_tap(PASS) && a.Ncols % 4 == 0 && a.Ncols >= 256 && (size_t)a.Ncols * sizeof(float) <= 64 * 1024 && !r.post.any())
+    hipLaunchKernelGGL(reduce_partials_rows, dim3(a.M), dim3(256), (size_t)a.Ncols * sizeof(float), ctx->stream, final_out,
+                       static_cast<const float*>(a.Out), r);
+  else if (a.Ncols % 4 == 0)   // partial buffers start 256-byte aligned
     hipLaunchKernelGGL(reduce_partials4, dim3((r.n + reduce4_block(r) - 1) / reduce4_block(r)), dim3(256), 0, ctx->stream, final_out,
                        static_cast<const float*>(a.Out), r);
   else
@@ -601,7 +606,8 @@ static size_t plan_tiles(ConvArgs& a, long long slots, bool allow_tail = false) 
 template <int PASS, int WM, int NTMAX>
 static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   constexpr int WN = 4 / WM, BM = 32 * WM;
-  const long long slots = ctx->cus;   // one 512-thread workgroup per compute unit
+  // one 512-thread workgroup per compute unit; two of the 64 x 128 tiles, whose three LDS stages take 72 KB
+  const long long slots = (long long)ctx->cus * (WM == 2 && NTMAX == 1 ? 2 : 1);
   float* final_out = a.Out;
   const int final_beta = a.beta;
   int grid_y = 1;
@@ -816,6 +822,19 @@ static int launch_classes(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_
 template <int PASS>
 static int launch_classes_by_m(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_t ws_off) {
   const int M = cls[0].M;
+  if (PASS == PASS_DGRAD_TAPW && M > 64 && cls.size() == 4) {
+    // Four classes of a deep layer (few pixels, long K): every workgroup's piece is a handful of K steps, and filling
+    // and draining the pipeline costs as much as computing.  On 64 x 128 tiles two workgroups share a compute unit and
+    // one computes while the other fills or stores (128 -> 256 and 256 -> 512 channels, 5x5 stride 2, at 16 x 16 and
+    // 8 x 8: 80 -> 73 and 74 -> 69 us; 64 x 256 tiles, one workgroup per compute unit: 82 and 83).
+    bool few = true;
+    for (const ConvArgs& a : cls) few = few && (long long)((a.M + 127) / 128) * ((a.Ncols + 31) / 32) < ctx->cus;
+    if (few) {
+      std::sort(cls.begin(), cls.end(), [](const ConvArgs& x, const ConvArgs& y) { return x.K > y.K; });
+      std::swap(cls[2], cls[3]);
+      return launch_classes<PASS, 2, 1>(ctx, cls, ws_off);
+    }
+  }
   if (M > 64) return launch_classes<PASS, 4, 4>(ctx, cls, ws_off);
   if (PASS == PASS_DGRAD_TAPW && M > 32 && cls.size() == 4) {
     // Four classes with many tiles each and different K lengths (5x5 stride 2: 9, 6, 6 and 4 taps): on 64 x 128
@@ -838,6 +857,16 @@ static int launch_classes_by_m(DeviceCtx* ctx, std::vector<ConvArgs>& cls, size_
 
 template <int PASS>
 static int launch_by_m(DeviceCtx* ctx, ConvArgs& a, bool flag) {
+  if (PASS == PASS_WGRAD_TAP && a.M > 64 && a.g.C % 64 == 0) {
+    // A weight gradient whose 128 x 256 tiles would each be cut into many short K slices (a deep layer: large weight
+    // tensor, few output pixels): on 64 x 128 tiles two workgroups share a compute unit, one computing while the other
+    // fills its pipeline or stores its partial sums (128 -> 256 channels 5x5 at 16 x 16 pixels, batch 16: 79 -> 74 us;
+    // with long slices, or hardly any K split, the larger tile's better operand reuse wins)
+    const int seg = a.g.C / 32, chunk = 2 * (seg < 4 ? seg : 4);
+    const long long total = (long long)((a.M + 127) / 128) * a.g.KK * seg;
+    const long long slices = (long long)ctx->cus * chunk / total, nkt = (a.K + BK - 1) / BK;
+    if (slices >= 4 && nkt < 14 * slices) return launch_pass<PASS, 2, 1>(ctx, a, flag);
+  }
   if (a.M > 64) return launch_pass<PASS, 4, 4>(ctx, a, flag);
   if (a.M > 32) return launch_pass<PASS, 2, 2>(ctx, a, flag);
   return launch_pass<PASS, 1, 1>(ctx, a, flag);

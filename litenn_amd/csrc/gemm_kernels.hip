@@ -110,7 +110,7 @@ static int launch_gemm_reduce(DeviceCtx* ctx, const float* part, int slices, int
                               const PostOp& post) {
   ReduceArgs r;
   r.n = M * N; r.slices = slices; r.slices_last = slices; r.beta = beta; r.ncols = N;
-  r.bm_log = 5; r.uw_log = 5; r.per_mt = 0; r.last_unit0 = 0x7fffffff;
+  r.bm_log = 5; r.uw_log = 5; r.per_mt = 0; r.last_unit0 = 0x7fffffff; r.kk = 0;
   r.dN = make_fastdiv((uint32_t)N);
   r.om.nchw = 0; r.om.ld = ldc; r.om.mtot = 0; r.om.dHW = FastDiv{0, 0, 1};
   r.om.dCW = FastDiv{0, 0, 1}; r.om.s = 0; r.om.iw = 0; r.om.org = 0;

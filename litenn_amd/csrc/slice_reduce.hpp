@@ -15,6 +15,7 @@ namespace {
 // only slices_last slices.
 struct ReduceArgs {
   int n, slices, slices_last, beta, ncols;
+  int kk;   // KH*KW when the columns are tap-major weight-gradient columns (tap*C + c), else 0
   int bm_log, uw_log, per_mt, last_unit0;
   FastDiv dN;
   OutMap om;
@@ -127,6 +128,52 @@ __device__ __forceinline__ void reduce_body4_few(float* out, const float* part, 
     }
   }
 }
+// Weight gradients (columns tap-major, tap*C + c; result stored [o][c][tap] or [c][o][tap]): one block per GEMM row.
+// The element-wise kernels above store a row's elements KK floats apart, 4 bytes at a time; here the row's sums are
+// parked in LDS at their permuted place c*KK + tap (KK odd for the usual kernels: no bank conflicts) and leave as one
+// contiguous run (whole runs of KK floats per channel for a gradient kept with swapped channel axes).  Slices are
+// added in ascending order, eight loads in flight.  ncols % 4 == 0; ncols floats of dynamic LDS.
+__global__ __launch_bounds__(256) void reduce_partials_rows(float* out, const float* part, ReduceArgs a) {
+  extern __shared__ float reduce_row[];
+  const uint32_t m = blockIdx.x, C = a.om.dHW.d;
+  const size_t n = (size_t)a.n;
+  for (int g = threadIdx.x; 4 * g < a.ncols; g += 256) {
+    const uint32_t col = 4u * g;
+    const size_t i4 = (size_t)m * a.ncols + col;
+    const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
+    const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+    f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+    int k = 0;
+    for (; k + 8 <= ns; k += 8) {
+      f32x4 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const f32x4*>(&part[(size_t)(k + j) * n + i4]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s += v[j];
+    }
+    if (k < ns) {
+      f32x4 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const f32x4*>(&part[(size_t)(k + j < ns ? k + j : k) * n + i4]);
+      const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s += k + j < ns ? v[j] : zero;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t cj = col + j, tap = a.om.dHW.div(cj), c = cj - tap * C;
+      reduce_row[c * a.kk + tap] = s[j];
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < a.ncols; e += 256) {
+    const uint32_t c = (uint32_t)e / (uint32_t)a.kk, tap = (uint32_t)e - c * (uint32_t)a.kk;
+    const size_t o = (size_t)a.om.col(tap * C + c) + (size_t)m * a.om.ld;
+    const float t = reduce_row[e];
+    out[o] = a.beta ? out[o] + t : t;
+  }
+}
+
 // elements per block of the 128-bit reductions
 __host__ __device__ inline int reduce4_block(const ReduceArgs& a) { return a.slices <= kFewSlices ? 1024 : 128; }
 __global__ __launch_bounds__(256) void reduce_partials4(float* out, const float* part, ReduceArgs a) {
