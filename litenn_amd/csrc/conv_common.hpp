@@ -312,10 +312,20 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
     // grid in which the last chunk, if it holds less work, is cut into proportionally fewer slices
     int slice = by, ns = a.ksplit;
     if (wgrad_tap(PASS)) {
-      const int b = bx, nfull = (a.n_chunks - 1) * a.ksplit;
-      if (b < nfull) {
-        chunk_i = b / a.ksplit;
-        slice = b - chunk_i * a.ksplit;
+      // The chunks of one K slice read the same pixels (the same dY, and X windows a few rows apart).  Consecutive
+      // workgroups go to the eight XCDs in turn, each with its own L2, so slices are dealt out in groups of eight:
+      // inside a group of 8 * (full chunks) workgroups the chunk is the slow index and the slice the fast one, which
+      // puts all chunks of a slice on one XCD, where they run side by side and meet their operands in its L2
+      // (3x3 dilated on 64 channels, 9 tap columns in 5 chunks: 162 -> 78 MB fetched per launch; the time does not move).
+      const int b = bx, nc = a.n_chunks - 1, nfull = nc * a.ksplit, grouped = (a.ksplit >> 3) * 8 * nc;
+      if (b < grouped) {
+        const int g = b / (8 * nc), r = b - g * (8 * nc);
+        chunk_i = r >> 3;
+        slice = 8 * g + (r & 7);
+      } else if (b < nfull) {
+        const int r = b - grouped, rem = a.ksplit & 7;
+        chunk_i = r / rem;
+        slice = (a.ksplit & ~7) + (r - chunk_i * rem);
       } else {
         chunk_i = a.n_chunks - 1;
         slice = b - nfull;
