@@ -127,7 +127,7 @@ __device__ __forceinline__ void dw_unit_rows(const float* lds, int lo, int srcH,
     float win[T][T];
 #pragma unroll
     for (int j = 0; j + 1 < KS; ++j) col.load_row(lds, lo, srcH, srcW, ra - pt + j, win[j + 1]);
-    for (int r = ra; r < rb; ++r) {
+    auto row = [&](int r, float old) {
 #pragma unroll
       for (int j = 0; j + 1 < KS; ++j)
 #pragma unroll
@@ -138,8 +138,30 @@ __device__ __forceinline__ void dw_unit_rows(const float* lds, int lo, int srcH,
       for (int a = 0; a < KS; ++a)
 #pragma unroll
         for (int b = 0; b < KS; ++b) v += win[a][b] * w[a * KS + b];
-      const int o = r * dstW + c;
-      dst[o] = beta ? dst[o] + v : v;
+      dst[r * dstW + c] = old + v;
+    };
+    if (!beta) {
+      for (int r = ra; r < rb; ++r) row(r, 0.0f);
+    } else {
+      // '+=': the old values of a run of rows are requested together, ahead of the arithmetic, so that the thread
+      // waits for memory once per run and not once per row
+      constexpr int RUN = 8;
+      int r = ra;
+      for (; r + RUN <= rb; r += RUN) {
+        float old[RUN];
+#pragma unroll
+        for (int j = 0; j < RUN; ++j) old[j] = dst[(r + j) * dstW + c];
+#pragma unroll
+        for (int j = 0; j < RUN; ++j) row(r + j, old[j]);
+      }
+      if (r < rb) {   // the last, shorter run
+        float old[RUN];
+#pragma unroll
+        for (int j = 0; j < RUN; ++j) old[j] = r + j < rb ? dst[(r + j) * dstW + c] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < RUN; ++j)
+          if (r + j < rb) row(r + j, old[j]);
+      }
     }
   }
 }
