@@ -146,6 +146,17 @@ class InStepTimer:
         return {k: v / steps for k, v in out.items()}
 
 
+def launch_floor_ms(api):
+    """What the box charges for any launch through the library: a one-word fill (a kernel with nothing to do), launched
+    back to back and timed like the passes, with HIP events on the library's stream."""
+    tiny = Dev(api, shape=(64,))
+    for _ in range(50):
+        api.fill_u32(0, tiny.ptr, 0, 1)
+    ms = min(time_events(api, lambda: api.fill_u32(0, tiny.ptr, 0, 1), 300) for _ in range(3))
+    tiny.free()
+    return ms
+
+
 def rel_err(got, ref):
     ref = np.asarray(ref, np.float64)
     return float(np.abs(np.asarray(got, np.float64) - ref).max() / max(np.abs(ref).max(), 1e-30))
@@ -293,6 +304,12 @@ def bench_conv(api, name, steps, warmup, cpu=True, cpu_steps=3):
         'frac_mfma_peak_step': 3 * flops / wall_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS,
         'roofline': roof, 'passes': per_pass,
     }
+    if flops < 1e9:   # a problem this small is a launch: say what a launch costs here
+        floor = launch_floor_ms(api)
+        result['launch_floor_ms'] = floor
+        for k in per_pass:
+            per_pass[k]['ms_min'] = min(time_events(api, passes[k], 300) for _ in range(3))
+            per_pass[k]['x_launch_floor'] = per_pass[k]['ms_min'] / floor
     if cpu:
         from oracle import refpath
         cores = refpath.num_threads()
