@@ -268,38 +268,73 @@ __device__ __forceinline__ void store_permuted(const MultiArgs& a, int k, uint64
   const uint32_t C = (uint32_t)(swapped ? -a.wp_c[k] : a.wp_c[k]), o = swapped ? lo : hi, c = swapped ? hi : lo;
   a.wp[k][((size_t)o * a.dKK[k].d + tap) * C + c] = value;
 }
-__global__ void sgd_multi_kernel(MultiArgs a, float momentum, float lr, int nesterov, float drop) {
+// One element of the SGD step (SGD.py:42-74): returns the new parameter value.  With momentum 0 the accumulator's old
+// value has no weight and is not read.
+__device__ __forceinline__ float sgd_element(const MultiArgs& a, int k, uint64_t i, float momentum, float lr, int nesterov,
+                                             float drop) {
+  // the reference's two kernels per tensor draw their dropout masks from separate seeds
+  const float gi = a.g[k][i];
+  const float lr0 = dropped_lr(lr, drop, i, a.seed0[k]);
+  float x;
+  if (momentum != 0.0f) x = momentum * a.s0[k][i] - lr0 * gi;
+  else x = -(lr0 * gi);
+  a.s0[k][i] = x;
+  const float nv = a.t[k][i] + (nesterov ? momentum * x - dropped_lr(lr, drop, i, a.seed1[k]) * gi : x);
+  a.t[k][i] = nv;
+  return nv;
+}
+// One element of the Adam step (Adam.py:44-69)
+__device__ __forceinline__ float adam_element(const MultiArgs& a, int k, uint64_t i, float beta1, float beta2, float lr,
+                                              float drop) {
+  const float gi = a.g[k][i];
+  const float mi = beta1 * a.s0[k][i] + (1.0f - beta1) * gi;
+  const float vi = beta2 * a.s1[k][i] + (1.0f - beta2) * gi * gi;
+  a.s0[k][i] = mi;
+  a.s1[k][i] = vi;
+  const float nt = a.t[k][i] + -dropped_lr(lr, drop, i, a.seed0[k]) * mi / (sqrtf(vi) + 1e-7f);
+  a.t[k][i] = nt;
+  return nt;
+}
+// The walk both optimizers share.  A tensor without a permuted copy: a grid-stride loop.  One stored [O][C][tap] with
+// a copy Wp[o][tap][c]: tiles of one o and up to 64 channels, kMultiTile floats at most - a contiguous run of the
+// tensor, updated in order and parked in LDS, then written to the copy tap by tap, so that the copy too is stored in
+// runs of consecutive channels instead of single floats a whole row apart.  Other copies are stored element by
+// element.
+constexpr int kMultiTile = 4096;
+template <class F>
+__device__ __forceinline__ void update_walk(const MultiArgs& a, F&& element) {
   const int k = blockIdx.y;
   const uint64_t n = a.n[k];
-  float* v = a.t[k];
-  const float* g = a.g[k];
-  float* acc = a.s0[k];
+  const int KK = (int)a.dKK[k].d, C = a.wp_c[k];
+  if (a.wp[k] && C > 0 && KK * (C < 64 ? C : 64) <= kMultiTile) {
+    __shared__ float tile[kMultiTile];
+    const int TL = C < 64 ? C : 64, per_o = (C + TL - 1) / TL;
+    const uint32_t tiles = (uint32_t)(n / ((uint64_t)C * KK)) * per_o;
+    for (uint32_t t = blockIdx.x; t < tiles; t += gridDim.x) {
+      const uint32_t o = t / per_o, c0 = (t - o * per_o) * TL;
+      const int tl = (int)(C - c0) < TL ? (int)(C - c0) : TL, len = tl * KK;
+      const uint64_t base = ((uint64_t)o * C + c0) * KK;
+      for (int e = threadIdx.x; e < len; e += blockDim.x) tile[e] = element(k, base + e);
+      __syncthreads();
+      float* dst = a.wp[k] + (size_t)o * KK * C + c0;
+      for (int e = threadIdx.x; e < len; e += blockDim.x) {
+        const int tap = e / tl, cl = e - tap * tl;
+        dst[(size_t)tap * C + cl] = tile[cl * KK + tap];
+      }
+      __syncthreads();
+    }
+    return;
+  }
   for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    // the reference's two kernels per tensor (SGD.py:42-74) draw their dropout masks from separate seeds
-    const float x = momentum * acc[i] - dropped_lr(lr, drop, i, a.seed0[k]) * g[i];
-    acc[i] = x;
-    const float nv = v[i] + (nesterov ? momentum * x - dropped_lr(lr, drop, i, a.seed1[k]) * g[i] : x);
-    v[i] = nv;
+    const float nv = element(k, i);
     if (a.wp[k]) store_permuted(a, k, i, nv);
   }
 }
-__global__ void adam_multi_kernel(MultiArgs a, float beta1, float beta2, float lr, float drop) {
-  const int k = blockIdx.y;
-  const uint64_t n = a.n[k];
-  float* t = a.t[k];
-  const float* g = a.g[k];
-  float* m = a.s0[k];
-  float* v2 = a.s1[k];
-  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
-    const float gi = g[i];
-    const float mi = beta1 * m[i] + (1.0f - beta1) * gi;
-    const float vi = beta2 * v2[i] + (1.0f - beta2) * gi * gi;
-    m[i] = mi;
-    v2[i] = vi;
-    const float nt = t[i] + -dropped_lr(lr, drop, i, a.seed0[k]) * mi / (sqrtf(vi) + 1e-7f);
-    t[i] = nt;
-    if (a.wp[k]) store_permuted(a, k, i, nt);
-  }
+__global__ __launch_bounds__(256) void sgd_multi_kernel(MultiArgs a, float momentum, float lr, int nesterov, float drop) {
+  update_walk(a, [&](int k, uint64_t i) { return sgd_element(a, k, i, momentum, lr, nesterov, drop); });
+}
+__global__ __launch_bounds__(256) void adam_multi_kernel(MultiArgs a, float beta1, float beta2, float lr, float drop) {
+  update_walk(a, [&](int k, uint64_t i) { return adam_element(a, k, i, beta1, beta2, lr, drop); });
 }
 
 // ---------------------------------------------------------------------------
@@ -497,7 +532,7 @@ constexpr int kEpiPiece = 2048;
 __global__ __launch_bounds__(256) void bias_act_bwd_kernel(int N, int O, int HW, int ppp, int slices,
                                                            const float* __restrict__ y, const float* dy,
                                                            int act, float slope, float* dpre,
-                                                           float* __restrict__ part, int vec) {
+                                                           float* __restrict__ part, int vec, float* dbias, int beta) {
   const int o = blockIdx.y, sl = blockIdx.x;
   const long long total = (long long)N * ppp;
   const long long p0 = total * sl / slices, p1 = total * (sl + 1) / slices;
@@ -530,13 +565,16 @@ __global__ __launch_bounds__(256) void bias_act_bwd_kernel(int N, int O, int HW,
       }
     }
   }
-  if (!part) return;
+  if (!part && !dbias) return;
   __shared__ float red[4];
 #pragma unroll
   for (int s = 32; s > 0; s >>= 1) acc += __shfl_xor(acc, s, 64);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
   __syncthreads();
-  if (threadIdx.x == 0) part[(size_t)o * slices + sl] = (red[0] + red[1]) + (red[2] + red[3]);
+  if (threadIdx.x != 0) return;
+  const float sum = (red[0] + red[1]) + (red[2] + red[3]);
+  if (dbias) dbias[o] = beta ? dbias[o] + sum : sum;   // the channel's only slice: no partial sums to add up
+  else part[(size_t)o * slices + sl] = sum;
 }
 
 // The same for planes of one element, a dense layer's y[rows][O]: a thread owns a feature and walks down its
@@ -600,9 +638,12 @@ int launch_bias_act_bwd(DeviceCtx* ctx, int N, int O, int HW, const float* y, co
   const long long total = (long long)N * ppp;
   long long slices = ((long long)ctx->cus * 8 + O - 1) / O;
   if (slices > total) slices = total;
+  // a block per channel already fills the device and a channel is short: the block stores the bias gradient itself
+  if (O >= ctx->cus && (long long)N * HW <= 8192) slices = 1;
   if (slices < 1) slices = 1;
+  const bool direct = dbias && slices == 1;
   float* part = nullptr;
-  if (dbias) {
+  if (dbias && !direct) {
     int st = ensure_workspace(ctx, (size_t)O * slices * sizeof(float));
     if (st != LNN_OK) return st;
     part = static_cast<float*>(ctx->ws);
@@ -610,9 +651,9 @@ int launch_bias_act_bwd(DeviceCtx* ctx, int N, int O, int HW, const float* y, co
   auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   const int vec = HW % 4 == 0 && aligned(dy) && aligned(y) && aligned(dpre);
   hipLaunchKernelGGL(bias_act_bwd_kernel, dim3((unsigned)slices, (unsigned)O), dim3(256), 0, ctx->stream, N, O, HW, ppp,
-                     (int)slices, y, dy, act, slope, dpre, part, vec);
+                     (int)slices, y, dy, act, slope, dpre, part, vec, direct ? dbias : nullptr, beta ? 1 : 0);
   LNN_HIP(hipGetLastError());
-  if (dbias) {
+  if (dbias && !direct) {
     hipLaunchKernelGGL(bias_act_bwd_finish_kernel, dim3((O + 255) / 256), dim3(256), 0, ctx->stream, O, (int)slices, part,
                        dbias, beta ? 1 : 0);
     LNN_HIP(hipGetLastError());

@@ -855,16 +855,21 @@ def test_multi_tensor_updates_refresh_permuted_copies(hip):
     Wp[o][tap][c] of the new values, for tensors stored [O][C][taps] and [C][O][taps]; tensors without a copy, an empty tensor and more tensors than one launch holds
     among them.  A copy whose channel and tap counts do not divide the tensor is refused."""
     rs = np.random.RandomState(78)
-    shapes = [(32, 32, 9), None, (64, 3, 49), (5, 7, 1), None, (40, 24, 25), (8, 130, 4)] + [None] * 12 + [(3, 5, 6)]
-    lays = [hip.W_OIHW, 0, hip.W_IOHW, hip.W_IOHW, 0, hip.W_OIHW, hip.W_IOHW] + [0] * 12 + [hip.W_IOHW]   # (O, C, KK) above
+    # (O, C, KK); [O][C][taps] tensors with fewer than 64 channels, a ragged last run of 64, whole runs, and taps x 64
+    # beyond what the kernel stages at once
+    shapes = ([(32, 32, 9), None, (64, 3, 49), (5, 7, 1), None, (40, 24, 25), (8, 130, 4), (6, 130, 9), (4, 64, 25),
+               (2, 200, 16), (2, 64, 81)] + [None] * 8 + [(3, 5, 6)])
+    lays = ([hip.W_OIHW, 0, hip.W_IOHW, hip.W_IOHW, 0, hip.W_OIHW, hip.W_IOHW] + [hip.W_OIHW] * 4 + [0] * 8
+            + [hip.W_IOHW])
     sizes = [int(np.prod(sh)) if sh else 37 + i for i, sh in enumerate(shapes)]
     sizes[4] = 0
     mk = lambda: [rs.standard_normal(max(n, 1)).astype(np.float32) for n in sizes]
     v0, g0, a0, b0 = mk(), mk(), mk(), [np.abs(x) for x in mk()]
     cs = [sh[1] if sh else 0 for sh in shapes]
     kks = [sh[2] if sh else 0 for sh in shapes]
-    for kind in ('sgd', 'sgd_nesterov', 'adam'):
+    for kind in ('sgd', 'sgd_nesterov', 'sgd_no_momentum', 'adam'):
         say(f'multi-tensor update with permuted copies {kind}')
+        mom = 0.0 if kind == 'sgd_no_momentum' else 0.9
         plain = [[DevArr(hip, x) for x in arrs] for arrs in (v0, g0, a0, b0)]
         fused = [[DevArr(hip, x) for x in arrs] for arrs in (v0, g0, a0, b0)]
         wps = [DevArr(hip, shape=(n,), fill=np.nan) if sh else None for sh, n in zip(shapes, sizes)]
@@ -874,8 +879,11 @@ def test_multi_tensor_updates_refresh_permuted_copies(hip):
             hip.adam_update_multi(0, sizes, pp[0], pp[1], pp[2], pp[3], 0.9, 0.999, 1e-2)
             hip.adam_update_multi_wp(0, sizes, pf[0], pf[1], pf[2], pf[3], 0.9, 0.999, 1e-2, wptrs, cs, kks, lays)
         else:
-            hip.sgd_update_multi(0, sizes, pp[0], pp[1], pp[2], 0.9, 1e-2, kind == 'sgd_nesterov')
-            hip.sgd_update_multi_wp(0, sizes, pf[0], pf[1], pf[2], 0.9, 1e-2, kind == 'sgd_nesterov', wptrs, cs, kks, lays)
+            hip.sgd_update_multi(0, sizes, pp[0], pp[1], pp[2], mom, 1e-2, kind == 'sgd_nesterov')
+            hip.sgd_update_multi_wp(0, sizes, pf[0], pf[1], pf[2], mom, 1e-2, kind == 'sgd_nesterov', wptrs, cs, kks, lays)
+            if mom == 0.0:   # the accumulator's old value is not read: the new one is -lr * g
+                for acc, g, n in zip(fused[2], g0, sizes):
+                    assert n == 0 or np.array_equal(acc.get(), np.float32(-1e-2) * g)
         for col_p, col_f in zip(plain, fused):
             for x, y in zip(col_p, col_f):
                 assert np.array_equal(x.get(), y.get())
@@ -895,7 +903,7 @@ def test_bias_act_bwd_one_pass(hip):
     the largest |dbias| on floats (fp32 sums against fp64)."""
     rs = np.random.RandomState(21)
     cases = [(1, 1, 1), (2, 3, 7), (4, 8, 56 * 56), (3, 5, 2048), (2, 4, 2049 * 4), (1, 2, 5000), (5, 130, 36),
-             (64, 16, 32 * 32), (1, 300, 3)]
+             (64, 16, 32 * 32), (1, 300, 3), (4, 300, 64), (2, 512, 100), (16, 256, 256)]
     for N, O, HW in cases:
         for act, slope in [(hip.ACT_LEAKY_RELU, 0.25), (hip.ACT_NONE, 0.0)]:
             say(f'bias_act_bwd N={N} O={O} HW={HW} act={act}')
