@@ -194,7 +194,10 @@ int lnn_conv2d_wgrad_iohw_f32(int dev, const lnn_conv2d_desc* d, const float* X,
  * device the partial sums never exceed 32 MiB, so only the added table of an unusually shaped problem can.
  * The one-time set-up of a device (stream, address of the array) happens in the first call of ANY entry point on
  * that device; after it this function calls no hipMalloc / hipFree or other allocating routine.  All calls on one
- * GPU share the array: calls that overlap in time on one GPU (from two threads) race. */
+ * GPU share the array: calls that overlap in time on one GPU (from two threads) race.  For its duration the call
+ * also points the device's scratch bookkeeping at the array and forbids allocation on that device, so it must not
+ * overlap with ANY other entry point of this library on the same GPU either: one running beside it from a second
+ * thread could fail with LNN_ERR_UNSUPPORTED or place its own scratch data in the array. */
 #define LNN_NOALLOC_SCRATCH_BYTES (32u << 20)
 int lnn_conv2d_wgrad_noalloc_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
                                  float* dW, int beta);

@@ -9,9 +9,10 @@ _seq = operator.methodcaller('_get_seq_id')
 
 # Per-sweep state for gradient functions that share an intermediate result (the fused convolution epilogue forms
 # its pre-activation gradient once for three gradient functions): a counter that identifies the running sweep
-# (None outside one) and callbacks run when the sweep ends, so nothing computed from one sweep's gradients is reused
-# by the next and nothing keeps gradient-sized tensors alive after it.
-_sweep = {'id': 0, 'active': None, 'cleanups': []}
+# (None outside one) and callbacks run when the gradient functions of the tensor being visited are done, so nothing
+# computed from one sweep's gradients is reused by the next and nothing keeps gradient-sized tensors alive longer
+# than their readers.
+_sweep = {'id': 0, 'active': None, 'tensor_cleanups': []}
 
 
 def current_sweep():
@@ -19,12 +20,20 @@ def current_sweep():
     return _sweep['active']
 
 
-def at_end_of_sweep(fn):
-    """Call fn() when the backward() call in progress returns (at once if none is running)."""
+def after_gradfns_of_tensor(fn):
+    """Call fn() once the gradient functions of the tensor the running backward() is visiting have all run (at once
+    if no backward() is running): what they share - an intermediate formed by the first and read by the others -
+    can be let go there instead of living until the sweep ends."""
     if _sweep['active'] is None:
         fn()
     else:
-        _sweep['cleanups'].append(fn)
+        _sweep['tensor_cleanups'].append(fn)
+
+
+def _run_tensor_cleanups():
+    fns, _sweep['tensor_cleanups'] = _sweep['tensor_cleanups'], []
+    for fn in fns:
+        fn()
 
 
 
@@ -48,9 +57,8 @@ def backward(loss, stop_grad=None, grad_for_non_trainables=False, keep_gradient_
     try:
         _backward(loss, stop_grad, grad_for_non_trainables)
     finally:
-        cleanups, _sweep['cleanups'], _sweep['active'] = _sweep['cleanups'], [], None
-        for fn in cleanups:
-            fn()
+        _run_tensor_cleanups()
+        _sweep['active'] = None
 
 
 def _backward(loss, stop_grad, grad_for_non_trainables):
@@ -99,6 +107,7 @@ def _backward(loss, stop_grad, grad_for_non_trainables):
                 src = input_t._get_top_reference_source()
                 if not any(src is p for p in pending):
                     pending.append(src)
+            _run_tensor_cleanups()
         if not grad_for_non_trainables and not t._is_trainable():
             t.free_grad()
 

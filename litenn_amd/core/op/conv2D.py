@@ -1,6 +1,6 @@
 import litenn_amd as nn
 import litenn_amd.core as nc
-from ..backward import at_end_of_sweep, current_sweep
+from ..backward import after_gradfns_of_tensor, current_sweep
 from ..hip import api, launch, permuted_weights, ShallowMode
 
 
@@ -100,11 +100,11 @@ class _EpilogueGrad:
         if want_pre:
             pre = nn.Tensor(dO_t.shape)
             self.value = pre
-            # valid for the gradient functions of this sweep only: the next sweep's dO holds other values in the same
-            # tensor object, and the tensors are released when the sweep ends
+            # valid for the gradient functions of this output in this sweep only: they run one after the other, and
+            # the tensor is let go when the last of them has
             if current_sweep() is not None:
                 self.key = (current_sweep(), dO_t)
-                at_end_of_sweep(self._drop)
+                after_gradfns_of_tensor(self._drop)
         args = [O_t, dO_t]
         if pre is not None:
             args.append((pre, 'w'))

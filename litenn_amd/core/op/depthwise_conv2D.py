@@ -21,18 +21,18 @@ def depthwise_conv2D(input_t, kernel_t, stride=1, dilation=1, padding='same'):
     output_t._set_op_name('depthwise_conv2D')
     output_t._assign_gradfn(input_t, lambda O_t, dO_t: depthwise_dI_gradfn(op, input_t, kernel_t, dO_t))
     output_t._assign_gradfn(kernel_t, lambda O_t, dO_t: depthwise_dK_gradfn(op, input_t, kernel_t, dO_t))
-    launch(lambda dev, x, k, y: api.depthwise_conv2d_fwd(dev, op.desc, x, k, y, 0), input_t, kernel_t, (output_t, 'w'))
+    launch(lambda dev, x, k, y: api.depthwise_conv2d_fwd(dev, op.desc, x, k, y, 0), (input_t, 'r'), (kernel_t, 'r'), (output_t, 'w'))
     return output_t
 
 
 def depthwise_dI_gradfn(op, input_t, kernel_t, dO_t):
     grad_t, beta = nc.op.accumulate_target(input_t.get_grad())
-    launch(lambda dev, dy, k, dx: api.depthwise_conv2d_dgrad(dev, op.desc, dy, k, dx, beta), dO_t, kernel_t, grad_t)
+    launch(lambda dev, dy, k, dx: api.depthwise_conv2d_dgrad(dev, op.desc, dy, k, dx, beta), (dO_t, 'r'), (kernel_t, 'r'), grad_t)
 
 
 def depthwise_dK_gradfn(op, input_t, kernel_t, dO_t):
     grad_t, beta = nc.op.accumulate_target(kernel_t.get_grad())
-    launch(lambda dev, x, dy, dk: api.depthwise_conv2d_wgrad(dev, op.desc, x, dy, dk, beta), input_t, dO_t, grad_t)
+    launch(lambda dev, x, dy, dk: api.depthwise_conv2d_wgrad(dev, op.desc, x, dy, dk, beta), (input_t, 'r'), (dO_t, 'r'), grad_t)
 
 
 class _DepthwiseConv2DOp:

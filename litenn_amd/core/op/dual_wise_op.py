@@ -26,7 +26,7 @@ def dual_wise_op(kind, a_t, b_t, output_t=None, is_add_to_output=False):
     aliased = src_out is a_t._get_top_reference_source() or src_out is b_t._get_top_reference_source()
     out_arg = output_t if (is_add_to_output or aliased) else (output_t, 'w')
     o_s, a_s, b_s = tuple(info.output_shape), tuple(info.a_br_shape), tuple(info.b_br_shape)
-    launch(lambda dev, a, b, o: api.binary_bcast(dev, code, o_s, a_s, b_s, a, b, o, beta), a_t, b_t, out_arg)
+    launch(lambda dev, a, b, o: api.binary_bcast(dev, code, o_s, a_s, b_s, a, b, o, beta), (a_t, 'r'), (b_t, 'r'), out_arg)
     return output_t
 
 
@@ -40,20 +40,20 @@ def _operand_gradfn(kind, info, which, a_t, b_t, dO_t):
         other_s = tuple((info.b_br_shape, info.a_br_shape)[which])
         if red.rank == 0:
             launch(lambda dev, do, ot, g: api.binary_bcast(dev, api.BIN_MUL, o_s, o_s, other_s, do, ot, g, 1),
-                   dO_t, other, target.get_grad())
+                   (dO_t, 'r'), (other, 'r'), target.get_grad())
             return
         tmp = nn.Tensor(info.output_shape)
         launch(lambda dev, do, ot, g: api.binary_bcast(dev, api.BIN_MUL, o_s, o_s, other_s, do, ot, g, 0),
-               dO_t, other, (tmp, 'w'))
+               (dO_t, 'r'), (other, 'r'), (tmp, 'w'))
         src, scale = tmp, 1.0
     else:
         src, scale = dO_t, (-1.0 if (kind == 'sub' and which == 1) else 1.0)
     if red.rank == 0:
         n = info.output_shape.size
-        launch(lambda dev, s, g: api.ew_fwd(dev, api.EW_MUL_CONST, n, s, g, scale, 1), src, target.get_grad())
+        launch(lambda dev, s, g: api.ew_fwd(dev, api.EW_MUL_CONST, n, s, g, scale, 1), (src, 'r'), target.get_grad())
     else:
         # sum over the broadcast axes into the operand's gradient
-        launch(lambda dev, s, g: api.reduce_sum(dev, o_s, tuple(red), scale, s, g, 1), src, target.get_grad())
+        launch(lambda dev, s, g: api.reduce_sum(dev, o_s, tuple(red), scale, s, g, 1), (src, 'r'), target.get_grad())
 
 
 def add_op(a_t, b_t, output_t=None, is_add_to_output=False): return dual_wise_op('add', a_t, b_t, output_t, is_add_to_output)

@@ -30,14 +30,14 @@ def element_wise_op(kind, param, input_t, output_t=None, is_add_to_output=False)
     beta = 1 if is_add_to_output else 0
     in_place = output_t._get_top_reference_source() is input_t._get_top_reference_source()
     out_arg = output_t if (is_add_to_output or in_place) else (output_t, 'w')
-    launch(lambda dev, i, o: api.ew_fwd(dev, code, n, i, o, param, beta), input_t, out_arg)
+    launch(lambda dev, i, o: api.ew_fwd(dev, code, n, i, o, param, beta), (input_t, 'r'), out_arg)
     return output_t
 
 
 def _input_gradfn(code, param, input_t, dO_t):
     n = input_t.shape.size
     grad_t, beta = nc.op.accumulate_target(input_t.get_grad())
-    launch(lambda dev, i, do, di: api.ew_bwd(dev, code, n, i, do, di, param, beta), input_t, dO_t, grad_t)
+    launch(lambda dev, i, do, di: api.ew_bwd(dev, code, n, i, do, di, param, beta), (input_t, 'r'), (dO_t, 'r'), grad_t)
 
 
 def add_const_op(input_t, value, output_t=None, is_add_to_output=False):

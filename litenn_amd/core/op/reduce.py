@@ -20,14 +20,14 @@ def reduce_op(op_type, input_t, axes=None, keepdims=False, output_t=None, is_add
         raise ValueError(f'output_t must have size {op.info.output_shape.size}')
     beta = 1 if is_add_to_output else 0
     out_arg = output_t if is_add_to_output else (output_t, 'w')
-    launch(lambda dev, i, o: api.reduce_sum(dev, op.shape, op.axes, op.scale, i, o, beta), input_t, out_arg)
+    launch(lambda dev, i, o: api.reduce_sum(dev, op.shape, op.axes, op.scale, i, o, beta), (input_t, 'r'), out_arg)
     return output_t
 
 
 def reduce_dI_gradfn(op, input_t, O_t, dO_t):
     # in.grad[idx] += dO[idx with reduced axes dropped] (/ count for mean)   (reduce.py:243-255)
     grad_t, beta = nc.op.accumulate_target(input_t.get_grad())
-    launch(lambda dev, do, di: api.reduce_sum_bwd(dev, op.shape, op.axes, op.scale, do, di, beta), dO_t, grad_t)
+    launch(lambda dev, do, di: api.reduce_sum_bwd(dev, op.shape, op.axes, op.scale, do, di, beta), (dO_t, 'r'), grad_t)
 
 
 class _ReduceOp:

@@ -21,7 +21,7 @@ def transpose_op(input_t, axes_order, output_t=None, is_add_to_output=False):
         raise ValueError(f'output_t must have size {op.info.output_shape.size}')
     beta = 1 if is_add_to_output else 0
     out_arg = output_t if is_add_to_output else (output_t, 'w')
-    launch(lambda dev, i, o: api.transpose(dev, op.shape, op.axes, i, o, beta), input_t, out_arg)
+    launch(lambda dev, i, o: api.transpose(dev, op.shape, op.axes, i, o, beta), (input_t, 'r'), out_arg)
     return output_t
 
 

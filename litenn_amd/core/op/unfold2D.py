@@ -32,5 +32,5 @@ def unfold2D(input_t, N, C, H, W, OH, OW, KH, KW, PADL, PADT, DILATION, STRIDE, 
     beta = 1 if is_add_to_output else 0
     out_arg = output_t if is_add_to_output else (output_t, 'w')
     launch(lambda dev, i, o: api.unfold2d(dev, N, C, H, W, OH, OW, KH, KW, PADL, PADT, DILATION, STRIDE, order,
-                                          bool(is_transpose), i, o, beta), input_t, out_arg)
+                                          bool(is_transpose), i, o, beta), (input_t, 'r'), out_arg)
     return output_t

@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
 #pragma unroll
         for (int c = 0; c < CN; ++c) acc[q][i][j][c] = 0.0f;
   const uint32_t plane = (uint32_t)a.OH * a.OW;
-  // this image's dY: a channel past the last one lies past the end of the buffer and reads as zero
+  // this image's dY
   const rsrc_t rs = make_rsrc(a.dY + (size_t)n * a.O * plane, (uint32_t)a.O * plane * 4u);
   // where this lane's element of each transfer lies in dY, relative to the chunk's first channel
   uint32_t voff[NTR];
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
     const bool ok = f < CHUNK && r < a.th && c < a.tw && (uint32_t)oh < (uint32_t)a.OH && (uint32_t)ow < (uint32_t)a.OW;
     voff[t] = ok ? ((uint32_t)o * plane + (uint32_t)oh * a.OW + (uint32_t)ow) * 4u : OOB;
   }
-  // the weights Wc[o][tap][4] of a chunk are WCH consecutive floats; output channels past the last read as zero
+  // the weights Wc[o][tap][4] of a chunk are WCH consecutive floats
   const rsrc_t rw = make_rsrc(a.wc, (uint32_t)a.O * KK * 16u);
   uint32_t woff[NTW];
 #pragma unroll
@@ -162,10 +162,16 @@ __global__ __launch_bounds__(256) void small_dgrad_kernel(SmallDgradArgs a) {
   for (int o0 = obeg; o0 < oend; o0 += kDsOC) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the previous chunk has been read
     const uint32_t soff = (uint32_t)o0 * plane * 4u;
+    // a last chunk with fewer than kDsOC channels: the lanes of the missing ones ask for nothing (their range test is
+    // made on the vector offset, whatever the hardware does with the scalar one)
+    const int live = a.O - o0;
 #pragma unroll
-    for (int t = 0; t < NTR; ++t) buf_load_lds4(rs, tile + t * 64, voff[t], soff);
+    for (int t = 0; t < NTR; ++t)
+      buf_load_lds4(rs, tile + t * 64, live >= kDsOC || (t * 64 + lane) / PLANE < live ? voff[t] : OOB, soff);
 #pragma unroll
-    for (int t = 0; t < NTW; ++t) buf_load_lds4(rw, tile + WOFF + t * 64, woff[t], (uint32_t)o0 * KK * 16u);
+    for (int t = 0; t < NTW; ++t)
+      buf_load_lds4(rw, tile + WOFF + t * 64, live >= kDsOC || (t * 64 + lane) / (KK * 4) < live ? woff[t] : OOB,
+                    (uint32_t)o0 * KK * 16u);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const int on = oend - o0 < kDsOC ? oend - o0 : kDsOC;
 #pragma unroll 1

@@ -135,6 +135,14 @@ def test_permuted_weight_copy_is_shared_and_follows_the_weights(nn_backend, monk
     k_t.np()                                    # reading does not invalidate
     step(np.ones_like(k_n))
     assert len(made) == 3
+    # ... nor do operators that only read the kernel (a weight-decay term, a norm, a transposed view of it)
+    nn.square(k_t).np()
+    nn.reduce_sum(k_t).np()
+    nn.transpose(k_t, (1, 0, 2, 3)).np()
+    nn.mul(k_t, k_t).np()
+    nn.add(k_t, nn.Tensor_from_value(np.ones((1,), np.float32))).np()
+    step(np.ones_like(k_n))
+    assert len(made) == 3
 
 
 def test_transposed_convolution_copy_survives_optimizer_steps(nn_backend, monkeypatch):
@@ -271,6 +279,29 @@ def test_fused_epilogue_backward_twice_over_one_graph(nn_backend):
         del x, k, b, y
     for a, f in zip(*outs):
         assert np.array_equal(a, f)
+
+
+def test_fused_epilogue_lets_its_intermediate_go_with_its_last_reader(nn_backend, monkeypatch):
+    """The pre-activation gradient the three gradient functions of a fused layer share is dropped when the last of
+    them has run - before backward() moves on to the layer below - not when the whole sweep ends."""
+    nn = nn_backend
+    import litenn_amd.core as nc
+    from litenn_amd.core.hip import api
+    import importlib
+    conv_mod = importlib.import_module('litenn_amd.core.op.conv2D')
+    events = []
+    real_bwd, real_drop = api.bias_act_bwd, conv_mod._EpilogueGrad._drop
+    monkeypatch.setattr(api, 'bias_act_bwd', lambda *a: (events.append('bwd'), real_bwd(*a))[1])
+    monkeypatch.setattr(conv_mod._EpilogueGrad, '_drop', lambda self: (events.append('drop'), real_drop(self))[1])
+    rs = np.random.RandomState(3)
+    x = nn.Tensor_from_value(rs.randint(-3, 4, size=(2, 3, 8, 8)).astype(np.float32))
+    k1 = nn.Tensor_from_value(rs.randint(-3, 4, size=(4, 3, 3, 3)).astype(np.float32))
+    k2 = nn.Tensor_from_value(rs.randint(-3, 4, size=(5, 4, 3, 3)).astype(np.float32))
+    b1, b2 = nn.Tensor_from_value(np.ones((4,), np.float32)), nn.Tensor_from_value(np.ones((5,), np.float32))
+    y = nc.op.conv2D_bias_act(x, k1, b1, 1, 1, 'same', leaky_relu_alpha=0.5)
+    z = nc.op.conv2D_bias_act(y, k2, b2, 1, 1, 'same', leaky_relu_alpha=0.5)
+    nn.backward({z: np.ones(tuple(z.shape), np.float32)}, grad_for_non_trainables=True)
+    assert events == ['bwd', 'drop', 'bwd', 'drop']
 
 
 def test_depthwise_conv2d_reference_style(nn_backend):
