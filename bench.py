@@ -493,8 +493,10 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
     # weights change once per step), and the kernel gradient is written straight into that storage.
     Wp = Dev(api, shape=(IC, KS * KS, OC))
 
-    def p_fwd():
+    def p_wp():
         api.conv2d_permute_weights(0, desc, K.ptr, api.W_IOHW, Wp.ptr)
+
+    def p_fwd():
         api.conv2d_dgrad_pw(0, desc, X.ptr, Wp.ptr, Y.ptr, 0)
 
     def p_di():
@@ -503,7 +505,7 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
     def p_dk():
         api.conv2d_wgrad_iohw(0, desc, dY.ptr, X.ptr, dK.ptr, 1)
 
-    passes = {'fwd': p_fwd, 'dI': p_di, 'dK': p_dk}
+    passes = {'weights': p_wp, 'fwd': p_fwd, 'dI': p_di, 'dK': p_dk}
 
     def step():
         for fn in passes.values():
@@ -513,8 +515,13 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
     per_pass = {}
     for name, fn in passes.items():
         ms = time_events(api, fn, max(steps, 5))
-        per_pass[name] = {'ms': ms, 'tflops': flops / ms / 1e9, 'frac_mfma': flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS}
-    dom = max(per_pass, key=lambda n: per_pass[n]['ms'])
+        if name == 'weights':   # the copy of the kernel in the kernels' layout: bytes, no arithmetic
+            per_pass[name] = {'ms': ms, 'alg_gbs': 2 * 4.0 * k.size / ms / 1e6, 'frac_hbm': 2 * 4.0 * k.size / ms / 1e6 / PEAK_HBM_GBS,
+                              'note': 'one launch per step here; in a training step through the Python API the optimizer '
+                                      'update writes this copy and the launch does not exist'}
+        else:
+            per_pass[name] = {'ms': ms, 'tflops': flops / ms / 1e9, 'frac_mfma': flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS}
+    dom = max(('fwd', 'dI', 'dK'), key=lambda n: per_pass[n]['ms'])
     dI.zero()
     dK.zero()
     step()
@@ -522,10 +529,10 @@ def bench_conv_transpose(api, steps, warmup, cpu=True):
            'ms_per_step_cold': cold_ms, 'n_gpus': 1, 'steps': steps, 'warmup': warmup, 'settle_s': SETTLE_S, 'ms_per_step': wall_ms, 'higher_is_better': True,
            'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
            'config': {'workload': f'cfgT_decoder: conv2DTranspose x[{N}, {IC}, {IH}, {IW}] k[{OC}, {IC}, {KS}, {KS}] '
-                                  f"stride {S} 'same', step = fwd + dI(+=) + dK(+=)"},
+                                  f"stride {S} 'same', step = weight copy + fwd + dI(+=) + dK(+=)"},
            'roofline': {'bound': 'mfma', 'kernel': dom, 'achieved': per_pass[dom]['tflops'],
                         'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s', 'frac': per_pass[dom]['frac_mfma'],
-                        'traffic': None},
+                        'traffic': MEASURED_TRAFFIC_BYTES.get('cfgT_decoder', {}).get(dom)},
            'passes': per_pass}
     if cpu:
         from oracle import conv2d_transpose_all
