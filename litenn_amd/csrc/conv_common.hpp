@@ -407,7 +407,7 @@ __global__ __launch_bounds__(512, 2) void conv_kernel(ConvArgs a) {
     // forward / data gradient cut along K: the sub-tiles of one K slice and one row of tiles read the same weights,
     // those of one slice the same activations; numbered slice by slice and handed to the XCDs in contiguous runs,
     // each weight is fetched by one XCD or two instead of all eight (256 -> 512 channels 5x5 stride 2 on 16 x 16
-    // pixels, batch 16: 110 -> 30 MB fetched per launch; the pass takes 1-2 % longer, the sub-tiles of an XCD now
+    // pixels, batch 16: 110 -> 18 MB fetched per launch; the pass takes 1-2 % longer, the sub-tiles of an XCD now
     // waiting for the same lines at the same time)
     const int j = xcd_contiguous(by * (int)gridDim.x + bx, (int)(gridDim.x * gridDim.y));
     by = j / (int)gridDim.x;

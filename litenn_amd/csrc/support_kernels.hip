@@ -593,15 +593,16 @@ __global__ __launch_bounds__(256) void bias_act_bwd_rows_kernel(int N, int O, in
     if (dpre) dpre[e] = g;
     acc += g;
   }
-  if (part) part[(size_t)o * slices + sl] = acc;
+  if (part) part[(size_t)sl * O + o] = acc;   // [slice][feature]: the finishing kernel's threads read side by side
 }
 
+// dbias[o] (+)= the slices' sums of channel o, in slice order; element (o, s) lies at part[o * so + s * ss]
 __global__ void bias_act_bwd_finish_kernel(int O, int slices, const float* __restrict__ part, float* __restrict__ dbias,
-                                           int beta) {
+                                           int beta, int so, int ss) {
   const int o = blockIdx.x * blockDim.x + threadIdx.x;
   if (o >= O) return;
   float v = 0.0f;
-  for (int s = 0; s < slices; ++s) v += part[(size_t)o * slices + s];
+  for (int s = 0; s < slices; ++s) v += part[(size_t)o * so + (size_t)s * ss];
   dbias[o] = beta ? dbias[o] + v : v;
 }
 
@@ -628,7 +629,7 @@ int launch_bias_act_bwd(DeviceCtx* ctx, int N, int O, int HW, const float* y, co
     LNN_HIP(hipGetLastError());
     if (dbias) {
       hipLaunchKernelGGL(bias_act_bwd_finish_kernel, dim3((O + 255) / 256), dim3(256), 0, ctx->stream, O, (int)sl, part1,
-                         dbias, beta ? 1 : 0);
+                         dbias, beta ? 1 : 0, 1, O);
       LNN_HIP(hipGetLastError());
     }
     return LNN_OK;
@@ -655,7 +656,7 @@ int launch_bias_act_bwd(DeviceCtx* ctx, int N, int O, int HW, const float* y, co
   LNN_HIP(hipGetLastError());
   if (dbias && !direct) {
     hipLaunchKernelGGL(bias_act_bwd_finish_kernel, dim3((O + 255) / 256), dim3(256), 0, ctx->stream, O, (int)slices, part,
-                       dbias, beta ? 1 : 0);
+                       dbias, beta ? 1 : 0, (int)slices, 1);
     LNN_HIP(hipGetLastError());
   }
   return LNN_OK;
