@@ -155,6 +155,11 @@ int lnn_conv2d_fwd_path(const lnn_conv2d_desc* d, int compute_units, int* path);
 /* dW (+)= wgrad(X, dY)                   conv2D.py:52-54 (the reference always accumulates) */
 int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, const float* dY,
                          float* dW, int beta);
+/* How the most recent weight gradient on `dev` (any of its entry points) was laid out on the chip:
+ * info = {workgroups of the main kernel, K slices (1: none; 2 with equal runs), 1 if the K steps of all sub-tiles
+ * were dealt out in equal runs that cross sub-tile borders, rows of a tile}; all 0 after an image-stem kernel.
+ * No counterpart in the reference (one GeMM launch per gradient, matmul.py:127-164); for tests and tuning. */
+int lnn_conv2d_wgrad_last_plan(int dev, int32_t* info);
 
 /* ---- weights kept in the kernels' own layout.  The kernels for channel counts that are multiples of 32 read the
  * weights as Wp[o][kh*KW + kw][c]; lnn_conv2d_fwd_f32 / lnn_conv2d_dgrad_f32 make that copy in scratch on every

@@ -79,6 +79,7 @@ SIGNATURES = {
     'lnn_conv2d_wgrad_iohw_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_wgrad_noalloc_f32': [_c_int, ctypes.POINTER(ConvDesc), _ptr, _ptr, _ptr, _c_int],
     'lnn_conv2d_fwd_path': [ctypes.POINTER(ConvDesc), _c_int, ctypes.POINTER(_c_int)],
+    'lnn_conv2d_wgrad_last_plan': [_c_int, _i32arr],
     'lnn_conv2d_dgrad_path': [ctypes.POINTER(ConvDesc), _c_int, _c_int, ctypes.POINTER(_c_int), _i32arr],
     'lnn_unfold2d_f32': [_c_int] + [_c_int] * 14 + [_ptr, _ptr, _c_int],
     'lnn_transpose_f32': [_c_int, _c_int, _i32arr, _i32arr, _ptr, _ptr, _c_int],
@@ -280,6 +281,13 @@ def conv2d_wgrad_noalloc(dev, desc, X, dY, dW, beta=1):
 
 
 FWD_PATH_IMPLICIT_GEMM, FWD_PATH_STEM_PATCH = 0, 1
+
+
+def conv2d_wgrad_last_plan(dev):
+    """(workgroups, K slices, equal runs across sub-tile borders?, tile rows) of the most recent weight gradient."""
+    info = (ctypes.c_int32 * 4)()
+    check(lib.lnn_conv2d_wgrad_last_plan(dev, info))
+    return tuple(info)
 
 
 def conv2d_fwd_path(desc, compute_units):

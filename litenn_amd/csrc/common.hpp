@@ -28,6 +28,9 @@ struct DeviceCtx {
   // true while an allocation-free entry point runs: ws / ws_bytes then describe the fixed array, requests that do
   // not fit fail instead of allocating, and gather tables are carved from its tail instead of being cached
   bool no_alloc = false;
+  // the plan of the most recent weight-gradient launch: {workgroups of the main kernel, K slices (1: none),
+  // 1 if the K steps were dealt out in equal runs across chunk borders, rows of its tiles}
+  int last_wgrad_plan[4] = {0, 0, 0, 0};
 };
 
 int set_error(int code, const std::string& msg);

@@ -42,6 +42,12 @@ struct ConvArgs {
   // tap-major wgrad: the columns of an M tile form segs_per_mt segments of seg_units units; a group's columns stay
   // inside one segment (one tap, for the loaders that assume it; the whole row for the one that does not)
   int seg_units, segs_per_mt;
+  // tap-major wgrad with equal K shares (eq_wgs > 0): the K steps of all chunks laid end to end are cut into eq_wgs
+  // equal runs, one per workgroup, each shorter than a chunk's K: a run ends in the middle of a chunk and may go on
+  // at the beginning of the next.  Workgroup w stores the sums of its first piece as a [BM][chunk width] block at
+  // Out[2w] and of its second at Out[2w + 1]; the slice reduction adds up the blocks of the workgroups that touch
+  // a chunk, in workgroup order.  (ksplit = 2 then only says "partial sums".)
+  int eq_wgs;
   // forward / dgrad without a K split: units that do not divide evenly among the workgroups.  The first main_units
   // units (a whole number per workgroup) are computed as usual; each of the tail_units left over is cut into
   // tail_split K slices, one per workgroup, whose partial sums go to tail_part[slice][unit][BM][unit width] and are
@@ -315,7 +321,8 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
   p.kend = a.K;
   float* out = a.Out;
   int chunk_i = bx;
-  if (a.ksplit > 1) {
+  const bool eq = wgrad_tap(PASS) && a.eq_wgs > 0;
+  if (a.ksplit > 1 && !eq) {
     // K slice of this workgroup: slices are in gridDim.y, except that the tap-major wgrad pass has a flat
     // grid in which the last chunk, if it holds less work, is cut into proportionally fewer slices
     int slice = by, ns = a.ksplit;
@@ -347,10 +354,41 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
   p.om = a.ksplit > 1 ? plain_map(a.Ncols) : final_map<PASS>(a);
   p.post = a.post;
   if (a.ksplit > 1) { p.post.bias = nullptr; p.post.act = 0; }   // applied by the slice reduction
-  if (wgrad_tap(PASS))
-    walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.seg_units, a.segs_per_mt, a.total_units,
-                              a.chunk_units, chunk_i);
-  else if (a.tail_units == 0) {
+  if (wgrad_tap(PASS)) {
+    // one chunk over one K slice - or, with equal K shares, this workgroup's run of the end-to-end K steps, piece
+    // by piece: the rest of the chunk it begins in, whole chunks, the beginning of the chunk it ends in
+    const int nkt = (a.K + BK - 1) / BK;
+    long long s0 = 0, s1 = 1;
+    if (eq) {
+      const long long T = (long long)a.n_chunks * nkt;
+      s0 = T * bx / a.eq_wgs;
+      s1 = T * (bx + 1) / a.eq_wgs;
+    }
+    int piece = 0;
+    while (s0 < s1) {
+      long long adv = 1;
+      if (eq) {
+        constexpr int WN = 4 / WM, BM = 32 * WM;
+        chunk_i = (int)(s0 / nkt);
+        const int t0 = (int)(s0 - (long long)chunk_i * nkt);
+        const int t1 = s1 - s0 < nkt - t0 ? t0 + (int)(s1 - s0) : nkt;
+        p.kbeg = t0 * BK;
+        p.kend = t1 * BK < a.K ? t1 * BK : a.K;
+        // element (m, n) of the chunk at (m - mt*BM) * CW + (n - n0) of the piece's block: a plain map of pitch CW
+        // over a buffer that begins that much before the block
+        const int CW = a.chunk_units * 32 * WN, per_mt = a.seg_units * a.segs_per_mt;
+        const int u0 = chunk_i * a.chunk_units, mt = u0 / per_mt, n0 = (u0 - mt * per_mt) * 32 * WN;
+        const int shift = mt * BM * CW + n0;
+        p.rc = make_rsrc(a.Out + (size_t)(2 * bx + piece) * (BM * CW) - shift, (uint32_t)(shift + BM * CW) * 4u);
+        p.om = plain_map(CW);
+        adv = t1 - t0;
+        ++piece;
+      }
+      walk_units_seg<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.seg_units, a.segs_per_mt,
+                                a.total_units, a.chunk_units, chunk_i, eq ? a.chunk_units >> 1 : NTMAX);
+      s0 += adv;
+    }
+  } else if (a.tail_units == 0) {
     walk_units<WM, NTMAX>(p, lds, lds + Cfg::STAGES * Cfg::SA, Cfg::SA, Cfg::SB, a.n_units, a.total_units,
                           bx, a.grid_x);
   } else {
@@ -550,7 +588,7 @@ static int permuted_weights(DeviceCtx* ctx, const ConvGeom& g, const float* W, i
 template <int PASS, int WM>
 static ReduceArgs reduce_args(const ConvArgs& a, int final_beta) {
   constexpr int WN = 4 / WM;
-  ReduceArgs r;
+  ReduceArgs r = {};
   r.n = a.M * a.Ncols; r.slices = a.ksplit; r.slices_last = a.ksplit; r.beta = final_beta; r.ncols = a.Ncols;
   r.bm_log = WM == 4 ? 7 : (WM == 2 ? 6 : 5); r.uw_log = WN == 4 ? 7 : (WN == 2 ? 6 : 5);
   r.per_mt = 0; r.last_unit0 = 0x7fffffff;
@@ -560,6 +598,10 @@ static ReduceArgs reduce_args(const ConvArgs& a, int final_beta) {
     r.slices_last = a.ks_last;
     r.per_mt = a.seg_units * a.segs_per_mt;
     r.last_unit0 = (a.n_chunks - 1) * a.chunk_units;
+    if (a.eq_wgs > 0) {
+      r.eq_wgs = a.eq_wgs; r.eq_nkt = (a.K + BK - 1) / BK; r.eq_chunk = a.chunk_units; r.eq_chunks = a.n_chunks;
+      r.eq_cw_log = r.uw_log + (a.chunk_units == 2 ? 1 : (a.chunk_units == 4 ? 2 : 3));
+    }
   }
   r.dN = make_fastdiv((uint32_t)a.Ncols);
   r.om = final_map<PASS>(a);
@@ -629,6 +671,35 @@ static size_t plan_tiles(ConvArgs& a, long long slots, bool allow_tail = false) 
   return 0;
 }
 
+// Tap-major weight gradient: when the plan "whole chunks x K slices" would leave much of the chip idle (200 sub-tiles
+// of 16 K steps on 256 compute units), cut the K steps of all chunks, laid end to end, into one equal run per
+// workgroup slot instead (ConvArgs::eq_wgs).  Chunks are half-width sub-tiles then (both groups at half their
+// accumulators: half the partial sums per piece).  Taken only when a run is shorter than a chunk's K (so a workgroup
+// has at most two pieces), its estimated time - steps per workgroup plus a refill of the pipeline for the second
+// piece - beats the plan it replaces by a tenth, and the slice sum can run row-wise.  The pieces' blocks take
+// 2 * slots * BM * (chunk width) floats whatever the problem: 32 MiB on 256 compute units.
+template <int WM, int NTMAX>
+static void plan_equal_shares(ConvArgs& a, long long slots, int nkt) {
+  constexpr int WN = 4 / WM;
+  if (a.post.any() || a.Ncols % 4 != 0 || a.Ncols < 256 || (size_t)a.Ncols * sizeof(float) > 64 * 1024) return;
+  const int half = a.chunk_units / 2, per_mt = a.seg_units * a.segs_per_mt;
+  if (half < 2 || half % 2 != 0 || half * 32 * WN < 128) return;
+  if (a.total_units % half != 0 || per_mt % half != 0) return;   // whole chunks, none across two rows of tiles
+  const long long chunks = a.total_units / half, T = chunks * nkt;
+  if (T < 8 * slots || nkt < 16 || chunks > slots) return;
+  // time in K steps of a half-width chunk: now, and with equal shares
+  const long long rounds = (a.grid_x + slots - 1) / slots;
+  const long long now = rounds * ((nkt + a.ksplit - 1) / a.ksplit) * 2;
+  const long long then = (T + slots - 1) / slots + 2;
+  if (then * 11 > now * 10) return;
+  a.eq_wgs = (int)slots;
+  a.chunk_units = half;
+  a.n_chunks = (int)chunks;
+  a.ksplit = 2;
+  a.ks_last = 2;
+  a.grid_x = (int)slots;
+}
+
 template <int PASS, int WM, int NTMAX>
 static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
   constexpr int WN = 4 / WM, BM = 32 * WM;
@@ -689,8 +760,13 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
     }
     a.ksplit = ksplit;
     a.grid_x = grid;
+    a.eq_wgs = 0;
+    if (wgrad_tap(PASS) && PASS != PASS_WGRAD_ANYC) plan_equal_shares<WM, NTMAX>(a, slots, nkt);
+    ksplit = a.ksplit;
+    grid = a.grid_x;
     if (ksplit > 1) {
-      const size_t need = (size_t)ksplit * a.M * a.Ncols * sizeof(float);
+      const size_t need = a.eq_wgs > 0 ? (size_t)2 * a.eq_wgs * BM * (a.chunk_units * 32 * WN) * sizeof(float)
+                                       : (size_t)ksplit * a.M * a.Ncols * sizeof(float);
       int st = ensure_workspace(ctx, need);
       if (st != LNN_OK) return st;
       a.Out = static_cast<float*>(ctx->ws);
@@ -712,6 +788,12 @@ static int launch_pass(DeviceCtx* ctx, ConvArgs& a, bool flag) {
         grid_y = a.ksplit;
       }
     }
+  }
+  if (PASS == PASS_WGRAD || wgrad_tap(PASS)) {
+    ctx->last_wgrad_plan[0] = a.grid_x * grid_y;
+    ctx->last_wgrad_plan[1] = a.ksplit;
+    ctx->last_wgrad_plan[2] = wgrad_tap(PASS) && a.eq_wgs > 0 ? 1 : 0;
+    ctx->last_wgrad_plan[3] = BM;
   }
   dim3 g(a.grid_x, grid_y, 1), b(512, 1, 1);
   constexpr bool kUsesFlag = PASS == PASS_WGRAD || PASS == PASS_WGRAD_TAP || PASS == PASS_WGRAD_ANYC;   // the other passes have one variant

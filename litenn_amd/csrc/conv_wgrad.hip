@@ -13,6 +13,7 @@ int launch_conv_wgrad(DeviceCtx* ctx, const lnn_conv2d_desc* d, const float* X, 
   int st = fill_geom(d, a.g);
   if (st != LNN_OK) return st;
   if (!X || !dY || !dW) return set_error(LNN_ERR_INVALID, "conv2d_wgrad: null pointer");
+  ctx->last_wgrad_plan[0] = ctx->last_wgrad_plan[1] = ctx->last_wgrad_plan[2] = ctx->last_wgrad_plan[3] = 0;   // image-stem kernel: no tile plan
   if (!w_iohw && stem_wgrad_applies(d, ctx->cus, dY)) return launch_stem_wgrad(ctx, d, X, dY, dW, beta);
   a.tab = nullptr;
   const ConvGeom& g = a.g;

@@ -108,7 +108,7 @@ __global__ __launch_bounds__(512, 2) void gemm_kernel(GemmArgs a) {
 // Sum of the K slices of a split GEMM into C (pitch ldc), with '+=' and the epilogue.
 static int launch_gemm_reduce(DeviceCtx* ctx, const float* part, int slices, int M, int N, float* C, int ldc, int beta,
                               const PostOp& post) {
-  ReduceArgs r;
+  ReduceArgs r = {};
   r.n = M * N; r.slices = slices; r.slices_last = slices; r.beta = beta; r.ncols = N;
   r.bm_log = 5; r.uw_log = 5; r.per_mt = 0; r.last_unit0 = 0x7fffffff; r.kk = 0;
   r.dN = make_fastdiv((uint32_t)N);

@@ -391,6 +391,13 @@ int lnn_conv2d_wgrad_f32(int dev, const lnn_conv2d_desc* d, const float* X, cons
   return launch_conv_wgrad(ctx, d, X, dY, dW, beta);
 }
 
+int lnn_conv2d_wgrad_last_plan(int dev, int32_t* info) {
+  CTX(dev);
+  if (!info) return set_error(LNN_ERR_INVALID, "conv2d_wgrad_last_plan: null pointer");
+  for (int i = 0; i < 4; ++i) info[i] = ctx->last_wgrad_plan[i];
+  return LNN_OK;
+}
+
 namespace {
 // For the duration of one call the device's scratch is the fixed array (single-threaded callers per device).
 struct FixedScratch {

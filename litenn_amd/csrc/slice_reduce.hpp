@@ -17,10 +17,25 @@ struct ReduceArgs {
   int n, slices, slices_last, beta, ncols;
   int kk;   // KH*KW when the columns are tap-major weight-gradient columns (tap*C + c), else 0
   int bm_log, uw_log, per_mt, last_unit0;
+  // Equal K shares (eq_wgs > 0): the K steps of all chunks (eq_chunk units each, eq_nkt steps per chunk), laid end
+  // to end, are cut into eq_wgs equal runs, one per workgroup and none longer than a chunk's; workgroup w's sums for
+  // the chunk its run begins in are the block part[2w] of [1 << bm_log][eq_chunk << uw_log] floats, those for the
+  // chunk it goes on in part[2w + 1].
+  int eq_wgs, eq_nkt, eq_chunk, eq_chunks, eq_cw_log;   // eq_cw_log: log2 of a block's width in floats
   FastDiv dN;
   OutMap om;
   PostOp post;
 };
+// The workgroup whose run of K steps holds step s of the end-to-end order: runs are [T*w/W, T*(w+1)/W) for T steps
+// and W workgroups, so it is the smallest w with T*(w+1)/W > s.
+__host__ __device__ inline int eq_owner(long long s, long long T, long long W) { return (int)(((s + 1) * W + T - 1) / T - 1); }
+// How many workgroups hold a piece of chunk c, and which is the first
+__host__ __device__ inline int eq_planes(int c, int nkt, int chunks, int wgs, int* first) {
+  const long long T = (long long)chunks * nkt, s = (long long)c * nkt;
+  const int f = eq_owner(s, T, wgs);
+  if (first) *first = f;
+  return eq_owner(s + nkt - 1, T, wgs) - f + 1;
+}
 __device__ __forceinline__ void reduce_body(float* out, const float* part, const ReduceArgs& a) {
   __shared__ float red[8][33];
   const int li = threadIdx.x & 31, ls = threadIdx.x >> 5;
@@ -137,13 +152,44 @@ __global__ __launch_bounds__(256) void reduce_partials_rows(float* out, const fl
   extern __shared__ float reduce_row[];
   const uint32_t m = blockIdx.x, C = a.om.dHW.d;
   const size_t n = (size_t)a.n;
+  // equal K shares: per chunk of this row, the first workgroup that holds a piece of it, how many do, and whether
+  // that first one's piece is its second (its run began in the chunk before)
+  __shared__ int eq_first[128], eq_count[128];
+  if (a.eq_wgs > 0) {
+    const int per_row = a.ncols >> a.eq_cw_log;
+    const long long T = (long long)a.eq_chunks * a.eq_nkt;
+    for (int j = threadIdx.x; j < per_row; j += 256) {
+      const int c = (int)(m >> a.bm_log) * per_row + j;
+      int first;
+      const int np = eq_planes(c, a.eq_nkt, a.eq_chunks, a.eq_wgs, &first);
+      const int second = (int)(T * first / a.eq_wgs / a.eq_nkt) == c ? 0 : 1;
+      eq_first[j] = first;
+      eq_count[j] = np | (second << 16);
+    }
+    __syncthreads();
+  }
   for (int g = threadIdx.x; 4 * g < a.ncols; g += 256) {
     const uint32_t col = 4u * g;
     const size_t i4 = (size_t)m * a.ncols + col;
     const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
-    const int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
+    int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
     f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
     int k = 0;
+    if (a.eq_wgs > 0) {
+      // the blocks of the workgroups whose runs touch this element's chunk, in workgroup order
+      const int j = (int)(col >> a.eq_cw_log), cw = 1 << a.eq_cw_log, bm = 1 << a.bm_log;
+      const size_t within = (size_t)(m & (uint32_t)(bm - 1)) * cw + (col & (uint32_t)(cw - 1));
+      const int first = eq_first[j], np = eq_count[j] & 0xffff, second = eq_count[j] >> 16;
+      const float* src = part + (size_t)(2 * first + second) * bm * cw + within;
+      f32x4 v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const f32x4*>(src + (size_t)(i < np ? (i ? 2 * i - second : 0) : 0) * bm * cw);
+      const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s += i < np ? v[i] : zero;
+      for (int i = 4; i < np; ++i) s += *reinterpret_cast<const f32x4*>(src + (size_t)(2 * i - second) * bm * cw);
+      ns = 0;
+    }
     for (; k + 8 <= ns; k += 8) {
       f32x4 v[8];
 #pragma unroll

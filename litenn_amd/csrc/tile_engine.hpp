@@ -1913,11 +1913,12 @@ __device__ __forceinline__ void walk_units(const P& p, float* ldsA, float* ldsB,
 // convolution tap): a group's columns never cross a segment, the two groups
 // of a sub-tile may sit in different segments of the same M tile.
 // Units are numbered (mt * segs_per_mt + segment) * seg_units + unit; workgroup
-// chunk_index takes units [chunk_index*chunk, (chunk_index+1)*chunk).
+// chunk_index takes units [chunk_index*chunk, (chunk_index+1)*chunk); group 0 takes at most cap of them at a time
+// (NTMAX, or half a chunk that is narrower than two full groups).
 template <int WM, int NTMAX, class P>
 __device__ __forceinline__ void walk_units_seg(const P& p, float* ldsA, float* ldsB, int strideA, int strideB,
                                                int seg_units, int segs_per_mt, int total_units, int chunk,
-                                               int chunk_index) {
+                                               int chunk_index, int cap) {
   constexpr int WN = 4 / WM;
   const int per_mt = seg_units * segs_per_mt;
   int pos = chunk_index * chunk;
@@ -1925,7 +1926,7 @@ __device__ __forceinline__ void walk_units_seg(const P& p, float* ldsA, float* l
   while (pos < end) {
     const int mt = pos / per_mt;
     int nt0 = seg_units - pos % seg_units;
-    if (nt0 > NTMAX) nt0 = NTMAX;
+    if (nt0 > cap) nt0 = cap;
     if (nt0 > end - pos) nt0 = end - pos;
     const int p1 = pos + nt0;
     int nt1 = 0;

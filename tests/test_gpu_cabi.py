@@ -694,6 +694,46 @@ def test_conv_few_tiles_split_k_integer_exact(hip):
             assert np.array_equal(dw - off, rdw), ('dW', xs, ws)
 
 
+def test_conv_wgrad_equal_k_shares_integer_exact(hip):
+    """Weight gradients whose whole sub-tiles times K slices would leave a fifth of the chip idle (256 -> 512 channels
+    5x5 at 8 x 8 output pixels: 200 sub-tiles of 16 K steps on 256 compute units) deal the K steps of all sub-tiles
+    out in equal runs that cross sub-tile borders; a run's two pieces go to blocks of their own and the slice sum
+    adds each sub-tile's two or three blocks.  lnn_conv2d_wgrad_last_plan confirms the plan; exact on integers, '='
+    into NaN and '+=', OIHW and channel-swapped storage, and the allocation-free entry point (whose fixed array the
+    blocks fill exactly) bit for bit the same."""
+    rs = np.random.RandomState(41)
+    cus = hip.device_info(0)['compute_units']
+    cases = [((16, 256, 16, 16), (512, 256, 5, 5), 2, 1, 2), ((16, 512, 8, 8), (512, 512, 3, 3), 1, 1, 'same'),
+             ((16, 256, 8, 8), (500, 256, 5, 5), 1, 1, 'same')]
+    for xs, ws, s, d, padding in cases:
+        say(f'wgrad equal K shares x={xs} w={ws} s={s} pad={padding}')
+        desc, ci = _desc(hip, xs, ws, s, d, padding)
+        x = rs.randint(4, size=xs).astype(np.float32)
+        dy = (rs.randint(4, size=(xs[0], ws[0], ci.OH, ci.OW)) - 1).astype(np.float32)
+        rdw = np.zeros(ws, np.float64)
+        for i0 in range(0, xs[0], 4):
+            rdw += conv2d_dw(x[i0:i0 + 4], dy[i0:i0 + 4], ws, s, d, padding)
+        X, dY = DevArr(hip, x), DevArr(hip, dy)
+        dW = DevArr(hip, shape=ws, fill=np.nan)
+        hip.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW.ptr, 0)
+        plan = hip.conv2d_wgrad_last_plan(0)
+        if cus == 256:
+            assert plan[2] == 1 and plan[0] == cus, (plan, xs, ws)
+        got = dW.get()
+        assert np.array_equal(got, rdw), ('dW =', xs, ws)
+        w0 = rs.randint(-3, 4, size=ws).astype(np.float32)
+        dW2 = DevArr(hip, w0)
+        hip.conv2d_wgrad(0, desc, X.ptr, dY.ptr, dW2.ptr, 1)
+        assert np.array_equal(dW2.get(), rdw + w0), ('dW +=', xs, ws)
+        dW3 = DevArr(hip, shape=(ws[1], ws[0], ws[2], ws[3]), fill=np.nan)
+        hip.conv2d_wgrad_iohw(0, desc, X.ptr, dY.ptr, dW3.ptr, 0)
+        assert np.array_equal(dW3.get(), rdw.transpose(1, 0, 2, 3)), ('dW swapped', xs, ws)
+        dW4 = DevArr(hip, shape=ws, fill=np.nan)
+        hip.conv2d_wgrad_noalloc(0, desc, X.ptr, dY.ptr, dW4.ptr, 0)
+        assert hip.conv2d_wgrad_last_plan(0) == plan
+        assert np.array_equal(dW4.get(), got), ('dW without allocation', xs, ws)
+
+
 def test_conv_fwd_bias_act_matches_separate_kernels(hip):
     """Fused forward through the C ABI against the three separate launches
     (convolution, broadcast bias add, leaky ReLU) of the same library, bit for
