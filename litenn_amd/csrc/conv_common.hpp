@@ -612,9 +612,14 @@ static ReduceArgs reduce_args(const ConvArgs& a, int final_beta) {
 template <int PASS, int WM>
 static int launch_reduce(DeviceCtx* ctx, const ConvArgs& a, float* final_out, int final_beta) {
   const ReduceArgs r = reduce_args<PASS, WM>(a, final_beta);
-  if (wgrad_tap(PASS) && a.Ncols % 4 == 0 && a.Ncols >= 256 && (size_t)a.Ncols * sizeof(float) <= 64 * 1024 && !r.post.any())
-    hipLaunchKernelGGL(reduce_partials_rows, dim3(a.M), dim3(256), (size_t)a.Ncols * sizeof(float), ctx->stream, final_out,
+  if (wgrad_tap(PASS) && a.Ncols % 4 == 0 && a.Ncols >= 256 && (size_t)a.Ncols * sizeof(float) <= 64 * 1024 && !r.post.any()) {
+    // rows fewer than four times the compute units: several blocks per row, each a run of channels
+    int parts = 1;
+    if (a.g.C % 4 == 0)
+      while (parts < 8 && a.M * parts < 4 * ctx->cus && a.g.C / (2 * parts) >= 16) parts *= 2;
+    hipLaunchKernelGGL(reduce_partials_rows, dim3(a.M, parts), dim3(256), (size_t)a.Ncols * sizeof(float), ctx->stream, final_out,
                        static_cast<const float*>(a.Out), r);
+  }
   else if (a.Ncols % 4 == 0)   // partial buffers start 256-byte aligned
     hipLaunchKernelGGL(reduce_partials4, dim3((r.n + reduce4_block(r) - 1) / reduce4_block(r)), dim3(256), 0, ctx->stream, final_out,
                        static_cast<const float*>(a.Out), r);

@@ -147,7 +147,8 @@ __device__ __forceinline__ void reduce_body4_few(float* out, const float* part, 
 // The element-wise kernels above store a row's elements KK floats apart, 4 bytes at a time; here the row's sums are
 // parked in LDS at their permuted place c*KK + tap (KK odd for the usual kernels: no bank conflicts) and leave as one
 // contiguous run (whole runs of KK floats per channel for a gradient kept with swapped channel axes).  Slices are
-// added in ascending order, eight loads in flight.  ncols % 4 == 0; ncols floats of dynamic LDS.
+// added in ascending order, eight loads in flight.  ncols % 4 == 0; a row may be shared out among gridDim.y blocks by
+// runs of channels (C % 4 == 0 then); (channels per block) * KK floats of dynamic LDS.
 __global__ __launch_bounds__(256) void reduce_partials_rows(float* out, const float* part, ReduceArgs a) {
   extern __shared__ float reduce_row[];
   const uint32_t m = blockIdx.x, C = a.om.dHW.d;
@@ -168,8 +169,14 @@ __global__ __launch_bounds__(256) void reduce_partials_rows(float* out, const fl
     }
     __syncthreads();
   }
-  for (int g = threadIdx.x; 4 * g < a.ncols; g += 256) {
-    const uint32_t col = 4u * g;
+  // blockIdx.y: which run of channels of the row this block sums (gridDim.y runs of cpb channels, cpb % 4 == 0)
+  const uint32_t cpb = gridDim.y > 1 ? (((C + gridDim.y - 1) / gridDim.y + 3) & ~3u) : C;
+  const uint32_t c0 = blockIdx.y * cpb, cn = c0 >= C ? 0u : (C - c0 < cpb ? C - c0 : cpb);
+  const int mine = (int)(cn * (uint32_t)a.kk);
+  for (int g = threadIdx.x; 4 * g < mine; g += 256) {
+    // the g-th group of four of this block's columns (tap-major: tap * C + c0 .. c0 + cn)
+    const uint32_t tap0 = gridDim.y > 1 ? (4u * g) / cn : 0u;
+    const uint32_t col = gridDim.y > 1 ? tap0 * C + c0 + (4u * g - tap0 * cn) : 4u * g;
     const size_t i4 = (size_t)m * a.ncols + col;
     const int unit = (int)(m >> a.bm_log) * a.per_mt + (int)(col >> a.uw_log);
     int ns = unit >= a.last_unit0 ? a.slices_last : a.slices;
@@ -208,12 +215,12 @@ __global__ __launch_bounds__(256) void reduce_partials_rows(float* out, const fl
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t cj = col + j, tap = a.om.dHW.div(cj), c = cj - tap * C;
-      reduce_row[c * a.kk + tap] = s[j];
+      reduce_row[(c - c0) * a.kk + tap] = s[j];
     }
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < a.ncols; e += 256) {
-    const uint32_t c = (uint32_t)e / (uint32_t)a.kk, tap = (uint32_t)e - c * (uint32_t)a.kk;
+  for (int e = threadIdx.x; e < mine; e += 256) {
+    const uint32_t cl = (uint32_t)e / (uint32_t)a.kk, tap = (uint32_t)e - cl * (uint32_t)a.kk, c = c0 + cl;
     const size_t o = (size_t)a.om.col(tap * C + c) + (size_t)m * a.om.ld;
     const float t = reduce_row[e];
     out[o] = a.beta ? out[o] + t : t;
