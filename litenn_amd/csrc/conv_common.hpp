@@ -359,10 +359,14 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
     // by piece: the rest of the chunk it begins in, whole chunks, the beginning of the chunk it ends in
     const int nkt = (a.K + BK - 1) / BK;
     long long s0 = 0, s1 = 1;
+    // Which run this workgroup takes: its number.  The runs of an XCD then stand at different K positions at any one
+    // time and share little in its L2 (the 256 -> 512 layer fetches 150 MB per launch where whole sub-tiles x 2 slices
+    // fetched 24); dealing contiguous runs to an XCD reads the same 150 MB, and the pass is faster all the same.
+    const int run = bx;
     if (eq) {
       const long long T = (long long)a.n_chunks * nkt;
-      s0 = T * bx / a.eq_wgs;
-      s1 = T * (bx + 1) / a.eq_wgs;
+      s0 = T * run / a.eq_wgs;
+      s1 = T * (run + 1) / a.eq_wgs;
     }
     int piece = 0;
     while (s0 < s1) {
@@ -379,7 +383,7 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
         const int CW = a.chunk_units * 32 * WN, per_mt = a.seg_units * a.segs_per_mt;
         const int u0 = chunk_i * a.chunk_units, mt = u0 / per_mt, n0 = (u0 - mt * per_mt) * 32 * WN;
         const int shift = mt * BM * CW + n0;
-        p.rc = make_rsrc(a.Out + (size_t)(2 * bx + piece) * (BM * CW) - shift, (uint32_t)(shift + BM * CW) * 4u);
+        p.rc = make_rsrc(a.Out + (size_t)(2 * run + piece) * (BM * CW) - shift, (uint32_t)(shift + BM * CW) * 4u);
         p.om = plain_map(CW);
         adv = t1 - t0;
         ++piece;
