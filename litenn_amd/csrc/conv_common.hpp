@@ -48,6 +48,9 @@ struct ConvArgs {
   // Out[2w] and of its second at Out[2w + 1]; the slice reduction adds up the blocks of the workgroups that touch
   // a chunk, in workgroup order.  (ksplit = 2 then only says "partial sums".)
   int eq_wgs;
+  // ... and the order in which the chunks are laid end to end: place q holds chunk (q % eq_d) * eq_g + q / eq_d
+  // (eq_d = 0: chunk q).  See plan_equal_shares.
+  int eq_d, eq_g;
   // forward / dgrad without a K split: units that do not divide evenly among the workgroups.  The first main_units
   // units (a whole number per workgroup) are computed as usual; each of the tail_units left over is cut into
   // tail_split K slices, one per workgroup, whose partial sums go to tail_part[slice][unit][BM][unit width] and are
@@ -359,9 +362,6 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
     // by piece: the rest of the chunk it begins in, whole chunks, the beginning of the chunk it ends in
     const int nkt = (a.K + BK - 1) / BK;
     long long s0 = 0, s1 = 1;
-    // Which run this workgroup takes: its number.  The runs of an XCD then stand at different K positions at any one
-    // time and share little in its L2 (the 256 -> 512 layer fetches 150 MB per launch where whole sub-tiles x 2 slices
-    // fetched 24); dealing contiguous runs to an XCD reads the same 150 MB, and the pass is faster all the same.
     const int run = bx;
     if (eq) {
       const long long T = (long long)a.n_chunks * nkt;
@@ -373,8 +373,9 @@ __device__ __forceinline__ void conv_body(const ConvArgs& a, int bx, int by) {
       long long adv = 1;
       if (eq) {
         constexpr int WN = 4 / WM, BM = 32 * WM;
-        chunk_i = (int)(s0 / nkt);
-        const int t0 = (int)(s0 - (long long)chunk_i * nkt);
+        const int place = (int)(s0 / nkt);
+        chunk_i = a.eq_d > 0 ? (place % a.eq_d) * a.eq_g + place / a.eq_d : place;
+        const int t0 = (int)(s0 - (long long)place * nkt);
         const int t1 = s1 - s0 < nkt - t0 ? t0 + (int)(s1 - s0) : nkt;
         p.kbeg = t0 * BK;
         p.kend = t1 * BK < a.K ? t1 * BK : a.K;
@@ -605,6 +606,7 @@ static ReduceArgs reduce_args(const ConvArgs& a, int final_beta) {
     if (a.eq_wgs > 0) {
       r.eq_wgs = a.eq_wgs; r.eq_nkt = (a.K + BK - 1) / BK; r.eq_chunk = a.chunk_units; r.eq_chunks = a.n_chunks;
       r.eq_cw_log = r.uw_log + (a.chunk_units == 2 ? 1 : (a.chunk_units == 4 ? 2 : 3));
+      r.eq_d = a.eq_d; r.eq_g = a.eq_g;
     }
   }
   r.dN = make_fastdiv((uint32_t)a.Ncols);
@@ -702,6 +704,22 @@ static void plan_equal_shares(ConvArgs& a, long long slots, int nkt) {
   const long long then = (T + slots - 1) / slots + 2;
   if (then * 11 > now * 10) return;
   a.eq_wgs = (int)slots;
+  // Runs w and w + P stand at the same K position all along when S * P is a multiple of nkt (S steps per run), and
+  // with 8 | P they also share an XCD (workgroups go to the XCDs in turn).  Their places in the end-to-end order lie
+  // D = S * P / nkt apart, so the order takes the chunks with a stride: the W / P runs that move through K together
+  // work on neighbouring chunks - neighbouring taps of one row of tiles, which read the same dY rows and X rows a
+  // few pixels apart - and meet their operands in that XCD's L2.
+  a.eq_d = a.eq_g = 0;
+  if (T % slots == 0) {
+    const long long S = T / slots;
+    long long gcd = S, r = nkt;
+    while (r) { const long long t = gcd % r; gcd = r; r = t; }
+    const long long P = nkt / gcd, D = S * P / nkt;
+    if (P % 8 == 0 && slots % P == 0 && D * (slots / P) == chunks) {
+      a.eq_d = (int)D;
+      a.eq_g = (int)(slots / P);
+    }
+  }
   a.chunk_units = half;
   a.n_chunks = (int)chunks;
   a.ksplit = 2;

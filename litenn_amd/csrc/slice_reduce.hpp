@@ -22,6 +22,7 @@ struct ReduceArgs {
   // the chunk its run begins in are the block part[2w] of [1 << bm_log][eq_chunk << uw_log] floats, those for the
   // chunk it goes on in part[2w + 1].
   int eq_wgs, eq_nkt, eq_chunk, eq_chunks, eq_cw_log;   // eq_cw_log: log2 of a block's width in floats
+  int eq_d, eq_g;   // the end-to-end order takes chunk (q % eq_d) * eq_g + q / eq_d at place q (eq_d = 0: chunk q)
   FastDiv dN;
   OutMap om;
   PostOp post;
@@ -161,9 +162,10 @@ __global__ __launch_bounds__(256) void reduce_partials_rows(float* out, const fl
     const long long T = (long long)a.eq_chunks * a.eq_nkt;
     for (int j = threadIdx.x; j < per_row; j += 256) {
       const int c = (int)(m >> a.bm_log) * per_row + j;
+      const int q = a.eq_d > 0 ? a.eq_d * (c % a.eq_g) + c / a.eq_g : c;   // the chunk's place in the end-to-end order
       int first;
-      const int np = eq_planes(c, a.eq_nkt, a.eq_chunks, a.eq_wgs, &first);
-      const int second = (int)(T * first / a.eq_wgs / a.eq_nkt) == c ? 0 : 1;
+      const int np = eq_planes(q, a.eq_nkt, a.eq_chunks, a.eq_wgs, &first);
+      const int second = (int)(T * first / a.eq_wgs / a.eq_nkt) == q ? 0 : 1;
       eq_first[j] = first;
       eq_count[j] = np | (second << 16);
     }
